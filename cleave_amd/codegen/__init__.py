@@ -1,0 +1,386 @@
+"""Code generation: a scheduled ``KernelPlan`` becomes HIP source text for gfx950.
+
+Takes the place of the reference's TileLang emitter
+(``python/cleave/codegen/__init__.py:24-60`` and ``kernel.py``/``split.py``/``macros.py``):
+``HipCodeGen().gen(plan)`` returns one self-contained translation unit, and
+``gen([partial, combine])`` the fused two-kernel form of a split pair
+(``python/cleave/codegen/split.py:13-123``) whose partial buffers are scratch parameters named
+``Partial_<X>_split`` / ``Partial_<X>_combine`` (one allocation, two names).
+
+A generated source is: a manifest comment (JSON: parameters in call order, launches with grid
+expressions, LDS bytes), a block of ``#define``s instantiating the template, the shared
+helpers, and the hand-written template body.  The kernel entry is ``main_kernel``; parameter
+names follow the reference's contract (``PlaceHolder_<NAME>``, run-time scalars between inputs
+and outputs, then ``OutputNode_<i>``; ``python/cleave/codegen/kernel.py:576-612``).
+"""
+
+from __future__ import annotations
+
+import json
+import math
+from pathlib import Path
+
+from ..core.errors import CodegenError
+from ..schedule.plan import KernelPlan, ParamSpec
+
+TEMPLATE_DIR = Path(__file__).resolve().parent / "templates"
+ENTRY = "main_kernel"
+COMBINE_ENTRY = "main_kernel_combine"
+MANIFEST_BEGIN = "// CLEAVE-HIP-MANIFEST-BEGIN"
+MANIFEST_END = "// CLEAVE-HIP-MANIFEST-END"
+LOG2E = 1.4426950408889634
+
+_C_TYPES = {"float16": "elem_t", "bfloat16": "elem_t", "float32": "float", "int32": "int"}
+
+
+def _template(name: str) -> str:
+    return (TEMPLATE_DIR / name).read_text()
+
+
+def _f(x: float) -> str:
+    """A C float literal that round-trips."""
+    text = repr(float(x))
+    if "e" not in text and "." not in text and "inf" not in text and "nan" not in text:
+        text += ".0"
+    return text + "f"
+
+
+def _c_param(p: ParamSpec) -> str:
+    if p.role == "scalar":
+        return f"{_C_TYPES[p.dtype]} {p.name}"
+    const = "const " if p.role == "input" else ""
+    return f"{const}{_C_TYPES[p.dtype]}* __restrict__ {p.name}"
+
+
+class _Unit:
+    """Accumulates one translation unit: defines, launches, parameters."""
+
+    def __init__(self, plan: KernelPlan):
+        self.plan = plan
+        self.defines: list = []
+        self.launches: list = []
+        self.templates: list = ["common.hip"]
+
+    def define(self, name, value):
+        if isinstance(value, bool):
+            value = int(value)
+        self.defines.append(f"#define {name} {value}")
+
+    def signature(self, macro, entry_macro, entry, params, dyn_dims, dyn_c_names=None):
+        """Define the C parameter list of one kernel; returns the manifest's argument names.
+        ``dyn_c_names``: the identifiers the template uses for the run-time extents, when the
+        operator spec renamed them."""
+        parts = [_c_param(p) for p in params] + [f"int {d}" for d in (dyn_c_names or dyn_dims)]
+        self.define(entry_macro, entry)
+        self.define(macro, ", ".join(parts))
+        return [p.name for p in params] + list(dyn_dims)
+
+    def launch(self, entry, grid, block, lds, args):
+        self.launches.append({"entry": entry, "grid": [str(g) for g in grid], "block": [int(block), 1, 1],
+                              "lds": int(lds), "args": list(args)})
+
+
+class HipCodeGen:
+    def gen(self, plan_or_pair, *, params=None) -> str:
+        """Source text for one plan, or for ``[partial, combine]`` fused into one unit."""
+        try:
+            if isinstance(plan_or_pair, (list, tuple)):
+                if len(plan_or_pair) == 1:
+                    return self._gen_one(plan_or_pair[0])
+                if len(plan_or_pair) != 2:
+                    raise CodegenError(f"expected one plan or a [partial, combine] pair, got {len(plan_or_pair)}")
+                return self._gen_fused(*plan_or_pair)
+            return self._gen_one(plan_or_pair)
+        except CodegenError:
+            raise
+        except (KeyError, ValueError, TypeError, ZeroDivisionError) as e:
+            raise CodegenError(f"{type(e).__name__} while instantiating a template: {e}") from e
+
+    # ------------------------------------------------------------------ drivers
+    def _gen_one(self, plan: KernelPlan) -> str:
+        unit = _Unit(plan)
+        emit = getattr(self, f"_emit_{plan.template}", None)
+        if emit is None:
+            raise CodegenError(f"no template named {plan.template!r}")
+        splits = plan.split_factor or 1
+        if plan.role == "main" and splits != 1:
+            raise CodegenError("a main kernel cannot carry a split factor")
+        params = list(plan.params)
+        emit(unit, plan, params, partial=plan.role in ("main", "partial", "fused"),
+             combine=plan.role in ("combine", "fused") and splits > 1, fused=plan.role == "fused")
+        return self._finish(unit, plan, params)
+
+    def _gen_fused(self, partial: KernelPlan, combine: KernelPlan) -> str:
+        """Partial and combine in one unit: the partial's outputs become scratch parameters."""
+        if partial.role != "partial" or combine.role != "combine":
+            raise CodegenError("a fused pair is [partial, combine]")
+        if partial.template != combine.template and not {partial.template, combine.template} <= {"gemm", "skinny"}:
+            raise CodegenError(f"partial ({partial.template}) and combine ({combine.template}) templates differ")
+        params = [p for p in partial.params if p.role in ("input", "scalar")]
+        operands = dict(partial.operands)
+        for p in partial.params:
+            if p.role == "output":
+                role = next(r for r, n in partial.operands.items() if n == p.name)
+                split_name, comb_name = f"Partial_{role}_split", f"Partial_{role}_combine"
+                params.append(ParamSpec(split_name, p.dtype, p.shape, "scratch"))
+                params.append(ParamSpec(comb_name, p.dtype, p.shape, "scratch", alias=split_name))
+                operands[role] = split_name
+                operands[f"{role}_COMBINE"] = comb_name
+        for p in combine.params:
+            if p.role == "output":
+                params.append(p)
+        operands.update({r: n for r, n in combine.operands.items() if r.startswith("OUT")})
+        fused = KernelPlan(template=partial.template, role="fused", family=partial.family, dtype=partial.dtype,
+                           problem=partial.problem, tiling=partial.tiling, params=params, operands=operands,
+                           split_factor=partial.split_factor, dyn_dims=partial.dyn_dims, n_threads=partial.n_threads,
+                           lds_bytes=partial.lds_bytes, label=f"{partial.label} + combine", extra=dict(partial.extra))
+        return self._gen_one(fused)
+
+    def _finish(self, unit: _Unit, plan: KernelPlan, params) -> str:
+        n_out = sum(p.role == "output" for p in params)
+        manifest = {
+            "format": 1, "generator": "cleave_amd", "arch": "gfx950", "template": plan.template,
+            "role": plan.role, "family": plan.family, "dtype": plan.dtype, "label": plan.label,
+            "split": plan.split_factor, "tiling": plan.tiling,
+            "params": [p.to_json() for p in params], "dyn_dims": list(plan.dyn_dims),
+            "out_idx": list(range(-n_out, 0)), "launches": unit.launches,
+        }
+        head = [MANIFEST_BEGIN] + ["// " + line for line in json.dumps(manifest, indent=1).splitlines()] + [MANIFEST_END]
+        body = [f"// ---- template: {plan.template}  role: {plan.role}  {plan.label}"]
+        body += unit.defines
+        for name in unit.templates:
+            body.append(_template(name))
+        return "\n".join(head + body) + "\n"
+
+    # ------------------------------------------------------------------ shared pieces
+    @staticmethod
+    def _common(unit: _Unit, plan: KernelPlan, partial: bool, combine: bool):
+        unit.define("CL_BF16", plan.dtype == "bfloat16")
+        unit.define("CL_SPLITS", plan.split_factor or 1)
+        unit.define("CL_EMIT_PARTIAL", partial)
+        unit.define("CL_EMIT_COMBINE", combine)
+
+    @staticmethod
+    def _by_name(params):
+        return {p.name: p for p in params}
+
+    # ------------------------------------------------------------------ matmul families
+    def _matmul_common(self, unit, plan, params, partial, combine, fused):
+        p, op = plan.problem, plan.operands
+        self._common(unit, plan, partial, combine)
+        norm = plan.family == "rmsnorm_matmul"
+        for k in ("M", "N", "K"):
+            unit.define(f"CL_{k}", p[k])
+        unit.define("CL_NORM", norm)
+        unit.define("CL_GAMMA", bool(norm and p.get("gamma")))
+        unit.define("CL_EPS", _f(p.get("eps", 0.0)))
+        unit.define("CL_BATCH_A", p["batch_A"])
+        unit.define("CL_BATCH_B", p["batch_B"])
+        unit.define("CL_TRANS_A", p["trans_A"])
+        unit.define("CL_TRANS_B", p["trans_B"])
+        splits = plan.split_factor or 1
+        names = self._by_name(params)
+        ins = [q for q in params if q.role in ("input", "scalar")]
+        outs = [q for q in params if q.role == "output"]
+        batch = max(p["batch_A"], p["batch_B"])
+        if partial:
+            if plan.role in ("main",):
+                sig = ins + outs
+                unit.define("CL_ARG_OUT", op["OUT"])
+            elif plan.role == "partial":
+                sig = ins + outs
+            else:  # fused
+                sig = ins + [names[op["PACC"]]] + ([names[op["PSS"]]] if norm else [])
+            if splits > 1:
+                unit.define("CL_ARG_PACC", op["PACC"])
+                if norm:
+                    unit.define("CL_ARG_PSS", op["PSS"])
+            for role, macro in (("A", "CL_ARG_A"), ("B", "CL_ARG_B"), ("GAMMA", "CL_ARG_GAMMA")):
+                if role in op:
+                    unit.define(macro, op[role])
+            unit.define("CL_ARG_X", op["A"])
+            unit.define("CL_ARG_W", op["B"])
+            args = unit.signature("CL_PARTIAL_PARAMS", "CL_PARTIAL_NAME", ENTRY, sig, ())
+            self._partial_args = args
+        if combine:
+            if plan.role == "combine":
+                sig, entry, suffix = ins + outs, ENTRY, ""
+            else:
+                # the combine reads the same allocation under its `_combine` name
+                sig = [names[op["PACC_COMBINE"]]] + ([names[op["PSS_COMBINE"]]] if norm else []) + outs
+                entry, suffix = COMBINE_ENTRY, "_COMBINE"
+            unit.define("CL_CARG_PACC", op["PACC" + suffix])
+            if norm:
+                unit.define("CL_CARG_PSS", op["PSS" + suffix])
+            unit.define("CL_CARG_OUT", op["OUT"])
+            args = unit.signature("CL_COMBINE_PARAMS", "CL_COMBINE_NAME", entry, sig, ())
+            self._combine_args = (entry, args, batch * p["M"] * p["N"])
+
+    def _emit_gemm(self, unit, plan, params, partial, combine, fused):
+        p, t = plan.problem, plan.tiling
+        self._matmul_common(unit, plan, params, partial, combine, fused)
+        tile = dict(BM=64, BN=64, BK=32, WM=1, WN=1)
+        tile.update(t)
+        for k, v in tile.items():
+            unit.define(f"CL_{k}", v)
+        splits = plan.split_factor or 1
+        batch = max(p["batch_A"], p["batch_B"])
+        unit.templates.append("gemm.hip")
+        if partial:
+            from ..schedule.policy import gemm_lds_bytes
+
+            if p["K"] % (splits * tile["BK"]):
+                raise CodegenError(f"K={p['K']} is not a multiple of splits*BK={splits * tile['BK']}")
+            grid = (-(-p["N"] // tile["BN"]), -(-p["M"] // tile["BM"]), batch * splits)
+            lds = gemm_lds_bytes(tile["BM"], tile["BN"], tile["BK"], plan.family == "rmsnorm_matmul")
+            unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, lds, self._partial_args)
+        if combine:
+            entry, args, total = self._combine_args
+            unit.launch(entry, (-(-(total // 4) // 256), 1, 1), 256, 0, args)
+
+    def _emit_skinny(self, unit, plan, params, partial, combine, fused):
+        p, t = plan.problem, plan.tiling
+        self._matmul_common(unit, plan, params, partial, combine, fused)
+        tile = dict(WAVES_N=1, WAVES_K=1)
+        tile.update(t)
+        for k, v in tile.items():
+            unit.define(f"CL_{k}", v)
+        unit.templates.append("skinny_matmul.hip")
+        splits = plan.split_factor or 1
+        if partial:
+            from ..schedule.policy import skinny_lds_bytes
+
+            if p["M"] > 64 or p["K"] % 32 or p["N"] % 8:
+                raise CodegenError("the few-row matmul template needs M <= 64, K % 32 == 0, N % 8 == 0")
+            grid = (-(-p["N"] // (128 * tile["WAVES_N"])), splits, 1)
+            lds = skinny_lds_bytes(-(-p["M"] // 16), tile["WAVES_N"], tile["WAVES_K"])
+            unit.launch(ENTRY, grid, tile["WAVES_N"] * tile["WAVES_K"] * 64, lds, self._partial_args)
+        if combine:
+            entry, args, total = self._combine_args
+            unit.launch(entry, (-(-(total // 8) // 256), 1, 1), 256, 0, args)
+
+    # ------------------------------------------------------------------ attention families
+    def _attn_common(self, unit, plan, params, partial, combine, fused, vdim, total_rows, emit_lse):
+        op = plan.operands
+        self._common(unit, plan, partial, combine)
+        unit.define("CL_VDIM", vdim)
+        unit.define("CL_TOTAL_ROWS", total_rows)
+        unit.define("CL_EMIT_LSE", emit_lse)
+        names = self._by_name(params)
+        ins = [q for q in params if q.role in ("input", "scalar")]
+        outs = [q for q in params if q.role == "output"]
+        dyn = tuple(plan.dyn_dims)
+        dyn_c = tuple((plan.problem.get("dim_names") or {}).keys()) or None
+        splits = plan.split_factor or 1
+        part_roles = ("PM", "PL", "PO")
+        if partial:
+            if plan.role == "fused":
+                sig = ins + [names[op[r]] for r in part_roles]
+            else:
+                sig = ins + outs
+            if splits > 1:
+                for r in part_roles:
+                    unit.define(f"CL_ARG_{r}", op[r])
+            else:
+                unit.define("CL_ARG_OUT", op["OUT"])
+                if emit_lse:
+                    unit.define("CL_ARG_LSE", op["OUT1"])
+            self._partial_args = unit.signature("CL_PARTIAL_PARAMS", "CL_PARTIAL_NAME", ENTRY, sig, dyn, dyn_c)
+        if combine:
+            if plan.role == "combine":
+                sig, entry, suffix = ins + outs, ENTRY, ""
+            else:
+                sig, entry, suffix = [names[op[f"{r}_COMBINE"]] for r in part_roles] + outs, COMBINE_ENTRY, "_COMBINE"
+            for r in part_roles:
+                unit.define(f"CL_CARG_{r}", op[r + suffix])
+            unit.define("CL_CARG_OUT", op["OUT"])
+            if emit_lse:
+                unit.define("CL_CARG_LSE", op["OUT1"])
+            args = unit.signature("CL_COMBINE_PARAMS", "CL_COMBINE_NAME", entry, sig, dyn, dyn_c)
+            self._combine_args = (entry, args)
+
+    def _emit_attn_decode(self, unit, plan, params, partial, combine, fused):
+        p, t, op = plan.problem, plan.tiling, plan.operands
+        paged = bool(p.get("paged"))
+        rows = p["group"] * p["sq"]
+        emit_lse = bool(p.get("emit_lse"))
+        if paged:
+            batch_name = p["dim_names"]["batch"]
+            total_rows = f"(batch * {p['q_heads']})"          # C expression inside the kernels
+            units = f"{batch_name} * {p['kv_heads']}"          # grid expression over manifest dims
+            grid_rows = f"({batch_name} * {p['q_heads']})"
+        else:
+            total_rows = p["units"] * rows
+            units = str(p["units"])
+            grid_rows = str(total_rows)
+        self._attn_common(unit, plan, params, partial, combine, fused, p["vdim"], total_rows, emit_lse)
+        waves = int(t.get("WAVES", 4))
+        unit.define("CL_HEAD_DIM", p["head_dim"])
+        unit.define("CL_ROWS", rows)
+        unit.define("CL_WAVES", waves)
+        unit.define("CL_PAGED", paged)
+        unit.define("CL_PAGE_SIZE", p.get("page_size", 1))
+        unit.define("CL_KV_HEADS", p.get("kv_heads", 1))
+        unit.define("CL_Q_HEADS", p.get("q_heads", 1))
+        unit.define("CL_SKV", p.get("skv", 0))
+        unit.define("CL_SCALE_LOG2E", _f(float(p.get("scale", 1.0)) * LOG2E))
+        for role, macro in (("Q", "CL_ARG_Q"), ("K", "CL_ARG_K"), ("V", "CL_ARG_V"), ("INDPTR", "CL_ARG_INDPTR"),
+                            ("INDICES", "CL_ARG_INDICES"), ("LAST", "CL_ARG_LAST")):
+            if role in op:
+                unit.define(macro, op[role])
+        if p["head_dim"] % 32 or not (p["vdim"] % 128 == 0 or p["vdim"] == 64):
+            raise CodegenError("decode attention needs head_dim % 32 == 0 and value width 64 or k*128")
+        splits = plan.split_factor or 1
+        row_tiles = -(-rows // 16)
+        unit.templates += ["attn_decode.hip", "attn_combine.hip"]
+        if partial:
+            from ..schedule.policy import attn_lds_bytes
+
+            unit.launch(ENTRY, (f"({units}) * {row_tiles}", splits, 1), waves * 64, attn_lds_bytes(waves, p["vdim"]),
+                        self._partial_args)
+        if combine:
+            entry, args = self._combine_args
+            unit.launch(entry, (f"ceildiv({grid_rows} * {p['vdim'] // 4}, 256)", 1, 1), 256, 0, args)
+
+    def _emit_mla_decode(self, unit, plan, params, partial, combine, fused):
+        p, t, op = plan.problem, plan.tiling, plan.operands
+        total_rows = p["batch"] * p["heads"]
+        emit_lse = bool(p.get("emit_lse"))
+        self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], total_rows, emit_lse)
+        waves = int(t.get("WAVES", 4))
+        if p["heads"] % (16 * waves):
+            raise CodegenError(f"{p['heads']} heads do not divide into {waves} waves of 16")
+        for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_SKV", p["skv"]),
+                     ("CL_WAVES", waves), ("CL_BATCH", p["batch"])):
+            unit.define(k, v)
+        unit.define("CL_SCALE_LOG2E", _f(float(p["scale"]) * LOG2E))
+        for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE")):
+            if role in op:
+                unit.define(macro, op[role])
+        splits = plan.split_factor or 1
+        unit.templates += ["mla_decode.hip", "attn_combine.hip"]
+        if partial:
+            from ..schedule.policy import mla_lds_bytes
+
+            grid = (p["batch"] * (p["heads"] // (16 * waves)), splits, 1)
+            unit.launch(ENTRY, grid, waves * 64, mla_lds_bytes(p["ckv"], p["kpe"]), self._partial_args)
+        if combine:
+            entry, args = self._combine_args
+            unit.launch(entry, (-(-(total_rows * (p["ckv"] // 4)) // 256), 1, 1), 256, 0, args)
+
+
+def parse_manifest(source: str) -> dict:
+    """The manifest a generated source carries (raises ``CodegenError`` when it has none)."""
+    try:
+        start = source.index(MANIFEST_BEGIN) + len(MANIFEST_BEGIN)
+        end = source.index(MANIFEST_END)
+    except ValueError:
+        raise CodegenError("source has no kernel manifest: not produced by HipCodeGen") from None
+    lines = [line[3:] if line.startswith("// ") else line.lstrip("/") for line in source[start:end].strip().splitlines()]
+    try:
+        return json.loads("\n".join(lines))
+    except json.JSONDecodeError as e:
+        raise CodegenError(f"kernel manifest is not valid JSON: {e}") from e
+
+
+__all__ = ["HipCodeGen", "parse_manifest", "ENTRY", "COMBINE_ENTRY", "TEMPLATE_DIR"]

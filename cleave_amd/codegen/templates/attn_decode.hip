@@ -1,0 +1,280 @@
+// ---- split-KV decode attention (GQA / MQA / MHA), dense or paged KV --------------------------
+//
+// One workgroup owns one (kv-head unit, 16-row query tile, KV split).  Its waves walk the
+// split's 32-token steps round-robin; nothing is staged through LDS on the way in: K and V
+// rows go HBM -> registers as 16-byte loads and straight into the matrix cores.
+//
+//   scores^T (tokens x rows) = K (tokens x d) * Q^T        K rows are the A operand as loaded
+//   out^T    (d x rows)     += V^T (d x tokens) * P^T      V is transposed 8x8 in registers;
+//                                                          P^T is the score tile *in place*
+//
+// so every softmax quantity of query row c lives in lanes with lane%16 == c and the running
+// max / sum / rescale never cross lanes except for one 4-way reduction per step.
+// The softmax is exact and online: each wave carries (m, l, O) and waves, then splits, are
+// merged by the usual max-rescale rule.  Emitter-supplied constants:
+//   CL_HEAD_DIM  d (multiple of 32)      CL_VDIM     value width (multiple of 128, or 64)
+//   CL_ROWS      query rows per kv unit  CL_WAVES    waves per workgroup
+//   CL_SPLITS    KV splits               CL_PAGED    0 dense, 1 paged
+//   CL_PAGE_SIZE tokens per page         CL_KV_HEADS kv heads in the cache (paged)
+//   CL_Q_HEADS   query heads (paged)     CL_SKV      kv length (dense)
+//   CL_SCALE_LOG2E softmax scale * log2(e) (dense; paged passes sm_scale at run time)
+//   CL_EMIT_LSE  also write the base-2 log-sum-exp
+
+#define ATT_STEP 32
+#define ATT_KJ (CL_HEAD_DIM / 32)            // score MFMAs per 16 tokens
+#define ATT_VC ((CL_VDIM + 127) / 128)       // 128-wide value chunks
+#define ATT_ROW_TILES ((CL_ROWS + 15) / 16)
+
+struct AttUnit {
+  const elem_t* q;      // first query row of this tile (row stride CL_HEAD_DIM)
+  const elem_t* k;      // dense: first K row of the unit; paged: cache base + head offset
+  const elem_t* v;
+  i64 row_stride;       // elements between consecutive tokens
+  int kv_len;           // valid tokens
+  int rows;             // real rows in this tile (1..16)
+  const int* pages;     // paged: this request's slice of the page table
+  int n_pages;          // paged: entries in that slice (>= 1 when kv_len > 0)
+  int pool_pages;       // paged: pages in the cache; page ids are clamped below this
+  i64 out_row;          // flattened (unit, row) index of the tile's first row
+};
+
+#if CL_PAGED
+CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) {
+  int pi = t / CL_PAGE_SIZE;
+  pi = pi < u.n_pages ? pi : u.n_pages - 1;
+  int pid = u.pages[pi];
+  pid = pid < u.pool_pages - 1 ? pid : u.pool_pages - 1;
+  pid = pid > 0 ? pid : 0;
+  const i64 page = pid;
+  return (page * CL_PAGE_SIZE + (t % CL_PAGE_SIZE)) * u.row_stride;
+}
+#else
+CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) { return (i64)t * u.row_stride; }
+#endif
+
+struct AttTile {               // one 32-token step's K and V, as loaded
+  u32x4 k[2][ATT_KJ];
+  u32x4 v[ATT_VC][8];
+};
+
+// Issue the loads of the step starting at token t0.  Tokens past kv_len are clamped onto the
+// last valid token (their scores are masked later), so no load leaves the tensor.
+CL_DEVICE void att_load(const AttUnit& u, int t0, int c, int g, AttTile& tile) {
+  const int last = u.kv_len - 1;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    int t = t0 + 16 * h + c;
+    t = t < last ? t : last;
+    const elem_t* row = u.k + att_token_offset(u, t) + 8 * g;
+#pragma unroll
+    for (int j = 0; j < ATT_KJ; ++j) tile.k[h][j] = ld16(row + 32 * j);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    int t = t0 + (e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4));
+    t = t < last ? t : last;
+    const elem_t* row = u.v + att_token_offset(u, t);
+#pragma unroll
+    for (int vc = 0; vc < ATT_VC; ++vc) {
+      int col = 128 * vc + 8 * c;
+      if (CL_VDIM % 128 != 0) col = col < CL_VDIM - 8 ? col : CL_VDIM - 8;
+      tile.v[vc][e] = ld16(row + col);
+    }
+  }
+}
+
+#if CL_EMIT_PARTIAL
+extern "C" __global__ void __launch_bounds__(CL_WAVES * 64)
+CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int split = blockIdx.y;
+  const int tile_id = blockIdx.x % ATT_ROW_TILES;
+  const int unit = blockIdx.x / ATT_ROW_TILES;
+
+  AttUnit u;
+  u.rows = CL_ROWS - 16 * tile_id < 16 ? CL_ROWS - 16 * tile_id : 16;
+#if CL_PAGED
+  // unit = request * kv_heads + kv head.  The request's length follows the page-granular
+  // CSR: every page but the last is full, the last holds kv_last_page_len tokens, and the
+  // sum is clamped to the pages the request owns.
+  const int req = unit / CL_KV_HEADS, head = unit % CL_KV_HEADS;
+  const int p0 = CL_ARG_INDPTR[req], p1 = CL_ARG_INDPTR[req + 1];
+  int n_pages = p1 - p0;
+  n_pages = n_pages > 0 ? n_pages : 0;
+  {
+    int avail = n_idx - p0;                       // never index past the table itself
+    n_pages = n_pages < avail ? n_pages : (avail > 0 ? avail : 0);
+  }
+#if CL_PAGE_SIZE > 1
+  int lastp = CL_ARG_LAST[req];
+  lastp = lastp > 0 ? lastp : 0;
+  int full = n_pages - 1 > 0 ? n_pages - 1 : 0;
+  int kv_len = full * CL_PAGE_SIZE + lastp;
+  kv_len = kv_len < n_pages * CL_PAGE_SIZE ? kv_len : n_pages * CL_PAGE_SIZE;
+#else
+  int kv_len = n_pages;
+#endif
+  u.kv_len = kv_len;
+  u.pages = CL_ARG_INDICES + p0;
+  u.n_pages = n_pages;
+  u.pool_pages = num_pages;
+  u.row_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
+  u.k = CL_ARG_K + (i64)head * CL_HEAD_DIM;
+  u.v = CL_ARG_V + (i64)head * CL_VDIM;
+  u.out_row = ((i64)req * CL_Q_HEADS + (i64)head * CL_ROWS) + 16 * tile_id;
+  u.q = CL_ARG_Q + u.out_row * CL_HEAD_DIM;
+  const float scale2 = sm_scale * 1.4426950408889634f;
+#else
+  u.kv_len = CL_SKV;
+  u.pages = nullptr;
+  u.n_pages = 0;
+  u.pool_pages = 0;
+  u.row_stride = CL_HEAD_DIM;
+  u.k = CL_ARG_K + (i64)unit * CL_SKV * CL_HEAD_DIM;
+  u.v = CL_ARG_V + (i64)unit * CL_SKV * CL_VDIM;
+  u.out_row = (i64)unit * CL_ROWS + 16 * tile_id;
+  u.q = CL_ARG_Q + u.out_row * CL_HEAD_DIM;
+  const float scale2 = CL_SCALE_LOG2E;
+#endif
+
+  // This split's steps: ceil(n_steps / SPLITS) each; a trailing split may own none.
+  const int n_steps = (u.kv_len + ATT_STEP - 1) / ATT_STEP;
+  const int per_split = (n_steps + CL_SPLITS - 1) / CL_SPLITS;
+  const int step_begin = split * per_split;
+  int step_end = step_begin + per_split;
+  step_end = step_end < n_steps ? step_end : n_steps;
+
+  // Query rows as the B operand: lane (c, g) holds Q[row c][32 j + 8 g .. +8]; padded rows are 0.
+  elem8 qf[ATT_KJ];
+  {
+    const bool live = c < u.rows;
+    const elem_t* row = u.q + (i64)(live ? c : 0) * CL_HEAD_DIM + 8 * g;
+#pragma unroll
+    for (int j = 0; j < ATT_KJ; ++j) {
+      u32x4 raw = ld16(row + 32 * j);
+      if (!live) raw = (u32x4){0u, 0u, 0u, 0u};
+      qf[j] = as_elem8(raw);
+    }
+  }
+
+  float m_run = CL_NEG_BIG;   // running max of the scaled scores (log2 domain), uniform over g
+  float l_run = 0.f;          // this lane's share of the running sum
+  f32x4 acc[ATT_VC][8];       // acc[vc][j][r] = O[row c][128 vc + 32 g + 8 r + j]
+#pragma unroll
+  for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[vc][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  AttTile cur, nxt;
+  int step = step_begin + wave;
+  if (step < step_end) att_load(u, step * ATT_STEP, c, g, cur);
+  for (; step < step_end; step += CL_WAVES) {
+    const int t0 = step * ATT_STEP;
+    const bool more = step + CL_WAVES < step_end;
+    if (more) att_load(u, (step + CL_WAVES) * ATT_STEP, c, g, nxt);
+
+    // scores^T for the two 16-token halves
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 st = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < ATT_KJ; ++j) st = mfma16(as_elem8(cur.k[h][j]), qf[j], st);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = t0 + 16 * h + 4 * g + r;
+        s[4 * h + r] = t < u.kv_len ? st[r] * scale2 : CL_NEG_BIG;
+      }
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+    mx = fmaxf(mx, lane_xor(mx, lane, 16));
+    mx = fmaxf(mx, lane_xor(mx, lane, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = fast_exp2(m_run - m_new);
+    m_run = m_new;
+    elem8 pf;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // masked slots hold CL_NEG_BIG; when the whole row is still masked m_new equals it too,
+      // so test the mask itself rather than trusting exp2 of a zero difference
+      float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;
+      elem_t pe = to_elem(p);
+      psum += to_f32(pe);            // the sum uses the weights the value product really sees
+      pf[i] = pe;
+    }
+    l_run = l_run * alpha + psum;
+
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // wave-uniform: skip when no max moved
+#pragma unroll
+      for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[vc][j] *= alpha;
+    }
+#pragma unroll
+    for (int vc = 0; vc < ATT_VC; ++vc) {
+      u32x4 vt[8];
+      transpose8x8(cur.v[vc], vt);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[vc][j] = mfma16(as_elem8(vt[j]), pf, acc[vc][j]);
+    }
+    if (more) cur = nxt;
+  }
+
+  // ---- merge the workgroup's waves through LDS ----------------------------------------------
+  l_run += lane_xor(l_run, lane, 16);
+  l_run += lane_xor(l_run, lane, 32);
+  extern __shared__ float att_lds[];
+  float* sh_m = att_lds;                               // [WAVES][16]
+  float* sh_l = att_lds + CL_WAVES * 16;               // [WAVES][16]
+  float* sh_o = att_lds + CL_WAVES * 32;               // [WAVES][16][VDIM]
+  if (g == 0) {
+    sh_m[wave * 16 + c] = m_run;
+    sh_l[wave * 16 + c] = l_run;
+  }
+#pragma unroll
+  for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int d = 128 * vc + 32 * g + 8 * r + j;
+        if (CL_VDIM % 128 == 0 || d < CL_VDIM) sh_o[(wave * 16 + c) * CL_VDIM + d] = acc[vc][j][r];
+      }
+  __syncthreads();
+
+  for (int idx = threadIdx.x; idx < 16 * CL_VDIM; idx += CL_WAVES * 64) {
+    const int row = idx / CL_VDIM, d = idx % CL_VDIM;
+    if (row >= u.rows) continue;
+    float m = sh_m[row];
+#pragma unroll
+    for (int w = 1; w < CL_WAVES; ++w) m = fmaxf(m, sh_m[w * 16 + row]);
+    float l = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < CL_WAVES; ++w) {
+      const float f = fast_exp2(sh_m[w * 16 + row] - m);
+      l += sh_l[w * 16 + row] * f;
+      o += sh_o[(w * 16 + row) * CL_VDIM + d] * f;
+    }
+    const i64 orow = u.out_row + row;
+#if CL_SPLITS > 1
+    const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
+    CL_ARG_PO[prow * CL_VDIM + d] = o;
+    if (d == 0) {
+      CL_ARG_PM[prow] = m;
+      CL_ARG_PL[prow] = l;
+    }
+#else
+    // An empty request has l == 0: the floor turns 0/0 into 0 and its lse is -inf.
+    CL_ARG_OUT[orow * CL_VDIM + d] = to_elem(o / fmaxf(l, 1.0e-30f));
+#if CL_EMIT_LSE
+    if (d == 0) CL_ARG_LSE[orow] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
+#endif
+#endif
+  }
+}
+#endif  // CL_EMIT_PARTIAL
+

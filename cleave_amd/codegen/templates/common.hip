@@ -1,0 +1,70 @@
+// ---- shared device helpers (gfx950: wave64, MFMA 16x16x32 f16/bf16) ------------------------
+// Element type is chosen by the emitter: CL_BF16 == 1 selects bfloat16, else half.
+#if CL_BF16
+typedef __bf16 elem_t;
+#else
+typedef _Float16 elem_t;
+#endif
+typedef elem_t elem8 __attribute__((ext_vector_type(8)));
+typedef elem_t elem4 __attribute__((ext_vector_type(4)));
+typedef elem_t elem2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef long long i64;
+
+#define CL_DEVICE static __device__ __forceinline__
+#define CL_METHOD __device__ __forceinline__
+#define CL_NEG_BIG (-1.0e30f)
+#define CL_NEG_INF (__builtin_bit_cast(float, 0xff800000u))
+
+// D(16x16 f32) += A(16x32) * B(32x16).  Lane l supplies A[row l%16][k-slots of group l/16] and
+// B[k-slots of group l/16][col l%16]; it receives D[rows 4*(l/16)+0..3][col l%16].  A and B are
+// paired slot by slot, so any consistent assignment of the contraction index to slots works.
+CL_DEVICE f32x4 mfma16(elem8 a, elem8 b, f32x4 c) {
+#if CL_BF16
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+CL_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+CL_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+CL_DEVICE float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+CL_DEVICE float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// Value of `v` held by lane (lane ^ mask); mask is a compile-time constant < 64.
+CL_DEVICE float lane_xor(float v, int lane, int mask) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __builtin_bit_cast(int, v)));
+}
+CL_DEVICE float lane_read(float v, int src_lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v)));
+}
+
+// 16-byte global load / store of eight elements.
+CL_DEVICE u32x4 ld16(const elem_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+CL_DEVICE void st16(elem_t* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+CL_DEVICE elem8 as_elem8(u32x4 v) { return __builtin_bit_cast(elem8, v); }
+CL_DEVICE u32x4 as_u32x4(elem8 v) { return __builtin_bit_cast(u32x4, v); }
+
+// In-register 8x8 transpose of 16-bit elements.  in[e] holds row e (eight columns); out[j]
+// receives column j (eight rows).  Row-major global tensors hand a lane eight neighbours of
+// the *minor* axis per 16-byte load, while a matrix-core operand wants eight neighbours of
+// the contraction axis: this turns one into the other without touching LDS.
+CL_DEVICE void transpose8x8(const u32x4 (&in)[8], u32x4 (&out)[8]) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {      // column pair (2q, 2q+1) lives in dword q of every row
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {    // row pair (2p, 2p+1) becomes dword p of the output
+      u32 x = in[2 * p][q], y = in[2 * p + 1][q];
+      out[2 * q][p] = (x & 0xffffu) | (y << 16);
+      out[2 * q + 1][p] = (x >> 16) | (y & 0xffff0000u);
+    }
+  }
+}
+
+CL_DEVICE elem_t to_elem(float x) { return (elem_t)x; }
+CL_DEVICE float to_f32(elem_t x) { return (float)x; }

@@ -1,0 +1,227 @@
+// ---- weight-streaming matmul for few rows: Y[M<=64, N] = f(X)[M, K] * W[K, N] ---------------
+//
+// With M this small the kernel is a pure stream of W out of HBM, so W never touches LDS:
+// each wave owns 128 output columns and walks its K range 32 rows at a time.  A lane loads
+// an 8(k) x 8(n) block of W as eight 16-byte row segments (sixteen lanes cover 256 contiguous
+// bytes of a row), transposes it in registers and feeds eight 16x16x32 MFMAs whose B operands
+// are the eight columns of that block; X rows are the A operand, read from L2.
+//
+// Optional fused RMSNorm (CL_NORM): f(X) = X * gamma (gamma optional), the row sum of squares
+// is accumulated from the same X fragments, and the epilogue multiplies row m by
+// rsqrt(sumsq[m] / K + eps).  With CL_SPLITS > 1 the block writes f32 partial products (and
+// partial sums of squares); the combine kernel adds them up and normalises.
+//
+//   CL_M, CL_N, CL_K   problem size (K % 32 == 0, N % 8 == 0)
+//   CL_WAVES_N         waves side by side along N (each 128 columns)
+//   CL_WAVES_K         waves sharing one column slab, splitting the block's K range
+//   CL_SPLITS          K splits across workgroups (grid.y)
+//   CL_NORM            0 plain, 1 RMSNorm epilogue; CL_GAMMA: 1 when a (K) weight multiplies X
+//   CL_EPS             epsilon inside the rsqrt
+
+#define SK_MT ((CL_M + 15) / 16)
+#define SK_COLS 128
+#define SK_STEP 32
+#define SK_THREADS (CL_WAVES_N * CL_WAVES_K * 64)
+
+struct SkTile {
+  u32x4 w[8];
+};
+
+CL_DEVICE void sk_load_w(const elem_t* __restrict__ W, int k0, int ncol, int g, SkTile& t) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) t.w[e] = ld16(W + (i64)(k0 + 8 * g + e) * CL_N + ncol);
+}
+
+#if CL_EMIT_PARTIAL
+extern "C" __global__ void __launch_bounds__(SK_THREADS)
+CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int wn = wave % CL_WAVES_N, wk = wave / CL_WAVES_N;
+  const int split = blockIdx.y;
+
+  // columns of this wave; the last slab may hang over N: loads are clamped, stores masked
+  const int n_base = (blockIdx.x * CL_WAVES_N + wn) * SK_COLS;
+  int ncol = n_base + 8 * c;
+  const bool col_live = ncol < CL_N;
+  ncol = col_live ? ncol : CL_N - 8;
+
+  // K range: split -> waves_k, contiguous chunks of whole 32-row steps
+  constexpr int steps_total = CL_K / SK_STEP;
+  constexpr int steps_per_split = (steps_total + CL_SPLITS - 1) / CL_SPLITS;
+  constexpr int steps_per_wave = (steps_per_split + CL_WAVES_K - 1) / CL_WAVES_K;
+  int s_begin = split * steps_per_split + wk * steps_per_wave;
+  int s_end = s_begin + steps_per_wave;
+  {
+    int lim = (split + 1) * steps_per_split;
+    lim = lim < steps_total ? lim : steps_total;
+    s_end = s_end < lim ? s_end : lim;
+  }
+
+  f32x4 acc[SK_MT][8];
+#pragma unroll
+  for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[mt][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float ss[SK_MT];
+#pragma unroll
+  for (int mt = 0; mt < SK_MT; ++mt) ss[mt] = 0.f;
+
+  SkTile cur, nx1, nx2;
+  if (s_begin < s_end) sk_load_w(CL_ARG_W, s_begin * SK_STEP, ncol, g, cur);
+  if (s_begin + 1 < s_end) sk_load_w(CL_ARG_W, (s_begin + 1) * SK_STEP, ncol, g, nx1);
+  for (int s = s_begin; s < s_end; ++s) {
+    const int k0 = s * SK_STEP;
+    if (s + 2 < s_end) sk_load_w(CL_ARG_W, (s + 2) * SK_STEP, ncol, g, nx2);
+
+    // X fragments (A operand): lane (c, g) holds X[16 mt + c][k0 + 8 g .. +8]
+    elem8 xa[SK_MT];
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt) {
+      const int m = 16 * mt + c;
+      const bool live = m < CL_M;
+      u32x4 raw = ld16(CL_ARG_X + (i64)(live ? m : 0) * CL_K + k0 + 8 * g);
+      if (!live) raw = (u32x4){0u, 0u, 0u, 0u};
+      elem8 x = as_elem8(raw);
+#if CL_NORM
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float xf = to_f32(x[i]);
+        ss[mt] += xf * xf;
+      }
+#if CL_GAMMA
+      elem8 gm = as_elem8(ld16(CL_ARG_GAMMA + k0 + 8 * g));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = to_elem(to_f32(x[i]) * to_f32(gm[i]));
+#endif
+#endif
+      xa[mt] = x;
+    }
+
+    u32x4 wt[8];
+    transpose8x8(cur.w, wt);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int mt = 0; mt < SK_MT; ++mt) acc[mt][j] = mfma16(xa[mt], as_elem8(wt[j]), acc[mt][j]);
+    cur = nx1;
+    nx1 = nx2;
+  }
+
+  // ---- reduce across the waves that share a column slab ------------------------------------
+  // acc[mt][j][r] = Y[16 mt + 4 g + r][n_base + 8 c + j]
+#if CL_NORM
+#pragma unroll
+  for (int mt = 0; mt < SK_MT; ++mt) {
+    ss[mt] += lane_xor(ss[mt], lane, 16);
+    ss[mt] += lane_xor(ss[mt], lane, 32);
+  }
+#endif
+  extern __shared__ float sk_lds[];
+  float* sh_acc = sk_lds;                                     // [WAVES_K-1][WAVES_N][MT*8*4][64]
+  float* sh_ss = sk_lds + (CL_WAVES_K - 1) * CL_WAVES_N * SK_MT * 32 * 64;  // [WAVES_K][MT*16]
+#if CL_WAVES_K > 1
+  if (wk > 0) {
+    float* dst = sh_acc + ((i64)((wk - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[((mt * 8 + j) * 4 + r) * 64 + lane] = acc[mt][j][r];
+  }
+#endif
+#if CL_NORM
+  if (wn == 0 && g == 0) {
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt) sh_ss[wk * SK_MT * 16 + mt * 16 + c] = ss[mt];
+  }
+#endif
+  __syncthreads();
+  if (wk != 0) return;
+#if CL_WAVES_K > 1
+#pragma unroll
+  for (int w = 1; w < CL_WAVES_K; ++w) {
+    const float* src = sh_acc + ((i64)((w - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[mt][j][r] += src[((mt * 8 + j) * 4 + r) * 64 + lane];
+  }
+#endif
+
+  // ---- epilogue ----------------------------------------------------------------------------
+#pragma unroll
+  for (int mt = 0; mt < SK_MT; ++mt) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = 16 * mt + 4 * g + r;
+      if (m >= CL_M) continue;
+#if CL_NORM
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < CL_WAVES_K; ++w) tot += sh_ss[w * SK_MT * 16 + mt * 16 + 4 * g + r];
+#endif
+#if CL_SPLITS > 1
+      float* prow = CL_ARG_PACC + ((i64)split * CL_M + m) * CL_N + n_base + 8 * c;
+      if (col_live) {
+        *reinterpret_cast<f32x4*>(prow) = (f32x4){acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]};
+        *reinterpret_cast<f32x4*>(prow + 4) = (f32x4){acc[mt][4][r], acc[mt][5][r], acc[mt][6][r], acc[mt][7][r]};
+      }
+#if CL_NORM
+      if (blockIdx.x == 0 && wn == 0 && c == 0) CL_ARG_PSS[(i64)split * CL_M + m] = tot;
+#endif
+#else
+#if CL_NORM
+      const float rs = fast_rsqrt(tot * (1.0f / CL_K) + CL_EPS);
+#else
+      const float rs = 1.0f;
+#endif
+      elem8 y;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = to_elem(acc[mt][j][r] * rs);
+      if (col_live) st16(CL_ARG_OUT + (i64)m * CL_N + n_base + 8 * c, as_u32x4(y));
+#endif
+    }
+  }
+}
+#endif  // CL_EMIT_PARTIAL
+
+#if CL_SPLITS > 1 && CL_EMIT_COMBINE
+// Combine: Y[m][n] = (sum_s P[s][m][n]) * rsqrt(sum_s ss[s][m] / K + eps).  Eight columns per thread.
+extern "C" __global__ void __launch_bounds__(256)
+CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
+  const i64 total = (i64)CL_M * (CL_N / 8);
+  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int m = (int)(idx / (CL_N / 8));
+  const int n = (int)(idx % (CL_N / 8)) * 8;
+  f32x4 a = (f32x4){0.f, 0.f, 0.f, 0.f}, b = a;
+#if CL_NORM
+  float tot = 0.f;
+#endif
+#pragma unroll
+  for (int s = 0; s < CL_SPLITS; ++s) {
+    const float* p = CL_CARG_PACC + ((i64)s * CL_M + m) * CL_N + n;
+    a += *reinterpret_cast<const f32x4*>(p);
+    b += *reinterpret_cast<const f32x4*>(p + 4);
+#if CL_NORM
+    tot += CL_CARG_PSS[(i64)s * CL_M + m];
+#endif
+  }
+#if CL_NORM
+  const float rs = fast_rsqrt(tot * (1.0f / CL_K) + CL_EPS);
+#else
+  const float rs = 1.0f;
+#endif
+  elem8 y;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    y[i] = to_elem(a[i] * rs);
+    y[4 + i] = to_elem(b[i] * rs);
+  }
+  st16(CL_CARG_OUT + (i64)m * CL_N + n, as_u32x4(y));
+}
+#endif

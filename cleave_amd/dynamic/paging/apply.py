@@ -1,0 +1,200 @@
+"""Wrap a scheduled dense attention plan in a paged access layer.
+
+Entry points and gates of ``python/cleave/dynamic/paging/apply.py:28-127`` and
+``constraints.py:20-142``: ``apply_paging(plan, spec)`` for a single kernel,
+``apply_paging_split([partial, combine], spec)`` / ``build_split_decode(spec, dense, split,
+comb)`` for a split-KV pair, ``can_page`` / ``paging_accept`` as search filters.  The dense
+plan contributes the tiling (waves per workgroup, 32-token steps); the spec contributes the
+operator: page table, per-request lengths, run-time scale, symbolic batch.
+
+Parameter order of the emitted kernel is the reference's
+(``tests/graph/handwritten/expected_kernels/gqa_paged_decode_h32_kv8_d128_ps64.py:301-312``):
+query, caches, indptr, indices, [last page len], scale, [partials], out, lse.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+from ...schedule.plan import KernelPlan, ParamSpec
+from .errors import NotDenseAttention, UnsupportedTiling
+from .kinds import BUILT_KINDS, PAGED_DECODE, PAGED_DECODE_SLAB
+from .specs import CombineTiling, MLASpec, PagingSpec
+
+KV_STEP = 32  # tokens one wave consumes per step of the decode template
+
+
+@dataclass(frozen=True)
+class DenseAttention:
+    """What the access layer reads off a scheduled dense attention plan
+    (``python/cleave/dynamic/paging/recognize.py:20-646``)."""
+
+    query_rows: int
+    kv_tile: int
+    head_dim: int
+    n_threads: int
+    dtype: str
+    out_dtype: str
+    accum_dtype: str = "float32"
+    waves: int = 4
+    split: int | None = None
+
+
+def read_dense_attention(plan: KernelPlan) -> DenseAttention:
+    if not isinstance(plan, KernelPlan) or plan.template != "attn_decode" or plan.family != "attention":
+        raise NotDenseAttention("expected a scheduled dense attention plan (template attn_decode)")
+    p = plan.problem
+    if p.get("paged"):
+        raise NotDenseAttention("the plan is already paged")
+    if p["head_dim"] != p["vdim"]:
+        raise NotDenseAttention(f"K width {p['head_dim']} != V width {p['vdim']}: not a GQA body")
+    expect = p["head_dim"] ** -0.5
+    if abs(p["scale"] - expect) > 1e-6 * expect:
+        raise NotDenseAttention(f"the dense body's scale {p['scale']} is not 1/sqrt(d) = {expect}; the run-time "
+                                "sm_scale replaces exactly that constant")
+    rows = p["group"] * p["sq"]
+    waves = int(plan.tiling.get("WAVES", 4))
+    return DenseAttention(query_rows=-(-rows // 16) * 16, kv_tile=KV_STEP, head_dim=p["head_dim"],
+                          n_threads=waves * 64, dtype=plan.dtype, out_dtype=plan.dtype, waves=waves,
+                          split=plan.split_factor)
+
+
+def read_dense_partial(plan: KernelPlan):
+    dense = read_dense_attention(plan)
+    if plan.role != "partial" or not plan.split_factor:
+        raise NotDenseAttention("expected the partial plan of a split pair")
+    return dense, int(plan.split_factor)
+
+
+def read_dense_combine(plan: KernelPlan) -> CombineTiling:
+    if not isinstance(plan, KernelPlan) or plan.role != "combine" or not plan.split_factor:
+        raise NotDenseAttention("expected the combine plan of a split pair")
+    return CombineTiling(split=int(plan.split_factor))
+
+
+def _check_tiling(spec, dense: DenseAttention, split: bool = False) -> None:
+    if isinstance(spec, MLASpec):
+        raise UnsupportedTiling("the paged MLA layer is not built by this back end yet (dense MLA decode is)")
+    if spec.kind not in BUILT_KINDS:
+        raise UnsupportedTiling(f"the {spec.kind!r} layer is not built by this back end yet "
+                                f"(built: {', '.join(BUILT_KINDS)})")
+    if split and spec.kind not in (PAGED_DECODE, PAGED_DECODE_SLAB):
+        raise UnsupportedTiling(f"split-KV is a decode transformation; got the {spec.kind!r} layer")
+    if dense.query_rows < spec.group:
+        raise UnsupportedTiling(f"a block's query tile holds {dense.query_rows} rows but the head group needs "
+                                f"{spec.group}; re-tile with at least {spec.group} query rows")
+    if dense.head_dim % 32 or not (dense.head_dim % 128 == 0 or dense.head_dim == 64):
+        raise UnsupportedTiling(f"head_dim {dense.head_dim} is not 64 or a multiple of 128")
+
+
+def _paged_params(spec: PagingSpec, dense: DenseAttention):
+    d, dt = dense.head_dim, dense.dtype
+    b, pages = spec.batch_dim, spec.pages_dim
+    ph = lambda n: f"PlaceHolder_{n}"  # noqa: E731
+    params = [
+        ParamSpec(ph(spec.query_input), dt, (b, spec.num_qo_heads, d), "input"),
+        ParamSpec(ph(spec.cache_inputs[0]), dt, (pages, spec.page_size, spec.num_kv_heads, d), "input"),
+        ParamSpec(ph(spec.cache_inputs[1]), dt, (pages, spec.page_size, spec.num_kv_heads, d), "input"),
+        ParamSpec(ph(spec.indptr_input), "int32", (spec.indptr_dim,), "input"),
+        ParamSpec(ph(spec.index_input), "int32", (spec.index_dim,), "input"),
+    ]
+    operands = {"Q": params[0].name, "K": params[1].name, "V": params[2].name,
+                "INDPTR": params[3].name, "INDICES": params[4].name}
+    if spec.kind == PAGED_DECODE_SLAB:
+        params.append(ParamSpec(ph(spec.last_page_len_input), "int32", (b,), "input"))
+        operands["LAST"] = params[-1].name
+    params.append(ParamSpec(spec.scale_input, "float32", (), "scalar"))
+    return params, operands
+
+
+def _paged_outputs(spec: PagingSpec, dense: DenseAttention):
+    outs = [ParamSpec("OutputNode_0", dense.out_dtype, (spec.batch_dim, spec.num_qo_heads, dense.head_dim), "output")]
+    operands = {"OUT": "OutputNode_0"}
+    if spec.emit_lse:
+        outs.append(ParamSpec("OutputNode_1", "float32", (spec.batch_dim, spec.num_qo_heads), "output"))
+        operands["OUT1"] = "OutputNode_1"
+    return outs, operands
+
+
+def _paged_problem(spec: PagingSpec, dense: DenseAttention) -> dict:
+    return {"paged": True, "page_size": spec.page_size, "kv_heads": spec.num_kv_heads,
+            "q_heads": spec.num_qo_heads, "group": spec.group, "sq": 1, "head_dim": dense.head_dim,
+            "vdim": dense.head_dim, "emit_lse": bool(spec.emit_lse), "units": None, "skv": 0, "scale": 1.0,
+            "dim_names": {"batch": spec.batch_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim}}
+
+
+def _plan(spec, dense, role, params, operands, split=None) -> KernelPlan:
+    dyn = (spec.batch_dim, spec.pages_dim, spec.index_dim)
+    label = f"kv={dense.kv_tile} q={dense.query_rows} thr={dense.n_threads}"
+    return KernelPlan(template="attn_decode", role=role, family="attention", dtype=dense.dtype,
+                      problem=_paged_problem(spec, dense), tiling={"WAVES": dense.waves}, params=params,
+                      operands=operands, split_factor=split, dyn_dims=dyn, n_threads=dense.n_threads, label=label)
+
+
+def apply_paging(plan: KernelPlan, spec) -> KernelPlan:
+    """A single paged decode kernel at ``plan``'s tiling."""
+    spec.validate()
+    dense = read_dense_attention(plan)
+    _check_tiling(spec, dense)
+    params, operands = _paged_params(spec, dense)
+    outs, out_ops = _paged_outputs(spec, dense)
+    return _plan(spec, dense, "main", params + outs, {**operands, **out_ops})
+
+
+def build_split_decode(spec, dense: DenseAttention, split: int, comb: CombineTiling) -> list:
+    """``[partial, combine]`` paged plans for a split-KV decode; ``HipCodeGen().gen`` fuses them
+    into one source with two kernels sharing the partial buffers."""
+    spec.validate()
+    if comb.split != split:
+        raise UnsupportedTiling(f"the combine tiling is for {comb.split} splits but the partial makes {split}")
+    comb.validate(dense.head_dim)
+    _check_tiling(spec, dense, split=True)
+    params, operands = _paged_params(spec, dense)
+    b, h, d = spec.batch_dim, spec.num_qo_heads, dense.head_dim
+    # split-major partials: one request's splits sit one stride apart
+    # (python/cleave/dynamic/paging/tensor_maps.py:41-69)
+    bufs = [("PM", (split, b, h)), ("PL", (split, b, h)), ("PO", (split, b, h, d))]
+    part_outs = [ParamSpec(f"OutputNode_{i}", "float32", shape, "output") for i, (_, shape) in enumerate(bufs)]
+    part_ops = {**operands, **{name: p.name for (name, _), p in zip(bufs, part_outs)}}
+    partial = _plan(spec, dense, "partial", params + part_outs, part_ops, split)
+    comb_ins = [ParamSpec(f"PlaceHolder_{name}", "float32", shape, "input") for name, shape in bufs]
+    outs, out_ops = _paged_outputs(spec, dense)
+    comb_ops = {**{name: p.name for (name, _), p in zip(bufs, comb_ins)}, **out_ops}
+    combine = _plan(spec, dense, "combine", comb_ins + outs, comb_ops, split)
+    return [partial, combine]
+
+
+def apply_paging_split(plans, spec) -> list:
+    if len(plans) != 2:
+        raise NotDenseAttention(f"expected a [partial, combine] pair, got {len(plans)} plans")
+    partial, combine = plans
+    spec.validate()
+    dense, split = read_dense_partial(partial)
+    comb = read_dense_combine(combine)
+    if comb.split != split:
+        raise NotDenseAttention(f"the partial makes {split} splits but the combine sums {comb.split}")
+    return build_split_decode(spec, dense, split, comb)
+
+
+def can_page(plan, spec) -> bool:
+    from ...core.errors import PagingRefusal
+
+    try:
+        spec.validate()
+        _check_tiling(spec, read_dense_attention(plan))
+    except PagingRefusal:
+        return False
+    return True
+
+
+def paging_accept(spec):
+    """A ``search_tiling(accept=...)`` filter: apply the candidate, then ``can_page`` it."""
+    from ...schedule import apply_tiling
+
+    def accept(cand) -> bool:
+        try:
+            return can_page(apply_tiling(cand), spec)
+        except Exception:  # noqa: BLE001 - a filter answers, it does not stop the search
+            return False
+
+    return accept

@@ -1,0 +1,147 @@
+"""Inputs and torch references of the paged attention operators, used to validate candidates.
+
+Restates ``python/cleave/dynamic/reference.py:23-200`` for the layers this back end builds,
+with two differences: the element dtype is a parameter (the reference hard-codes bf16 at
+``:19,136-140``) and so is the device (default "cuda").  Conventions kept: page tables are a
+seeded random permutation of the pool so the gather is genuinely scattered (``:44-49``); a
+request with no keys yields 0 in the output and -inf in the base-2 lse (``:71-82``); logits
+are evaluated in fp32, in query chunks so they stay bounded (``:62-105``).
+"""
+
+from __future__ import annotations
+
+import math
+
+SEED = 0
+NEG_INF = float("-inf")
+CHUNK_ELEMS = 1 << 27   # most fp32 logits alive at once
+
+
+def _torch():
+    import torch
+
+    return torch
+
+
+def _indptr(lengths) -> list:
+    out = [0]
+    for n in lengths:
+        out.append(out[-1] + int(n))
+    return out
+
+
+def _i32(values, device):
+    torch = _torch()
+    return torch.tensor(list(values), device=device, dtype=torch.int32)
+
+
+def _generator(device, seed=SEED):
+    torch = _torch()
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    return gen
+
+
+def _page_table(num_pages, count, device, seed=SEED):
+    torch = _torch()
+    perm = torch.randperm(num_pages, device=device, generator=_generator(device, seed))
+    return perm[:count].to(torch.int32)
+
+
+def _pad_indices(kv_indices, n_idx):
+    torch = _torch()
+    short = n_idx - kv_indices.numel()
+    assert short >= 0, (kv_indices.numel(), n_idx)
+    if short == 0:
+        return kv_indices
+    return torch.cat([kv_indices, torch.zeros(short, device=kv_indices.device, dtype=torch.int32)])
+
+
+def _finish(logits):
+    """Softmax weights and base-2 lse of a (n_q, heads, n_kv) block; fully masked rows get zero
+    weights and -inf instead of NaN."""
+    torch = _torch()
+    lse = torch.logsumexp(logits, dim=-1) / math.log(2.0)
+    weights = torch.softmax(logits, dim=-1)
+    dead = torch.isneginf(lse)
+    if dead.any():
+        weights = weights.masked_fill(dead[..., None], 0.0)
+    return weights, lse
+
+
+def _attend(q, k, v, scale, mask=None):
+    """One request: ``q`` (n_q, heads, d), ``k``/``v`` (n_kv, heads, d) -> out fp32, lse."""
+    torch = _torch()
+    n_q, heads, _ = q.shape
+    kf, vf = k.float(), v.float()
+    step = max(1, min(n_q, CHUNK_ELEMS // max(1, heads * k.shape[0])))
+    outs, lses = [], []
+    for lo in range(0, n_q, step):
+        hi = min(lo + step, n_q)
+        logits = torch.einsum("qhd,khd->qhk", q[lo:hi].float(), kf) * scale
+        if mask is not None:
+            logits = logits.masked_fill(~mask[lo:hi, None, :], NEG_INF)
+        w, lse = _finish(logits)
+        outs.append(torch.einsum("qhk,khd->qhd", w, vf))
+        lses.append(lse)
+    return torch.cat(outs), torch.cat(lses)
+
+
+def paged_tokens(kv_indices, base, kv_len, page_size):
+    """``(page_of, slot_of)`` for the ``kv_len`` tokens of the request whose table slice starts at
+    ``base``: pages in table order, each page's slots in order, clipped to the length."""
+    torch = _torch()
+    n_pages = -(-kv_len // page_size)
+    pages = kv_indices[base:base + n_pages].long()
+    if page_size == 1:
+        return pages, torch.zeros_like(pages)
+    slot = torch.arange(page_size, device=kv_indices.device)
+    page_of = pages[:, None].expand(-1, page_size).reshape(-1)[:kv_len]
+    slot_of = slot[None, :].expand(pages.numel(), -1).reshape(-1)[:kv_len]
+    return page_of, slot_of
+
+
+def gqa_paged_decode_inputs(dims, kv_lens, page_size=1, scale=None, dtype=None, device="cuda", seed=SEED):
+    """The operator's arguments in declaration order: q, k_cache, v_cache, kv_indptr, kv_indices,
+    [kv_last_page_len], sm_scale.  ``dims`` = (batch, qo_heads, kv_heads, head_dim, num_pages, n_idx)."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    batch, hq, hkv, d, num_pages, n_idx = dims[:6]
+    gen = _generator(device, seed)
+    pages_per_req = [-(-int(n) // page_size) for n in kv_lens]
+    kv_indices = _pad_indices(_page_table(num_pages, sum(pages_per_req), device, seed), n_idx)
+
+    def randn(*shape):
+        return torch.randn(*shape, device=device, dtype=dtype, generator=gen)
+
+    args = [randn(batch, hq, d), randn(num_pages, page_size, hkv, d), randn(num_pages, page_size, hkv, d),
+            _i32(_indptr(pages_per_req), device), kv_indices]
+    if page_size != 1:
+        args.append(_i32([n - (p - 1) * page_size if p else 0 for n, p in zip(kv_lens, pages_per_req)], device))
+    args.append(float(d) ** -0.5 if scale is None else float(scale))
+    return args
+
+
+def gqa_paged_decode_reference(dims, kv_lens, page_size=1, dtype=None):
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    batch, hq, hkv, d = dims[:4]
+    group = hq // hkv
+
+    def reference(q, k_cache, v_cache, kv_indptr, kv_indices, *rest):
+        sm_scale = rest[-1]
+        out = torch.zeros(batch, hq, d, device=q.device, dtype=dtype)
+        lse = torch.full((batch, hq), NEG_INF, device=q.device, dtype=torch.float32)
+        starts = kv_indptr.tolist()
+        for b, kv_len in enumerate(kv_lens):
+            if kv_len <= 0:
+                continue
+            page_of, slot_of = paged_tokens(kv_indices, int(starts[b]), int(kv_len), page_size)
+            kk = k_cache[page_of, slot_of].repeat_interleave(group, dim=1)
+            vv = v_cache[page_of, slot_of].repeat_interleave(group, dim=1)
+            o, l = _attend(q[b:b + 1], kk, vv, sm_scale)
+            out[b] = o[0].to(dtype)
+            lse[b] = l[0]
+        return [out, lse]
+
+    return reference

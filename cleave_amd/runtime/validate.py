@@ -1,0 +1,141 @@
+"""Tolerances, the on-disk reference a worker validates against, and the check itself
+(``python/cleave/runtime/validate.py:19-197``)."""
+
+from __future__ import annotations
+
+import contextlib
+import os
+from dataclasses import dataclass
+from pathlib import Path
+
+from .gpu import _gpu_exec_guard
+from .timer import mean_launch_ms
+
+
+@dataclass(frozen=True)
+class Tolerance:
+    rtol: float
+    atol: float
+    equal_nan: bool = False
+
+
+# The loose default bound of the reference; per-operator tolerances tighten it.
+DEFAULT_TOLERANCE = Tolerance(rtol=0.5, atol=0.5)
+# What every selected candidate of this back end is held to against the fp32-accumulated reference.
+STRICT_TOLERANCE = Tolerance(rtol=1e-2, atol=1e-2)
+
+
+@dataclass(frozen=True)
+class BenchOptions:
+    warmup: int = 16
+    iters: int = 1000
+
+
+@contextlib.contextmanager
+def _stage(name):
+    """Tag an escaping exception with the stage (compile / validate / bench) it came from."""
+    try:
+        yield
+    except BaseException as exc:
+        if getattr(exc, "_cleave_stage", None) is None:
+            try:
+                exc._cleave_stage = name
+            except Exception:  # noqa: BLE001 - some builtins refuse attributes
+                pass
+        raise
+
+
+def _live_bytes(tensors) -> int:
+    return sum(t.element_size() * t.nelement() for t in tensors)
+
+
+_BENCH_BATCH = 100
+
+
+def benchmark_compiled_kernel(kernel, input_tensors, *, warmup_iters=0, profile_iters=1) -> float:
+    """Mean milliseconds per launch of ``kernel(*input_tensors)``."""
+    return mean_launch_ms(kernel, input_tensors, warmup=warmup_iters, iters=profile_iters, batch=_BENCH_BATCH)
+
+
+_REFERENCE_FILE = "reference.pt"
+
+
+def _reference_path(cache_dir) -> Path:
+    return Path(cache_dir) / _REFERENCE_FILE
+
+
+def publish_reference(reference_cache_dir, graph, dtype, device: str = "cuda"):
+    """Build inputs + reference once in the parent and save them for the workers.
+    Returns ``(out_idx, io_bytes)``; ``io_bytes`` sizes worker parallelism."""
+    import torch
+
+    from .reference import build_inputs_and_reference
+
+    with _gpu_exec_guard():
+        inputs_by_name, reference, out_idx = build_inputs_and_reference(graph, dtype, device)
+        path = _reference_path(reference_cache_dir)
+        os.makedirs(reference_cache_dir, exist_ok=True)
+        tmp = path.with_name(f"{path.name}.tmp.{os.getpid()}")
+        torch.save({"inputs_by_name": {k: v.cpu() for k, v in inputs_by_name.items()},
+                    "reference": [r.cpu() for r in reference]}, tmp)
+        os.replace(tmp, path)
+        io_bytes = _live_bytes(inputs_by_name.values()) + _live_bytes(reference)
+        del inputs_by_name, reference
+        if torch.cuda.is_available():
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+    return out_idx, io_bytes
+
+
+def _load_reference(reference_cache_dir, device: str = "cuda"):
+    import torch
+
+    payload = torch.load(_reference_path(reference_cache_dir), map_location=device, weights_only=True)
+    return dict(payload["inputs_by_name"]), list(payload["reference"])
+
+
+def _as_list(x):
+    return list(x) if isinstance(x, (tuple, list)) else [x]
+
+
+def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance = DEFAULT_TOLERANCE):
+    """Run ``kernel(*inputs)`` and assert every output is within ``tolerance`` of ``reference``."""
+    import torch
+
+    from .reference import reconcile_output_layout
+
+    actual = _as_list(kernel(*inputs))
+    torch.cuda.synchronize()
+    assert len(actual) == len(reference), (
+        f"Kernel returned {len(actual)} outputs but the reference has {len(reference)}.")
+    for got, want in zip(actual, reference):
+        want = reconcile_output_layout(want, got.shape)
+        torch.testing.assert_close(got.float(), want.float().to(got.device), rtol=tolerance.rtol,
+                                   atol=tolerance.atol, equal_nan=tolerance.equal_nan)
+
+
+def _check_kernel(kernel, *, graph=None, dtype=None, reference_cache_dir=None,
+                  tolerance: Tolerance = DEFAULT_TOLERANCE, benchmark: BenchOptions | None = None):
+    """Validate against the published (or freshly built) reference, then optionally time, all
+    under one hold of the GPU lock.  Returns mean latency in ms, or None without ``benchmark``."""
+    from .reference import build_inputs_and_reference, order_inputs_for_kernel
+
+    with _gpu_exec_guard():
+        with _stage("validate"):
+            if reference_cache_dir is not None:
+                inputs_by_name, reference = _load_reference(reference_cache_dir)
+            else:
+                inputs_by_name, reference, _ = build_inputs_and_reference(graph, dtype)
+            inputs = order_inputs_for_kernel(inputs_by_name, kernel)
+            _validate_kernel_outputs(kernel, inputs, reference, tolerance=tolerance)
+        if benchmark is None:
+            return None
+        with _stage("bench"):
+            return benchmark_compiled_kernel(kernel, inputs, warmup_iters=benchmark.warmup,
+                                             profile_iters=benchmark.iters)
+
+
+def _run_and_validate_kernel(kernel, *, graph=None, dtype=None, reference_cache_dir=None,
+                             tolerance: Tolerance = DEFAULT_TOLERANCE):
+    _check_kernel(kernel, graph=graph, dtype=dtype, reference_cache_dir=reference_cache_dir, tolerance=tolerance)
+    return kernel.get_kernel_source()

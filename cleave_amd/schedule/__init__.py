@@ -1,0 +1,93 @@
+"""Tiling search and application for gfx950.
+
+``search_tiling(graph, topk, force_fusion, accept)`` and ``apply_tiling(cand)`` keep the
+reference's entry points (``python/cleave/schedule/search.py:10-33``,
+``python/cleave/schedule/tiling.py:593``); what they search and produce is specific to this
+back end (see ``policy``).
+"""
+
+from __future__ import annotations
+
+from ..core.errors import ScheduleRejected
+from ..core.target import current_target
+from . import policy
+from .hint import TileDict
+from .plan import KernelPlan, ParamSpec
+
+
+def _candidates(graph, arch):
+    low, role, factor = graph.lowered, graph.role, graph.split_factor
+    if role == "combine":
+        return policy.combine_candidates(low, factor, arch)
+    fam = low.family
+    if fam in ("matmul", "rmsnorm_matmul"):
+        cands = []
+        if policy.skinny_ok(low):
+            cands += policy.skinny_candidates(low, role, factor, arch)
+        if not (fam == "rmsnorm_matmul" and low.problem["trans_A"]):
+            cands += policy.gemm_candidates(low, role, factor, arch)
+        return cands
+    if fam == "attention":
+        if not policy.attn_ok(low):
+            raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "
+                                   f"a multiple of 128, got {low.problem['head_dim']}/{low.problem['vdim']}")
+        return policy.attn_candidates(low, role, factor, arch)
+    if fam == "mla":
+        if not policy.mla_ok(low):
+            raise ScheduleRejected("MLA template needs heads % 16 == 0 and widths that are multiples of 32")
+        return policy.mla_candidates(low, role, factor, arch)
+    raise ScheduleRejected(f"no template for family {fam!r}")
+
+
+def search_tiling(graph, topk: int = 10, force_fusion: bool = False, accept=None, arch=None):
+    """Up to ``topk`` ``TileDict`` candidates for a stage graph, best modelled cost first.
+    ``accept(cand) -> bool`` filters before the cut.  ``force_fusion`` is accepted for API
+    compatibility: every template here is already one fused kernel."""
+    arch = arch or current_target().arch
+    if not hasattr(graph, "lowered"):
+        raise ScheduleRejected("search_tiling needs a recognised stage graph (cleave_amd.lower.to_ir)")
+    cands = _candidates(graph, arch)
+    if accept is not None:
+        cands = [c for c in cands if accept(c)]
+    cands.sort(key=lambda c: (c.score, c.key()))
+    seen, unique = set(), []
+    for c in cands:
+        if c.key() not in seen:
+            seen.add(c.key())
+            c.flat_graph = graph
+            unique.append(c)
+    return unique[:max(1, int(topk))]
+
+
+def _name(node_name: str) -> str:
+    return node_name
+
+
+def apply_tiling(cand: TileDict) -> KernelPlan:
+    """The scheduled plan of one candidate: parameter list in call order plus template knobs."""
+    from ..lower.stages import partial_buffers
+
+    graph = cand.flat_graph
+    low, role = graph.lowered, graph.role
+    dtype = graph.dtype
+    params, operands = [], {}
+    if role in ("main", "partial"):
+        by_node = {id(n): r for r, n in low.operands.items()}
+        for ph in graph.placeholders:
+            params.append(ParamSpec(ph.name, ph.dtype, tuple(ph.shape), "input"))
+            operands[by_node[id(ph)]] = ph.name
+    else:
+        for ph in graph.placeholders:
+            params.append(ParamSpec(ph.name, ph.dtype, tuple(ph.shape), "input"))
+            operands[ph.name.replace("PlaceHolder_", "")] = ph.name
+    if role == "partial":
+        for out, (bname, shape, dt) in zip(graph.outputs, partial_buffers(low, cand.split_factor)):
+            params.append(ParamSpec(out.name, dt, tuple(shape), "output"))
+            operands[bname] = out.name
+    else:
+        for i, out in enumerate(graph.outputs):
+            params.append(ParamSpec(out.name, out.dtype, tuple(out.shape), "output"))
+            operands["OUT" if i == 0 else f"OUT{i}"] = out.name
+    return KernelPlan(template=cand.template, role=role, family=low.family, dtype=dtype, problem=dict(low.problem),
+                      tiling=dict(cand.tiling), params=params, operands=operands, split_factor=cand.split_factor,
+                      n_threads=cand.n_threads, lds_bytes=cand.lds_bytes, label=cand.label)

@@ -1,0 +1,246 @@
+"""Launch-plan search space for gfx950 and the model that ranks it.
+
+Stands where the reference's roller-style policy stands
+(``python/cleave/schedule/policy/default.py:23-1110``): enumerate tilings, discard the ones
+the hardware cannot hold, rank by a traffic x waves model, keep ``topk``.  Nothing of its
+CUDA-shaped space is kept (warp 32, 64x32x32 wmma base tile, 164 KB shared memory, 128/256
+threads).  The space here is written for one MI355X:
+
+* 64-lane wavefronts, four SIMDs and 512 vector registers per lane per SIMD, up to 160 KiB of
+  LDS per workgroup, 256 compute units;
+* matrix-core tiles of 16x16x32 (f16/bf16, f32 accumulate), so every tile extent is a
+  multiple of 16 and every contraction step a multiple of 32;
+* 16-byte (dwordx4) global accesses: eight elements per lane, rows walked so that sixteen
+  lanes cover 256 contiguous bytes;
+* bandwidth-bound families (few-row matmul, decode attention) stream operands HBM -> registers
+  and are tiled by *waves in flight*, not by LDS tiles; the split factor is what fills the
+  256 compute units.
+"""
+
+from __future__ import annotations
+
+import itertools
+import math
+
+from ..arch import Arch
+from .hint import TileDict
+
+ELEM_BYTES = {"float16": 2, "bfloat16": 2}
+
+
+def _ceil(a, b):
+    return -(-a // b)
+
+
+def _waves_time(blocks, per_cu, arch: Arch):
+    """Number of full passes the grid makes over the machine."""
+    return _ceil(blocks, max(1, per_cu * arch.compute_units))
+
+
+# ----------------------------------------------------------------------------- GEMM
+def gemm_lds_bytes(bm, bn, bk, norm=False):
+    return 2 * (bm + bn) * (bk + 8) * 2 + (bm * 4 if norm else 0)
+
+
+def gemm_candidates(low, role, factor, arch: Arch):
+    p = low.problem
+    splits = factor or 1
+    M, N, K = p["M"], p["N"], p["K"]
+    if K % splits:
+        return []
+    kps = K // splits
+    batch = max(p["batch_A"], p["batch_B"])
+    norm = low.family == "rmsnorm_matmul"
+    out = []
+    shapes = (16, 32, 64, 128, 256)
+    for bm, bn, bk, (wm, wn) in itertools.product(shapes, shapes, (32, 64),
+                                                  ((1, 1), (1, 2), (2, 1), (2, 2), (1, 4), (4, 1), (2, 4), (4, 2))):
+        if bm % (16 * wm) or bn % (16 * wn) or kps % bk:
+            continue
+        if bm > max(16, 2 * M) or bn > max(16, 2 * N):
+            continue
+        threads = wm * wn * 64
+        tm, tn = bm // wm // 16, bn // wn // 16
+        acc_regs = tm * tn * 4
+        if acc_regs > 256:
+            continue
+        # loader granularity: K-minor tiles move 16-byte chunks, K-major ones 8x8 blocks
+        a_units = bm * (bk // 8) if not p["trans_A"] else (bm // 8) * (bk // 8)
+        b_units = bn * (bk // 8) if p["trans_B"] else (bn // 8) * (bk // 8)
+        if p["trans_A"] and (bm % 8 or M % 8):
+            continue
+        if not p["trans_B"] and (bn % 8 or N % 8):
+            continue
+        stage_regs = _ceil(a_units, threads) * (32 if p["trans_A"] else 4) \
+            + _ceil(b_units, threads) * (4 if p["trans_B"] else 32)
+        vgprs = acc_regs + stage_regs + (tm + tn) * 4 + 40
+        if vgprs > arch.vgprs_per_lane:
+            continue
+        lds = gemm_lds_bytes(bm, bn, bk, norm)
+        if lds > arch.lds_bytes:
+            continue
+        blocks = _ceil(M, bm) * _ceil(N, bn) * batch * splits
+        per_cu = arch.blocks_per_cu(threads, lds, vgprs)
+        if per_cu < 1:
+            continue
+        passes = _waves_time(blocks, per_cu, arch)
+        # per-block cost: matrix-core cycles vs bytes pulled through L2, whichever is longer
+        mfma_clk = (bm * bn * kps * 2) / (1024.0 * min(4, wm * wn))
+        l2_clk = ((bm + bn) * kps * 2) / 48.0
+        lds_clk = (tm * 16 * wm * wn + tn * 16 * wm * wn) * kps * 2 / 128.0 * 0.5
+        block_clk = max(mfma_clk, l2_clk, lds_clk) + 2000
+        util = min(1.0, blocks / (per_cu * arch.compute_units)) if passes == 1 else 1.0
+        score = passes * block_clk * (1.0 + 0.15 * (1 - util))
+        tiling = dict(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn)
+        out.append(TileDict("gemm", role, tiling, output_tile=[bm, bn], rstep_map={"k": bk}, n_threads=threads,
+                            split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+    return out
+
+
+# ----------------------------------------------------------------------------- few-row matmul
+def skinny_ok(low) -> bool:
+    p = low.problem
+    return (p["M"] <= 64 and not p["trans_A"] and not p["trans_B"] and p["batch_A"] == 1 and p["batch_B"] == 1
+            and p["K"] % 32 == 0 and p["N"] % 8 == 0 and p["N"] >= 8)
+
+
+def skinny_lds_bytes(mt, waves_n, waves_k):
+    return ((waves_k - 1) * waves_n * mt * 32 * 64 + waves_k * mt * 16) * 4 + 16
+
+
+def skinny_candidates(low, role, factor, arch: Arch):
+    p = low.problem
+    splits = factor or 1
+    M, N, K = p["M"], p["N"], p["K"]
+    mt = _ceil(M, 16)
+    steps = K // 32
+    if steps % splits:
+        return []
+    out = []
+    for waves_n, waves_k in itertools.product((1, 2, 4), (1, 2, 4, 8)):
+        threads = waves_n * waves_k * 64
+        if threads > 1024:
+            continue
+        per_split = steps // splits
+        if per_split < waves_k:
+            continue
+        lds = skinny_lds_bytes(mt, waves_n, waves_k)
+        if lds > arch.lds_bytes:
+            continue
+        vgprs = mt * 32 + 3 * 32 + 32 + mt * 4 + 40
+        blocks = _ceil(N, 128 * waves_n) * splits
+        per_cu = arch.blocks_per_cu(threads, max(lds, 1), vgprs)
+        if per_cu < 1:
+            continue
+        passes = _waves_time(blocks, per_cu, arch)
+        waves_live = min(blocks, per_cu * arch.compute_units) * waves_n * waves_k
+        # a wave keeps ~3 steps of 8 KiB in flight; HBM wants ~16 MiB outstanding machine-wide
+        inflight = waves_live * 24 * 1024
+        bw_frac = min(1.0, inflight / (12 * 1024 * 1024))
+        stream_us = (K * N * 2) / (arch.hbm_gbps * 1e3 * bw_frac)
+        partial_us = (2 * splits * M * N * 4) / (arch.hbm_gbps * 1e3) if splits > 1 else 0.0
+        tail = 1.0 + 0.25 * (passes - 1) + 0.02 * waves_k
+        score = (stream_us * tail + partial_us) * 2400
+        tiling = dict(WAVES_N=waves_n, WAVES_K=waves_k)
+        out.append(TileDict("skinny", role, tiling, output_tile=[M, 128 * waves_n], rstep_map={"k": 32},
+                            n_threads=threads, split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+    return out
+
+
+# ----------------------------------------------------------------------------- decode attention
+def attn_lds_bytes(waves, vdim):
+    return waves * (32 + 16 * vdim) * 4
+
+
+def attn_ok(low) -> bool:
+    p = low.problem
+    return p["head_dim"] % 32 == 0 and (p["vdim"] % 128 == 0 or p["vdim"] == 64)
+
+
+def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
+    p = low.problem
+    splits = factor or 1
+    rows = p["group"] * p["sq"]
+    row_tiles = _ceil(rows, 16)
+    d, vd = p["head_dim"], p["vdim"]
+    steps = _ceil(p["skv"], 32)
+    out = []
+    for waves in waves_options:
+        lds = attn_lds_bytes(waves, vd)
+        if lds > arch.lds_bytes:
+            continue
+        kv_regs = (2 * (d // 32) + 8 * _ceil(vd, 128)) * 4
+        vgprs = 2 * kv_regs + 32 * _ceil(vd, 128) + 4 * (d // 32) + 32 + 48
+        if vgprs > arch.vgprs_per_lane:
+            continue
+        blocks = p["units"] * row_tiles * splits
+        per_cu = arch.blocks_per_cu(waves * 64, lds, vgprs)
+        if per_cu < 1:
+            continue
+        passes = _waves_time(blocks, per_cu, arch)
+        steps_per_wave = _ceil(_ceil(steps, splits), waves)
+        waves_live = min(blocks, per_cu * arch.compute_units) * min(waves, _ceil(steps, splits))
+        inflight = waves_live * 2 * kv_regs * 64 * 4 / 2
+        bw_frac = min(1.0, inflight / (12 * 1024 * 1024))
+        bytes_total = p["units"] * row_tiles * p["skv"] * (d + vd) * 2
+        stream_us = bytes_total / (arch.hbm_gbps * 1e3 * bw_frac)
+        ramp_us = 1.5 + 0.02 * steps_per_wave * 0  # fixed launch + drain cost
+        partial_us = (2 * splits * p["units"] * rows * (vd + 2) * 4) / (arch.hbm_gbps * 1e3) if splits > 1 else 0.0
+        score = (stream_us * (1.0 + 0.2 * (passes - 1)) + ramp_us + partial_us + 0.05 * waves) * 2400
+        tiling = dict(WAVES=waves)
+        out.append(TileDict("attn_decode", role, tiling, output_tile=[16, vd], rstep_map={"kv": 32},
+                            n_threads=waves * 64, split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+    return out
+
+
+# ----------------------------------------------------------------------------- MLA decode
+def mla_lds_bytes(ckv, kpe):
+    return 2 * (32 * (ckv + kpe + 8) + ckv * (32 + 8)) * 2
+
+
+def mla_ok(low) -> bool:
+    p = low.problem
+    return p["heads"] % 16 == 0 and p["ckv"] % 32 == 0 and p["kpe"] % 32 == 0 and p["ckv"] % 16 == 0
+
+
+def mla_candidates(low, role, factor, arch: Arch):
+    p = low.problem
+    splits = factor or 1
+    lds = mla_lds_bytes(p["ckv"], p["kpe"])
+    if lds > arch.lds_bytes:
+        return []
+    out = []
+    groups16 = p["heads"] // 16
+    for waves in (1, 2, 4, 8):
+        if groups16 % waves:
+            continue
+        vgprs = (p["ckv"] + p["kpe"]) // 32 * 4 + p["ckv"] // 16 * 4 + 40 + 48
+        if vgprs > arch.vgprs_per_lane:
+            continue
+        blocks = p["batch"] * (groups16 // waves) * splits
+        per_cu = arch.blocks_per_cu(waves * 64, lds, vgprs)
+        if per_cu < 1:
+            continue
+        passes = _waves_time(blocks, per_cu, arch)
+        steps = _ceil(_ceil(p["skv"], 32), splits)
+        # per step and wave: 2*(D/32) + ckv/16 matrix-core issues of 16 clocks; LDS operand reads
+        # of every wave share one 128 B/clk port
+        mfma_clk = (2 * (p["ckv"] + p["kpe"]) // 32 + p["ckv"] // 16) * 16 * _ceil(waves, 4)
+        lds_clk = waves * (32 * (p["ckv"] + p["kpe"]) + 32 * p["ckv"]) * 2 / 128.0
+        load_clk = 32 * (p["ckv"] + p["kpe"]) * 2 / 24.0
+        step_clk = max(mfma_clk, lds_clk, load_clk) + 200
+        util = min(1.0, blocks / (per_cu * arch.compute_units))
+        score = passes * steps * step_clk * (1.0 + 0.3 * (1 - util)) + 3000
+        out.append(TileDict("mla_decode", role, dict(WAVES=waves), output_tile=[16 * waves, p["ckv"]],
+                            rstep_map={"kv": 32}, n_threads=waves * 64, split_factor=factor, score=score,
+                            lds_bytes=lds, est_vgprs=vgprs))
+    return out
+
+
+# ----------------------------------------------------------------------------- combine kernels
+def combine_candidates(low, factor, arch: Arch):
+    """The combine of a split has one shape: one thread per 4 (attention) or 4/8 (matmul)
+    output columns, 256 threads; it is memory-trivial next to its partial."""
+    family = {"matmul": "gemm", "rmsnorm_matmul": "gemm", "attention": "attn_decode", "mla": "mla_decode"}[low.family]
+    return [TileDict(family, "combine", {}, output_tile=[1, 256], rstep_map={"split": factor}, n_threads=256,
+                     split_factor=factor, score=1.0, lds_bytes=0, est_vgprs=32)]

@@ -1,0 +1,127 @@
+"""The five graded operators as ``@jit`` programs, with their seeded inputs.
+
+Shapes at ``FULL`` are the benchmark configurations; ``SMALL`` are the same programs at sizes
+the numpy oracle finishes in well under a second.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+import cleave_amd
+import cleave_amd.lang as cl
+
+
+@cleave_amd.jit
+def matmul(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
+    return x @ w
+
+
+@cleave_amd.jit
+def rmsnorm_matmul(x: cl.Tensor["M", "K"], gamma: cl.Tensor[1, "K"], w: cl.Tensor["K", "N"]):
+    return (cl.rms_norm(x, dim=-1, eps=1e-6) * gamma) @ w
+
+
+@cleave_amd.jit
+def rmsnorm_matmul_plain(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
+    return cl.rms_norm(x, dim=-1) @ w
+
+
+@cleave_amd.jit
+def gqa_decode_exact(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
+    return cl.softmax((q @ k.mT) / q.shape[-1] ** 0.5, dim=-1) @ v
+
+
+@cleave_amd.jit
+def gqa_decode_shift(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
+    n = q.shape[-1] ** 0.5
+    return cl.softmax((q @ k.mT) / n, dim=-1, shift=-50 / n) @ v
+
+
+@cleave_amd.jit
+def mla_decode(q: cl.Tensor["B", "H", "D"], kv: cl.Tensor["B", "SKV", "D"], q_pe: cl.Tensor["B", "H", "PE"],
+               k_pe: cl.Tensor["B", "SKV", "PE"]):
+    s = (q @ kv.mT + q_pe @ k_pe.mT) * (192 ** -0.5)
+    return cl.softmax(s, dim=-1) @ kv
+
+
+FULL = {
+    "c1": dict(M=128, N=128, K=4096),
+    "c2": dict(M=16, K=4096, N=11008),
+    "c3": dict(HQ=256, HKV=64, SQ=1, SKV=8192, D=128),
+    "c4": dict(B=16, H=128, D=512, PE=64, SKV=4096),
+}
+SMALL = {
+    "c1": dict(M=32, N=64, K=256),
+    "c2": dict(M=16, K=256, N=384),
+    "c3": dict(HQ=8, HKV=2, SQ=1, SKV=200, D=128),
+    "c4": dict(B=2, H=16, D=512, PE=64, SKV=100),
+}
+
+
+def _gen(seed):
+    return torch.Generator(device="cpu").manual_seed(seed)
+
+
+def inputs_c1(shapes, seed=1, device="cpu"):
+    g = _gen(seed)
+    M, N, K = shapes["M"], shapes["N"], shapes["K"]
+    x = (torch.rand(M, K, generator=g) * 2 - 1) / math.sqrt(K)
+    w = (torch.rand(K, N, generator=g) * 2 - 1) / math.sqrt(K)
+    return [x.to(torch.float16).to(device), w.to(torch.float16).to(device)]
+
+
+def inputs_c2(shapes, seed=2, device="cpu"):
+    g = _gen(seed)
+    M, N, K = shapes["M"], shapes["N"], shapes["K"]
+    x = torch.randn(M, K, generator=g)
+    gamma = 1 + 0.1 * torch.randn(1, K, generator=g)
+    w = torch.randn(K, N, generator=g) / math.sqrt(K)
+    return [t.to(torch.float16).to(device) for t in (x, gamma, w)]
+
+
+def inputs_c3(shapes, seed=3, device="cpu"):
+    g = _gen(seed)
+    s = shapes
+    q = torch.randn(s["HQ"], s["SQ"], s["D"], generator=g)
+    k = torch.randn(s["HKV"], s["SKV"], s["D"], generator=g)
+    v = torch.randn(s["HKV"], s["SKV"], s["D"], generator=g)
+    return [t.to(torch.float16).to(device) for t in (q, k, v)]
+
+
+def inputs_c4(shapes, seed=4, device="cpu"):
+    g = _gen(seed)
+    s = shapes
+    q = 0.5 * torch.randn(s["B"], s["H"], s["D"], generator=g)
+    kv = 0.5 * torch.randn(s["B"], s["SKV"], s["D"], generator=g)
+    q_pe = 0.5 * torch.randn(s["B"], s["H"], s["PE"], generator=g)
+    k_pe = 0.5 * torch.randn(s["B"], s["SKV"], s["PE"], generator=g)
+    return [t.to(torch.bfloat16).to(device) for t in (q, kv, q_pe, k_pe)]
+
+
+CASES = {
+    "c1": (matmul, cl.f16, inputs_c1),
+    "c2": (rmsnorm_matmul, cl.f16, inputs_c2),
+    "c3": (gqa_decode_exact, cl.f16, inputs_c3),
+    "c4": (mla_decode, cl.bf16, inputs_c4),
+}
+
+
+def paged_workload(lens, page_size=64, num_pages=None, hq=32, hkv=8, d=128, seed=5, dtype=torch.float16,
+                   device="cpu", pool_scale=1.0):
+    """C5-style paged decode arguments: q, k_cache, v_cache, kv_indptr, kv_indices,
+    kv_last_page_len, sm_scale.  The block table is a seeded random permutation of the pool."""
+    g = _gen(seed)
+    pages = [-(-n // page_size) for n in lens]
+    total = sum(pages)
+    num_pages = num_pages or max(total, 1)
+    kv_indices = torch.randperm(num_pages, generator=g)[:total].to(torch.int32)
+    indptr = torch.tensor([0] + list(torch.tensor(pages).cumsum(0).tolist()), dtype=torch.int32)
+    last = torch.tensor([n - (p - 1) * page_size if p else 0 for n, p in zip(lens, pages)], dtype=torch.int32)
+    q = torch.randn(len(lens), hq, d, generator=g).to(dtype)
+    k_cache = (torch.randn(num_pages, page_size, hkv, d, generator=g) * pool_scale).to(dtype)
+    v_cache = (torch.randn(num_pages, page_size, hkv, d, generator=g) * pool_scale).to(dtype)
+    args = [q, k_cache, v_cache, indptr, kv_indices, last]
+    return [a.to(device) for a in args] + [float(d) ** -0.5]

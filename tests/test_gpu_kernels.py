@@ -1,0 +1,115 @@
+"""GPU parity: every template against the numpy oracle on the same seeded inputs.
+
+Tolerance: rtol 1e-2 / atol 1e-2 against the fp32-accumulated oracle for f16/bf16 outputs.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import program_oracle as po
+from tests import _cases as C
+from tests._lowlevel import kernel_for
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def _check(program, make_inputs, shapes, **kw):
+    ins = make_inputs(shapes, device="cpu")
+    want = po.evaluate(program, ins)[0]
+    kernel = kernel_for(program, **kw)
+    print(f"case {program.name} {shapes} {kw}", flush=True)
+    got = kernel(*[t.cuda() for t in ins])
+    torch.cuda.synchronize()
+    got = got.float().cpu().numpy().reshape(want.shape)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+GEMM_TILES = [dict(BM=32, BN=32, BK=32, WM=1, WN=1), dict(BM=64, BN=64, BK=64, WM=2, WN=2),
+              dict(BM=128, BN=128, BK=32, WM=2, WN=2)]
+
+
+@pytest.mark.parametrize("tiling", GEMM_TILES, ids=lambda t: "x".join(str(v) for v in t.values()))
+@pytest.mark.parametrize("split", [None, 4])
+def test_matmul_gemm_small(tiling, split):
+    fn, dt, mk = C.CASES["c1"]
+    shapes = dict(M=96, N=136, K=512)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=tiling, split=split)
+
+
+@pytest.mark.parametrize("split", [None, 4, 8, 16])
+def test_matmul_c1_full(split):
+    fn, dt, mk = C.CASES["c1"]
+    _check(fn.trace(dt, **C.FULL["c1"]), mk, C.FULL["c1"], template="gemm",
+           tiling=dict(BM=64, BN=64, BK=64, WM=2, WN=2), split=split)
+
+
+@pytest.mark.parametrize("tiling", [dict(WAVES_N=1, WAVES_K=1), dict(WAVES_N=2, WAVES_K=2), dict(WAVES_N=1, WAVES_K=4)],
+                         ids=lambda t: "x".join(str(v) for v in t.values()))
+@pytest.mark.parametrize("split", [None, 2])
+def test_rmsnorm_matmul_skinny_small(tiling, split):
+    fn, dt, mk = C.CASES["c2"]
+    shapes = dict(M=16, K=512, N=392)     # N not a multiple of 128: the last slab is masked
+    _check(fn.trace(dt, **shapes), mk, shapes, template="skinny", tiling=tiling, split=split)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 33])
+def test_skinny_row_counts(m):
+    fn, dt, mk = C.CASES["c2"]
+    shapes = dict(M=m, K=256, N=256)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="skinny", tiling=dict(WAVES_N=1, WAVES_K=2))
+
+
+@pytest.mark.parametrize("split", [None, 4, 8, 16])
+def test_rmsnorm_matmul_c2_full(split):
+    fn, dt, mk = C.CASES["c2"]
+    _check(fn.trace(dt, **C.FULL["c2"]), mk, C.FULL["c2"], template="skinny",
+           tiling=dict(WAVES_N=1, WAVES_K=4), split=split)
+
+
+def test_rmsnorm_matmul_gemm_path():
+    fn, dt, mk = C.CASES["c2"]
+    shapes = dict(M=128, K=512, N=256)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=32, WM=2, WN=2))
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=32, WM=2, WN=2), split=4)
+
+
+@pytest.mark.parametrize("waves", [1, 2, 4])
+@pytest.mark.parametrize("split", [None, 2, 8])
+def test_gqa_decode_small(waves, split):
+    fn, dt, mk = C.CASES["c3"]
+    shapes = dict(HQ=8, HKV=2, SQ=1, SKV=416, D=128)   # 13 steps: ragged over waves and splits
+    _check(fn.trace(dt, **shapes), mk, shapes, template="attn_decode", tiling=dict(WAVES=waves), split=split)
+
+
+def test_gqa_decode_ragged_tail_and_shift_program():
+    shapes = dict(HQ=8, HKV=2, SQ=1, SKV=200, D=128)   # 200 = 6 steps + 8 tokens
+    _check(C.gqa_decode_shift.trace(C.cl.f16, **shapes), C.inputs_c3, shapes, template="attn_decode",
+           tiling=dict(WAVES=2), split=None)
+
+
+def test_gqa_decode_many_rows():
+    shapes = dict(HQ=12, HKV=2, SQ=5, SKV=160, D=128)  # 30 rows per kv head: two row tiles
+    _check(C.gqa_decode_exact.trace(C.cl.f16, **shapes), C.inputs_c3, shapes, template="attn_decode",
+           tiling=dict(WAVES=2), split=2)
+
+
+@pytest.mark.parametrize("split", [8, 16, 32])
+def test_gqa_decode_c3_full(split):
+    fn, dt, mk = C.CASES["c3"]
+    _check(fn.trace(dt, **C.FULL["c3"]), mk, C.FULL["c3"], template="attn_decode", tiling=dict(WAVES=4), split=split)
+
+
+@pytest.mark.parametrize("split", [None, 2])
+def test_mla_decode_small(split):
+    fn, dt, mk = C.CASES["c4"]
+    _check(fn.trace(dt, **C.SMALL["c4"]), mk, C.SMALL["c4"], template="mla_decode", tiling=dict(WAVES=1), split=split)
+    shapes = dict(B=2, H=64, D=512, PE=64, SKV=160)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=4), split=split)
+
+
+@pytest.mark.parametrize("split", [4, 8])
+def test_mla_decode_c4_full(split):
+    fn, dt, mk = C.CASES["c4"]
+    _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=dict(WAVES=4), split=split)
