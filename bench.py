@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the compile path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops c1,c2,c3,c4,c5,mm] [--no-cpu]
+
+For every operator the staged pipeline searches candidates (``cleave_amd.compile``, preset
+fast): each candidate is compiled with hiprtc, validated against the torch evaluation of the
+traced program at rtol = atol = 1e-2 and timed; the best variant is then re-timed here for
+exactly K steps, one step being one launch of the winning kernel (a split variant is its fused
+partial + combine pair) on one set of seeded synthetic inputs already resident in HBM.  Steps
+rotate through several independent input sets so a working set smaller than the 256 MB
+last-level cache cannot be served from it.
+
+One JSON line is printed.  ``value`` is the best-candidate latency in microseconds of the
+headline workload (fused RMSNorm->matmul at the decode shape M=16, K=4096, N=11008, fp16);
+``ops`` carries the same figures for every other operator.  ``roofline`` prices the dominant
+kernel of the headline workload: algorithmic bytes per launch over its mean duration from
+HIP events on the launch stream, against the published 8 TB/s.  ``cpu_baseline`` is the numpy
+port of the reference's CPU evaluation of the same program, timed on this host.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+HBM_GBPS = 8000.0
+MFMA_TFLOPS = 2516.6
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+# ----------------------------------------------------------------------------- operator table
+def op_table():
+    import cleave_amd.lang as cl
+    from tests import _cases as C
+
+    return {
+        "c1": dict(title="matmul f16 128x128x4096", fn=C.matmul, dtype=cl.f16, shapes=C.FULL["c1"], inputs=C.inputs_c1,
+                   split=cl.Split("K", (4, 8, 16)), bytes=2_129_920, flops=134_217_728, bound="hbm", sets=4),
+        "c2": dict(title="rmsnorm(x)*gamma @ w f16 M=16 K=4096 N=11008", fn=C.rmsnorm_matmul, dtype=cl.f16,
+                   shapes=C.FULL["c2"], inputs=C.inputs_c2, split=cl.Split("K", (2, 4, 8, 16)), bytes=90_669_056,
+                   flops=1_442_840_576, bound="hbm", sets=6),
+        "c3": dict(title="GQA decode f16 B=8 Hq=32 Hkv=8 D=128 SKV=8192 exact softmax", fn=C.gqa_decode_exact,
+                   dtype=cl.f16, shapes=C.FULL["c3"], inputs=C.inputs_c3, split=cl.Split("SKV", (8, 16, 32)),
+                   bytes=268_566_528, flops=1_073_741_824, bound="hbm", sets=3),
+        "c4": dict(title="MLA decode bf16 B=16 H=128 512+64 SKV=4096", fn=C.mla_decode, dtype=cl.bf16,
+                   shapes=C.FULL["c4"], inputs=C.inputs_c4, split=cl.Split("SKV", (2, 4, 8, 16)), bytes=79_953_920,
+                   flops=18_253_611_008, bound="hbm", sets=6),
+        "mm": dict(title="matmul f16 4096x14336x4096", fn=C.matmul, dtype=cl.f16, shapes=dict(M=4096, N=14336, K=4096),
+                   inputs=C.inputs_c1, split=False, bytes=2 * (4096 * 4096 + 4096 * 14336 + 4096 * 14336),
+                   flops=2 * 4096 * 14336 * 4096, bound="mfma", sets=2),
+    }
+
+
+def roofline(bound, nbytes, flops, us, traffic=None):
+    if bound == "mfma":
+        achieved = flops / us / 1e6
+        return {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / MFMA_TFLOPS, 4), "traffic": traffic}
+    achieved = nbytes / us / 1e3
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_GBPS, 4), "traffic": traffic}
+
+
+# ----------------------------------------------------------------------------- dense operators
+def fused_kernel(kernel):
+    """The winning variant as one compiled object: its single stage, or partial + combine fused."""
+    from cleave_amd.codegen import HipCodeGen
+    from cleave_amd.runtime.compile import _compile, _load_main_kernel_from_code
+    from cleave_amd.schedule import apply_tiling
+
+    if len(kernel.stages) == 1:
+        src = kernel.stages[0].source
+    else:
+        src = HipCodeGen().gen([apply_tiling(p.tile) for p in kernel.plans])
+    loaded = _load_main_kernel_from_code(src)
+    return _compile(loaded, loaded.manifest["out_idx"])
+
+
+def run_dense(name, op, steps, warmup, search_iters):
+    import torch
+
+    import cleave_amd
+    from cleave_amd import pipeline as P
+
+    t0 = time.perf_counter()
+    program = op["fn"].trace(op["dtype"], **op["shapes"])
+    kernel = cleave_amd.compile(program, preset="fast", split=op["split"], cache_kernels=False,
+                                schedule=P.ScheduleConfig(topk=12, split_k=getattr(op["split"], "factors", ())),
+                                eval=P.EvalConfig(warmup=3, iters=search_iters, max_parallel=0))
+    report = kernel.report
+    log(f"[{name}] search {time.perf_counter() - t0:.1f}s: {len(report)} candidates, {len(report.correct)} valid; "
+        f"best {kernel.variant} {kernel.label}")
+    fused = fused_kernel(kernel)
+    sets = [[t.cuda() for t in op["inputs"](op["shapes"], seed=100 + i)] for i in range(op["sets"])]
+    ms = fused.time(*sets[0], warmup=warmup, iters=steps, rotate=sets[1:])
+    us = ms * 1e3
+    dom_us = fused.time(*sets[0], warmup=warmup, iters=steps, rotate=sets[1:], only=[0]) * 1e3
+    torch.cuda.synchronize()
+    out = {"op": name, "workload": op["title"], "best_us": round(us, 3), "dominant_kernel_us": round(dom_us, 3),
+           "variant": kernel.variant, "plan": kernel.label, "candidates": len(report), "validated": len(report.correct),
+           "hbm": roofline("hbm", op["bytes"], op["flops"], us), "mfma": roofline("mfma", op["bytes"], op["flops"], us)}
+    out["roofline"] = roofline(op["bound"], op["bytes"], op["flops"], dom_us)
+    return out, program
+
+
+def cpu_dense(program, op, budget_s=12.0):
+    import numpy as np  # noqa: F401
+
+    from oracle import program_oracle
+
+    ins = op["inputs"](op["shapes"], seed=100)
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_all < budget_s and len(times) < 20):
+        t0 = time.perf_counter()
+        program_oracle.evaluate(program, ins)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_all > 3 * budget_s:
+            break
+    return statistics.median(times) * 1e6, len(times)
+
+
+# ----------------------------------------------------------------------------- paged decode (C5)
+def run_paged(steps, warmup, with_cpu):
+    import torch
+
+    from cleave_amd.codegen import HipCodeGen
+    from cleave_amd.dynamic import reference as dref
+    from cleave_amd.dynamic.paging import (PAGED_DECODE_SLAB, CombineTiling, DenseAttention, PagingSpec,
+                                           build_split_decode)
+    from cleave_amd.runtime.compile import _compile, _load_main_kernel_from_code
+
+    page, hq, hkv, d, pool = 64, 32, 8, 128, 300_000
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    lens = torch.randint(256, 16384 + 1, (32,), generator=gen).tolist()
+    pages = [-(-n // page) for n in lens]
+    total_pages = sum(pages)
+    dims = (32, hq, hkv, d, pool, total_pages)
+    t0 = time.perf_counter()
+    args = dref.gqa_paged_decode_inputs(dims, lens, page_size=page, dtype=torch.float16, device="cuda", seed=5)
+    torch.cuda.synchronize()
+    log(f"[c5] pools built in {time.perf_counter() - t0:.1f}s: {sum(lens)} tokens, {total_pages} pages")
+    want = dref.gqa_paged_decode_reference(dims, lens, page_size=page, dtype=torch.float16)(*args)
+    spec = PagingSpec(num_qo_heads=hq, num_kv_heads=hkv, kind=PAGED_DECODE_SLAB, page_size=page)
+    best = None
+    tried = valid = 0
+    for waves in (1, 2, 4):
+        for split in (4, 8, 16):
+            dense = DenseAttention(16, 32, d, waves * 64, "float16", "float16", waves=waves)
+            src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split)))
+            loaded = _load_main_kernel_from_code(src)
+            k = _compile(loaded, loaded.manifest["out_idx"])
+            tried += 1
+            out, lse = k(*args)
+            torch.cuda.synchronize()
+            try:
+                torch.testing.assert_close(out.float(), want[0].float(), rtol=1e-2, atol=1e-2)
+                torch.testing.assert_close(lse, want[1], rtol=1e-2, atol=1e-2)
+            except AssertionError as e:
+                log(f"[c5] waves={waves} split={split} INVALID: {str(e).splitlines()[0]}")
+                continue
+            valid += 1
+            us = k.time(*args, warmup=2, iters=10) * 1e3
+            log(f"[c5] waves={waves} split={split}: {us:.1f} us")
+            if best is None or us < best[0]:
+                best = (us, waves, split, k)
+    _, waves, split, k = best
+    us = k.time(*args, warmup=warmup, iters=steps) * 1e3
+    dom = k.time(*args, warmup=warmup, iters=steps, only=[0]) * 1e3
+    nbytes = sum(lens) * hkv * d * 2 * 2 + total_pages * 4 + 2 * 32 * hq * d * 2 + 32 * hq * 4 + 33 * 4 + 32 * 4
+    flops = 4 * sum(lens) * hq * d
+    res = {"op": "c5", "workload": f"paged GQA decode f16, 32 requests ({sum(lens)} tokens), page 64, 300k-page pool",
+           "best_us": round(us, 3), "dominant_kernel_us": round(dom, 3), "variant": f"split-kv={split}",
+           "plan": f"waves={waves}", "candidates": tried, "validated": valid,
+           "hbm": roofline("hbm", nbytes, flops, us), "mfma": roofline("mfma", nbytes, flops, us),
+           "roofline": roofline("hbm", nbytes, flops, dom), "algorithmic_bytes": nbytes}
+    if with_cpu:
+        from oracle import paged_oracle
+
+        # bounded sample: the two shortest requests, their pages compacted into a small pool
+        order = sorted(range(32), key=lambda i: lens[i])[:2]
+        q, kc, vc, indptr, indices = args[:5]
+        ptr = indptr.tolist()
+        sample_pages = torch.cat([indices[ptr[b]:ptr[b + 1]] for b in order]).long()
+        kc_s, vc_s = kc[sample_pages].cpu(), vc[sample_pages].cpu()
+        new_ptr, acc = [0], 0
+        for b in order:
+            acc += ptr[b + 1] - ptr[b]
+            new_ptr.append(acc)
+        t0 = time.perf_counter()
+        paged_oracle.decode(q[order].cpu(), kc_s, vc_s, new_ptr, list(range(acc)), [lens[b] for b in order], page,
+                            args[-1])
+        dt = time.perf_counter() - t0
+        tokens = sum(lens[b] for b in order)
+        res["cpu_us"] = round(dt * 1e6 * sum(lens) / tokens, 1)
+        res["cpu_sample"] = f"2 shortest requests ({tokens} of {sum(lens)} tokens), scaled by token count"
+    del args, want
+    torch.cuda.empty_cache()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--search-iters", type=int, default=30)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU form (its units are independent per "
+                 "request and kv head); run with --gpus 1")
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    torch.zeros(1, device="cuda")
+    ops = op_table()
+    wanted = [o.strip() for o in args.ops.split(",") if o.strip()]
+    if "c2" not in wanted:
+        wanted.insert(0, "c2")
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    results = {}
+    for name in wanted:
+        if name == "c5":
+            results[name] = run_paged(max(10, args.steps // 4), max(2, args.warmup // 4), not args.no_cpu)
+            continue
+        steps = args.steps if name != "mm" else max(10, args.steps // 10)
+        res, program = run_dense(name, ops[name], steps, args.warmup, args.search_iters)
+        if not args.no_cpu:
+            cpu_us, runs = cpu_dense(program, ops[name], budget_s=8.0 if name != "c4" else 15.0)
+            res["cpu_us"] = round(cpu_us, 1)
+            res["cpu_sample"] = f"full workload, median of {runs} runs"
+        results[name] = res
+        log(f"[{name}] {res['best_us']} us  hbm {res['hbm']['frac']:.3f}  mfma {res['mfma']['frac']:.3f}")
+    head = results["c2"]
+    line = {
+        "metric": "best-candidate us and % HBM/MFMA roofline per op on 1 MI355X vs CPU ref",
+        "value": head["best_us"], "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["best_us"] / 1e3, 6), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": head["workload"], "variant": head["variant"], "plan": head["plan"]},
+        "roofline": head["roofline"],
+        "cpu_baseline": None if args.no_cpu else {
+            "value": head.get("cpu_us"), "unit": "us", "cores": min(threads, cores), "kind": "port",
+            "sample": head.get("cpu_sample")},
+        "ops": [results[n] for n in wanted],
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,72 @@
+"""Shipped dynamic operators: the spec that names each one's inputs and the tiling it is
+built at (``python/cleave/dynamic/registry.py:37-231``).  Of the reference's nine operators
+the paged GQA decode family is built here; the others are recognised by the frontend and
+refused by the access layer until their templates exist."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from ..runtime.validate import Tolerance
+from . import workloads as _wl
+from .paging import PAGED_DECODE_SLAB, PagingSpec
+
+# Paged kernels reproduce their references far more tightly than the loose default bound;
+# equal_nan stays off: an empty request is defined as 0 / -inf, so a NaN is a defect.
+GATHER_TOLERANCE = Tolerance(rtol=0.01, atol=0.01, equal_nan=False)
+
+
+@dataclass(frozen=True)
+class DynamicOperator:
+    name: str
+    spec: PagingSpec
+    tuned_tiling: dict
+    dims: tuple            # (qo_heads, kv_heads, head_dim)
+    workloads: tuple
+    tolerance: Tolerance = GATHER_TOLERANCE
+    page_size: int = 1
+    scale: float | None = None
+
+    @property
+    def is_mla(self) -> bool:
+        return False
+
+    def matches(self, attention) -> bool:
+        a = attention
+        return (not a.is_mla and (a.num_qo_heads, a.num_kv_heads, a.head_dim) == tuple(self.dims[:3])
+                and a.page_size == self.page_size and a.kind == self.spec.kind)
+
+    def keyed_workloads(self, *, keep: int = 0, dtype=None):
+        from ..runtime.autotune import sampled, workload_key
+
+        chosen = sampled(list(self.workloads), keep)
+
+        def generate():
+            for axes in chosen:
+                inputs, expected = _wl.case(self.name, axes, self.dims, self.page_size, self.scale, dtype=dtype)
+                yield workload_key(axes), inputs, expected
+
+        return generate
+
+    def kernel_source(self) -> str:
+        """HIP source of this operator at its tuned tiling (single kernel)."""
+        from ..codegen import HipCodeGen
+        from .paging import DenseAttention
+        from .paging.apply import _paged_outputs, _paged_params, _plan
+
+        t = self.tuned_tiling
+        dense = DenseAttention(t["query_rows"], t["kv_tile"], t["head_dim"], t["waves"] * 64, "bfloat16", "bfloat16",
+                               waves=t["waves"])
+        params, ops = _paged_params(self.spec, dense)
+        outs, out_ops = _paged_outputs(self.spec, dense)
+        return HipCodeGen().gen(_plan(self.spec, dense, "main", params + outs, {**ops, **out_ops}))
+
+
+OPERATORS = {op.name: op for op in (
+    DynamicOperator(
+        "gqa_paged_decode_h32_kv8_d128_ps64",
+        PagingSpec(num_qo_heads=32, num_kv_heads=8, kind=PAGED_DECODE_SLAB, page_size=64, grid_order=("head", "batch"),
+                   pass_configs={}),
+        dict(query_rows=16, kv_tile=32, head_dim=128, waves=4), (32, 8, 128),
+        _wl.WORKLOADS["gqa_paged_decode_h32_kv8_d128_ps64"], page_size=64),
+)}

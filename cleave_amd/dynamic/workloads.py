@@ -1,0 +1,53 @@
+"""Workload axes of the shipped paged operators and the request lengths derived from them.
+
+The reference ships axes captured from SOL-ExecBench runs as ``wl_<batch>_<num_pages>_<n_idx>``
+(``python/cleave/dynamic/workloads.py:15-326``) and synthesises per-request lengths from them
+deterministically (``:329-361``).  The four axes of each operator below are the ones its
+checked-in H100 baseline names (``tests/perf/baselines/h100-80gb-hbm3.json``); length
+synthesis follows the same scheme: ``n_idx`` split into ``batch`` positive page counts by a
+generator seeded with ``crc32(repr((operator, axes)))``, every page full but the last.
+"""
+
+from __future__ import annotations
+
+import random
+import zlib
+
+WORKLOADS = {
+    "gqa_paged_decode_h32_kv8_d128_ps64": ((4, 349, 212), (16, 1686, 1033), (32, 15178, 14103), (128, 52033, 47438)),
+}
+
+
+def _rng(operator, axes):
+    return random.Random(zlib.crc32(repr((operator, axes)).encode()))
+
+
+def _positive(total, parts, rng):
+    """``total`` split into exactly ``parts`` positive integers."""
+    cuts = sorted(rng.sample(range(1, total), parts - 1)) if parts > 1 else []
+    bounds = [0, *cuts, total]
+    return [b - a for a, b in zip(bounds, bounds[1:])]
+
+
+def _tokens(pages, page_size, rng):
+    return [(n - 1) * page_size + (page_size if page_size == 1 else rng.randint(1, page_size)) for n in pages]
+
+
+def decode_lengths(operator, axes, page_size):
+    """``(batch, num_pages, n_idx, kv_lens)`` of one captured decode workload."""
+    batch, pool, n_idx = axes
+    rng = _rng(operator, axes)
+    batch = min(batch, n_idx)
+    kv_lens = _tokens(_positive(n_idx, batch, rng), page_size, rng)
+    return batch, max(pool, n_idx), n_idx, kv_lens
+
+
+def case(operator, axes, dims, page_size=1, scale=None, dtype=None, device="cuda"):
+    """``(inputs, expected outputs)`` of one workload of a decode operator."""
+    from . import reference
+
+    batch, pool, n_idx, kv_lens = decode_lengths(operator, axes, page_size)
+    wl = (batch, *dims[:3], pool, n_idx)
+    inputs = reference.gqa_paged_decode_inputs(wl, kv_lens, page_size=page_size, scale=scale, dtype=dtype, device=device)
+    expected = reference.gqa_paged_decode_reference(wl, kv_lens, page_size=page_size, dtype=dtype)
+    return inputs, expected(*inputs)

@@ -242,10 +242,11 @@ class CompiledKernel:
             return None
         return outs[0] if len(outs) == 1 else outs
 
-    def time(self, *args, warmup: int = 4, iters: int = 100, rotate=None) -> float:
+    def time(self, *args, warmup: int = 4, iters: int = 100, rotate=None, only=None) -> float:
         """Milliseconds per call measured with HIP events inside the native library.  ``rotate``:
         further argument tuples (same signature) cycled through call by call, so a working set
-        larger than the 256 MB last-level cache keeps every call reading HBM."""
+        larger than the 256 MB last-level cache keeps every call reading HBM.  ``only``: indices
+        of the launches to time (e.g. ``[0]`` for the partial kernel of a fused pair alone)."""
         import torch
 
         sets = [args] + list(rotate or [])
@@ -258,6 +259,8 @@ class CompiledKernel:
                 descs, keep = self._descs(bound, dims)
             if not descs:
                 raise ValueError("cannot time an empty launch")
+            if only is not None:
+                descs, keep = [descs[i] for i in only], [keep[i] for i in only]
             all_descs.append(descs)
             all_keep.append(keep)
         with torch.cuda.device(device):

@@ -1,0 +1,129 @@
+"""GPU: ``compile()`` end to end, split-K plans chained as a two-stage Kernel, save / load /
+cache, and the paged operator through ``compile_dynamic`` (the scenarios of the reference's
+``tests/pipeline_api/test_e2e.py`` and ``tests/frontend_dynamic``)."""
+
+import time
+
+import numpy as np
+import pytest
+import torch
+
+import cleave_amd
+import cleave_amd.lang as cl
+from cleave_amd import pipeline as P
+from oracle import paged_oracle, program_oracle
+from tests import _cases as C
+
+pytestmark = pytest.mark.gpu
+SHAPES = dict(M=128, N=128, K=256)
+FAST = dict(schedule=P.ScheduleConfig(topk=3), eval=P.EvalConfig(warmup=2, iters=20, max_parallel=2))
+
+
+def _close(out, want):
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
+
+
+def test_compile_matmul_end_to_end(cache_root, tmp_path):
+    kernel = P.compile(C.matmul, shapes=SHAPES, dtype=cl.f16, split=False, **FAST)
+    report = kernel.report
+    assert kernel.variant == "solo" and kernel.latency_us > 0 and kernel.unrunnable is None
+    assert len(report.correct) >= 1 and set(report.timings) >= {"superoptimize", "schedule", "build"}
+    assert "main_kernel" in kernel.source
+    assert "superoptimize" in report.summary() and "benchmark" in report.summary()
+
+    prog = cleave_amd.trace(C.matmul, SHAPES, cl.f16)
+    x, w = prog.random_inputs(seed=1)
+    want = program_oracle.evaluate(prog, [x, w])[0]
+    _close(kernel(x, w), want)
+    _close(kernel(w=w, x=x), want)
+    with pytest.raises(ValueError):
+        kernel(w, x)   # wrong shapes are rejected, not silently transposed
+
+    loaded = P.load(kernel.save(tmp_path / "saved"))
+    assert loaded.latency_us == kernel.latency_us and loaded.input_names == ["x", "w"]
+    _close(loaded(x, w), want)
+
+    t0 = time.perf_counter()
+    again = P.compile(C.matmul, shapes=SHAPES, dtype=cl.f16, split=False, **FAST)
+    assert again.meta["cache"] == "hit" and time.perf_counter() - t0 < 30
+    _close(again(x, w), want)
+
+
+def test_split_k_schedule_and_chained_kernel(cache_root):
+    prog = cleave_amd.trace(C.matmul, SHAPES, cl.f16)
+    graphs = P.superoptimize(prog, P.SuperoptConfig(split=("K",)))
+    assert any(g.is_split for g in graphs) and any(not g.is_split for g in graphs)
+    plans = P.schedule(graphs, P.ScheduleConfig(topk=3, split_k=(4, 8)))
+    roles = {(p.variant, p.role) for p in plans}
+    assert {("solo", "main"), ("split-k=4", "partial"), ("split-k=4", "combine"), ("split-k=8", "partial"),
+            ("split-k=8", "combine")} <= roles
+    assert all(p.inputs is not None for p in plans if p.role != "combine")
+    assert not plans.refused, plans.summary()
+    cached = P.superoptimize(prog, P.SuperoptConfig(split=("K",)))
+    assert cached.from_cache and len(cached) == len(graphs)
+
+    split4 = plans.filter(lambda p: p.variant == "split-k=4")
+    report = P.evaluate(split4, P.EvalConfig(warmup=2, iters=20, max_parallel=2))
+    kernel = report.best("split-k=4")
+    assert [s.role for s in kernel.stages] == ["partial", "combine"]
+    parts = report.variants()["split-k=4"].members
+    assert kernel.latency_us == pytest.approx(sum(m.latency_us for m in parts))
+    x, w = prog.random_inputs(seed=2)
+    _close(kernel(x, w), program_oracle.evaluate(prog, [x, w])[0])
+
+
+def test_compile_picks_a_split_variant_for_decode_attention(cache_root):
+    shapes = dict(HQ=32, HKV=8, SQ=1, SKV=2048, D=128)
+    kernel = P.compile(C.gqa_decode_exact, shapes=shapes, dtype=cl.f16, split=cl.Split("SKV", (4, 8)),
+                       schedule=P.ScheduleConfig(topk=2, split_k=(4, 8)), eval=P.EvalConfig(warmup=2, iters=20, max_parallel=0))
+    assert set(kernel.report.variants()) >= {"solo", "split-k=4", "split-k=8"}
+    prog = cleave_amd.trace(C.gqa_decode_exact, shapes, cl.f16)
+    ins = C.inputs_c3(shapes, device="cuda")
+    _close(kernel(*ins), program_oracle.evaluate(prog, ins)[0])
+
+
+def test_session_scopes_compile(tmp_path, monkeypatch):
+    monkeypatch.setenv("CLEAVE_CACHE_ROOT", str(tmp_path / "env"))
+    with cleave_amd.Session(cache_root=tmp_path / "session", max_parallel=2):
+        kernel = P.compile(C.matmul, shapes=SHAPES, dtype=cl.f16, split=False, **FAST)
+    assert str(tmp_path / "session") in kernel.meta["saved"]
+    (built,) = kernel.kernels
+    assert built.source == kernel.source and built.entry == "main_kernel"
+    assert len(built.inputs) == 2 and len(built.outputs) == 1
+    assert [p.role for p in built.params][-1] == "output" and built.plan is kernel.plan
+
+
+batch, num_pages, n_idx = cl.dims("batch num_pages n_idx", dynamic=True)
+kv_len = cl.Dim("kv_len", dynamic=True, hint=4096)
+
+
+def paged_op(H_Q=32, H_KV=8, D=128, PAGE=64):
+    @cleave_amd.jit(name=f"gqa_paged_decode_h{H_Q}_kv{H_KV}_d{D}_ps{PAGE}_test", dtype=cl.f16)
+    def op(q: cl.Tensor[batch, H_Q, D], k_cache: cl.Tensor[num_pages, PAGE, H_KV, D],
+           v_cache: cl.Tensor[num_pages, PAGE, H_KV, D], kv_indptr: cl.Tensor[batch + 1, cl.i32],
+           kv_indices: cl.Tensor[n_idx, cl.i32], kv_last_page_len: cl.Tensor[batch, cl.i32] | None,
+           sm_scale: cl.Scalar[cl.f32]):
+        pages = cl.PageTable(kv_indptr, kv_indices, last_page_len=kv_last_page_len, length=kv_len)
+        k, v = cl.paged_gather(k_cache, pages), cl.paged_gather(v_cache, pages)
+        qg = q.view(batch, H_KV, H_Q // H_KV, D)
+        p, lse = cl.softmax((qg @ k.mT) * sm_scale, dim=-1, return_lse=True)
+        return (p @ v).view(batch, H_Q, D), lse.view(batch, H_Q)
+
+    return op
+
+
+def test_compile_dynamic_paged_decode(cache_root):
+    op = paged_op()
+    kernel = cleave_amd.compile(op, schedule=P.ScheduleConfig(topk=2), split=cl.Split("kv_len", (4,)),
+                                workloads=cl.workloads.paged_decode(batch=(1, 5), kv_len=(40, 900), samples=2),
+                                max_workloads=2)
+    rep = kernel.report
+    assert rep.best() is not None and len(rep.correct) >= 2 and "validate" in rep.summary()
+    lens = [70, 0, 513, 64]
+    args = C.paged_workload(lens, page_size=64, num_pages=64, device="cuda")
+    out, lse = kernel(*args)
+    want_o, want_l = paged_oracle.decode(*[a.cpu() if isinstance(a, torch.Tensor) else a for a in args[:5]], lens, 64,
+                                         args[-1])
+    _close(out, want_o)
+    live = np.isfinite(want_l)
+    np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
