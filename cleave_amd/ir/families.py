@@ -324,7 +324,7 @@ def _try_attention(view, out):
         return "mla", prob, {"Q": q, "QPE": qpe, "KV": kv, "KPE": kpe}
     (q, k), = terms
     sq_, sk_ = tuple(q.shape), tuple(k.shape)
-    if len(sq_) != len(sk_) or len(sq_) < 3 or tuple(v.shape[:-1]) != sk_[:-1]:
+    if len(sq_) != len(sk_) or len(sq_) < 2 or tuple(v.shape[:-1]) != sk_[:-1]:
         raise LoweringRejected(f"attention operands do not line up: q {sq_}, k {sk_}, v {tuple(v.shape)}")
     bq, bk = sq_[:-2], sk_[:-2]
     for i, (x, y) in enumerate(zip(bq, bk)):

@@ -181,7 +181,7 @@ def run_candidates(candidates, dtype, *, max_parallel: int = 8, tolerance: Toler
 
     if max_parallel == 0:  # in-process: no isolation, no timeouts
         try:
-            with tqdm(total=total) as bar:
+            with tqdm(total=total, disable=None) as bar:
                 for i, cand in enumerate(candidates, start=1):
                     job, task = prepare(i, cand)
                     if task is not None:
@@ -247,7 +247,7 @@ def run_candidates(candidates, dtype, *, max_parallel: int = 8, tolerance: Toler
     except Exception:  # noqa: BLE001 - surfaces per candidate in prepare()
         pass
     try:
-        with tqdm(total=total) as bar:
+        with tqdm(total=total, disable=None) as bar:
             fill(bar)
             last_beat = time.monotonic()
             while active:

@@ -83,6 +83,14 @@ def load():
             raise BackendUnavailable(
                 f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C cleave_amd/csrc`; there is no fallback path")
+        # PyTorch bundles its own HIP runtime under the same sonames as the system one.  A
+        # process must end up with exactly one of them: importing torch first makes the
+        # dynamic loader resolve this library's libamdhip64 / libhiprtc to the copies torch
+        # already mapped (the other order leaves torch unable to see the GPU).
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         try:
             lib = ctypes.CDLL(str(path))
         except OSError as e:
