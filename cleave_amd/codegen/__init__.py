@@ -318,6 +318,7 @@ class HipCodeGen:
         unit.define("CL_HEAD_DIM", p["head_dim"])
         unit.define("CL_ROWS", rows)
         unit.define("CL_WAVES", waves)
+        unit.define("CL_PREFETCH", int(t.get("PREFETCH", 1)))
         unit.define("CL_PAGED", paged)
         unit.define("CL_PAGE_SIZE", p.get("page_size", 1))
         unit.define("CL_KV_HEADS", p.get("kv_heads", 1))

@@ -19,6 +19,7 @@
 //   CL_Q_HEADS   query heads (paged)     CL_SKV      kv length (dense)
 //   CL_SCALE_LOG2E softmax scale * log2(e) (dense; paged passes sm_scale at run time)
 //   CL_EMIT_LSE  also write the base-2 log-sum-exp
+//   CL_PREFETCH  steps of K/V in flight ahead of the one being computed (1 or 2)
 
 #define ATT_STEP 32
 #define ATT_KJ (CL_HEAD_DIM / 32)            // score MFMAs per 16 tokens
@@ -166,62 +167,84 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[vc][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  AttTile cur, nxt;
-  int step = step_begin + wave;
-  if (step < step_end) att_load(u, step * ATT_STEP, c, g, cur);
-  for (; step < step_end; step += CL_WAVES) {
-    const int t0 = step * ATT_STEP;
-    const bool more = step + CL_WAVES < step_end;
-    if (more) att_load(u, (step + CL_WAVES) * ATT_STEP, c, g, nxt);
+  // Ring of CL_PREFETCH + 1 register tiles: while step n is in the matrix cores the loads of
+  // steps n+1 .. n+CL_PREFETCH are in flight.  The ring position is a compile-time constant of
+  // the unrolled inner loop, so every tile stays in registers.
+  AttTile ring[CL_PREFETCH + 1];
+  const int step0 = step_begin + wave;
+  // Prefetch loads are issued unconditionally: a step past the end is clamped onto this wave's
+  // last real step (an L2 hit, its tile is never consumed).  A branch around the loads would
+  // make the hardware load counter differ between paths, and the waits the compiler then has
+  // to insert drain the prefetch before every value product.
+  int last_step = step0;
+  if (step_end > step0) last_step = step0 + ((step_end - 1 - step0) / CL_WAVES) * CL_WAVES;
+  if (step0 < step_end) {
+#pragma unroll
+    for (int i = 0; i < CL_PREFETCH; ++i) {
+      int sidx = step0 + i * CL_WAVES;
+      sidx = sidx < last_step ? sidx : last_step;
+      att_load(u, sidx * ATT_STEP, c, g, ring[i]);
+    }
+  }
+  for (int base = step0; base < step_end; base += (CL_PREFETCH + 1) * CL_WAVES) {
+#pragma unroll
+    for (int r = 0; r <= CL_PREFETCH; ++r) {
+      const int step = base + r * CL_WAVES;
+      if (step >= step_end) break;
+      int ahead = step + CL_PREFETCH * CL_WAVES;
+      ahead = ahead < last_step ? ahead : last_step;
+      att_load(u, ahead * ATT_STEP, c, g, ring[(r + CL_PREFETCH) % (CL_PREFETCH + 1)]);
+      const AttTile& cur = ring[r];
+      const int t0 = step * ATT_STEP;
 
-    // scores^T for the two 16-token halves
-    float s[8];
+      // scores^T for the two 16-token halves
+      float s[8];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      f32x4 st = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int h = 0; h < 2; ++h) {
+        f32x4 st = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < ATT_KJ; ++j) st = mfma16(as_elem8(cur.k[h][j]), qf[j], st);
+        for (int j = 0; j < ATT_KJ; ++j) st = mfma16(as_elem8(cur.k[h][j]), qf[j], st);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = t0 + 16 * h + 4 * g + r;
-        s[4 * h + r] = t < u.kv_len ? st[r] * scale2 : CL_NEG_BIG;
+        for (int q = 0; q < 4; ++q) {
+          const int t = t0 + 16 * h + 4 * g + q;
+          s[4 * h + q] = t < u.kv_len ? st[q] * scale2 : CL_NEG_BIG;
+        }
+      }
+      float mx = s[0];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
+      mx = fmaxf(mx, lane_xor(mx, lane, 16));
+      mx = fmaxf(mx, lane_xor(mx, lane, 32));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2(m_run - m_new);
+      m_run = m_new;
+      elem8 pf;
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        // masked slots hold CL_NEG_BIG; when the whole row is still masked m_new equals it too,
+        // so test the mask itself rather than trusting exp2 of a zero difference
+        float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;
+        elem_t pe = to_elem(p);
+        psum += to_f32(pe);            // the sum uses the weights the value product really sees
+        pf[i] = pe;
+      }
+      l_run = l_run * alpha + psum;
+
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // wave-uniform: skip when no max moved
+#pragma unroll
+        for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[vc][j] *= alpha;
+      }
+#pragma unroll
+      for (int vc = 0; vc < ATT_VC; ++vc) {
+        u32x4 vt[8];
+        transpose8x8(cur.v[vc], vt);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[vc][j] = mfma16(as_elem8(vt[j]), pf, acc[vc][j]);
       }
     }
-    float mx = s[0];
-#pragma unroll
-    for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-    mx = fmaxf(mx, lane_xor(mx, lane, 16));
-    mx = fmaxf(mx, lane_xor(mx, lane, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = fast_exp2(m_run - m_new);
-    m_run = m_new;
-    elem8 pf;
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      // masked slots hold CL_NEG_BIG; when the whole row is still masked m_new equals it too,
-      // so test the mask itself rather than trusting exp2 of a zero difference
-      float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;
-      elem_t pe = to_elem(p);
-      psum += to_f32(pe);            // the sum uses the weights the value product really sees
-      pf[i] = pe;
-    }
-    l_run = l_run * alpha + psum;
-
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // wave-uniform: skip when no max moved
-#pragma unroll
-      for (int vc = 0; vc < ATT_VC; ++vc)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[vc][j] *= alpha;
-    }
-#pragma unroll
-    for (int vc = 0; vc < ATT_VC; ++vc) {
-      u32x4 vt[8];
-      transpose8x8(cur.v[vc], vt);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[vc][j] = mfma16(as_elem8(vt[j]), pf, acc[vc][j]);
-    }
-    if (more) cur = nxt;
   }
 
   // ---- merge the workgroup's waves through LDS ----------------------------------------------
