@@ -94,14 +94,19 @@ def run_dense(name, op, steps, warmup, search_iters):
     import cleave_amd
     from cleave_amd import pipeline as P
 
+    import contextlib
+
     t0 = time.perf_counter()
     program = op["fn"].trace(op["dtype"], **op["shapes"])
-    kernel = cleave_amd.compile(program, preset="fast", split=op["split"], cache_kernels=False,
-                                schedule=P.ScheduleConfig(topk=12, split_k=getattr(op["split"], "factors", ())),
-                                eval=P.EvalConfig(warmup=3, iters=search_iters, max_parallel=0))
+    with contextlib.redirect_stdout(sys.stderr):   # stdout carries the one JSON line and nothing else
+        kernel = cleave_amd.compile(program, preset="fast", split=op["split"], cache_kernels=False,
+                                    schedule=P.ScheduleConfig(topk=12, split_k=getattr(op["split"], "factors", ())),
+                                    eval=P.EvalConfig(warmup=3, iters=search_iters, max_parallel=0))
     report = kernel.report
     log(f"[{name}] search {time.perf_counter() - t0:.1f}s: {len(report)} candidates, {len(report.correct)} valid; "
         f"best {kernel.variant} {kernel.label}")
+    for r in report.failures[:3]:
+        log(f"[{name}]   failed {r.label}: {str(r.error).strip().splitlines()[1:4]}")
     fused = fused_kernel(kernel)
     sets = [[t.cuda() for t in op["inputs"](op["shapes"], seed=100 + i)] for i in range(op["sets"])]
     ms = fused.time(*sets[0], warmup=warmup, iters=steps, rotate=sets[1:])

@@ -299,7 +299,7 @@ int chip_time_launches(const chip_launch_desc* seq, int n, void* stream, int war
   HIP_TRY(hipEventCreate(&t0));
   hipError_t e = hipEventCreate(&t1);
   if (e != hipSuccess) {
-    hipEventDestroy(t0);
+    (void)hipEventDestroy(t0);
     return hip_fail("hipEventCreate", e);
   }
   int rc = CHIP_OK;
@@ -319,8 +319,8 @@ int chip_time_launches(const chip_launch_desc* seq, int n, void* stream, int war
     e = hipEventElapsedTime(&ms, t0, t1);
     if (e != hipSuccess) rc = hip_fail("hipEventElapsedTime", e);
   }
-  hipEventDestroy(t0);
-  hipEventDestroy(t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
   if (rc == CHIP_OK) *ms_per_iter = ms / (float)iters;
   return rc;
 }

@@ -73,22 +73,29 @@ class _View:
                     if self._is_split_sum(n):
                         self.carries[n] = False
                     else:
+                        # an unsplit graph input next to a split operand is a broadcast over the
+                        # splits (the query of a split-KV attention); an unsplit *computed* tensor
+                        # there means two siblings took different sides of the cut
                         tensors_mixed = any(flags) and not all(flags) and any(
-                            not f and not self._is_row_constant(i) for f, i in zip(flags, n.inputs))
+                            not f and not isinstance(i, PlaceHolderNode) for f, i in zip(flags, n.inputs))
                         if tensors_mixed and n.op in ("matmul", "add", "sub", "mul", "div"):
                             raise LoweringRejected(
                                 f"{n.name} mixes a split operand with an unsplit one: the split boundary is not clear")
                         self.carries[n] = any(flags)
+        # An input that is split for one consumer must be split for all of them: horizontally
+        # fusable siblings have to share one splitting, or the partial kernel has no single grid.
+        for n in graph.nodes:
+            if isinstance(n, ComputeOpNode) and n.op != "split":
+                for i in n.inputs:
+                    if isinstance(i, PlaceHolderNode) and i.name in self.split_axes:
+                        raise LoweringRejected(f"input {i.name} is consumed both split and unsplit ({n.name}): "
+                                               "the split boundary is not clear")
         for out in graph.outputs:
             if self.carries.get(out.source):
                 raise LoweringRejected("a graph output still carries the split axis (no reduction over it)")
 
     def _is_split_sum(self, n) -> bool:
         return _is(n, "reduce_sum") and n.attrs.get("dim") == 0 and self.carries.get(n.inputs[0], False)
-
-    @staticmethod
-    def _is_row_constant(n) -> bool:
-        return False
 
     @property
     def is_split(self) -> bool:

@@ -67,6 +67,13 @@ class BuiltKernel:
         return _compile(_load_main_kernel_from_code(self.source), list(self.out_idx))
 
 
+def resolve_tolerance(config):
+    """The bound candidates are validated against: the config's, else the strict 1e-2 / 1e-2."""
+    from ..runtime.validate import STRICT_TOLERANCE
+
+    return config.tolerance or STRICT_TOLERANCE
+
+
 def built_kernels(plans: Sequence[Plan], runs) -> list:
     out = []
     for plan, run in zip(plans, runs):
@@ -107,7 +114,7 @@ def build(plans, workers: int | None = None, *, config: EvalConfig | None = None
     Parallelism: ``workers``, else the active ``Session.max_parallel``, else ``config``."""
     from ..core.session import current_session
     from ..runtime.evaluate import run_candidates
-    from ..runtime.validate import STRICT_TOLERANCE, BenchOptions
+    from ..runtime.validate import BenchOptions
 
     config = config or EvalConfig()
     session = current_session()
@@ -118,7 +125,7 @@ def build(plans, workers: int | None = None, *, config: EvalConfig | None = None
     t0 = time.perf_counter()
     parallel = workers if workers is not None else (session.max_parallel or config.max_parallel)
     runs = run_candidates([p.tile for p in plan_list], _program_dtype(plans), max_parallel=parallel,
-                          tolerance=config.tolerance or STRICT_TOLERANCE, timeout_s=timeout,
+                          tolerance=resolve_tolerance(config), timeout_s=timeout,
                           compiler_pass_options=compiler_pass_options,
                           benchmark=BenchOptions(config.warmup, config.iters))
     kernels = built_kernels(plan_list, runs)

@@ -77,7 +77,7 @@ def publish_reference(reference_cache_dir, graph, dtype, device: str = "cuda"):
         os.makedirs(reference_cache_dir, exist_ok=True)
         tmp = path.with_name(f"{path.name}.tmp.{os.getpid()}")
         torch.save({"inputs_by_name": {k: v.cpu() for k, v in inputs_by_name.items()},
-                    "reference": [r.cpu() for r in reference]}, tmp)
+                    "reference": [r.cpu() for r in reference], "compare": compare_mode(graph)}, tmp)
         os.replace(tmp, path)
         io_bytes = _live_bytes(inputs_by_name.values()) + _live_bytes(reference)
         del inputs_by_name, reference
@@ -87,18 +87,37 @@ def publish_reference(reference_cache_dir, graph, dtype, device: str = "cuda"):
     return out_idx, io_bytes
 
 
-def _load_reference(reference_cache_dir, device: str = "cuda"):
+def compare_mode(graph) -> str:
+    """How a stage's raw outputs are compared.  Softmax partials (m, l, O) are unnormalised sums
+    whose low-order bits depend on the order the running maximum was met in, so they are
+    compared as (m, l, O / l): the quantities the combine actually consumes."""
+    low = getattr(graph, "lowered", None)
+    if low is not None and getattr(graph, "role", "main") == "partial" and low.family in ("attention", "mla"):
+        return "softmax_partial"
+    return "plain"
+
+
+def _comparable(outputs, mode):
+    if mode != "softmax_partial":
+        return list(outputs)
+    pm, pl, po = (t.float() for t in outputs)
+    return [pm, pl, po / pl.clamp_min(1e-30).unsqueeze(-1)]
+
+
+def _load_reference(reference_cache_dir, device: str = "cuda", with_mode: bool = False):
     import torch
 
     payload = torch.load(_reference_path(reference_cache_dir), map_location=device, weights_only=True)
-    return dict(payload["inputs_by_name"]), list(payload["reference"])
+    loaded = dict(payload["inputs_by_name"]), list(payload["reference"])
+    return (*loaded, payload.get("compare", "plain")) if with_mode else loaded
 
 
 def _as_list(x):
     return list(x) if isinstance(x, (tuple, list)) else [x]
 
 
-def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance = DEFAULT_TOLERANCE):
+def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance = DEFAULT_TOLERANCE,
+                             compare: str = "plain"):
     """Run ``kernel(*inputs)`` and assert every output is within ``tolerance`` of ``reference``."""
     import torch
 
@@ -108,8 +127,9 @@ def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance 
     torch.cuda.synchronize()
     assert len(actual) == len(reference), (
         f"Kernel returned {len(actual)} outputs but the reference has {len(reference)}.")
+    reference = [reconcile_output_layout(want, got.shape).to(got.device) for got, want in zip(actual, reference)]
+    actual, reference = _comparable(actual, compare), _comparable(reference, compare)
     for got, want in zip(actual, reference):
-        want = reconcile_output_layout(want, got.shape)
         torch.testing.assert_close(got.float(), want.float().to(got.device), rtol=tolerance.rtol,
                                    atol=tolerance.atol, equal_nan=tolerance.equal_nan)
 
@@ -123,11 +143,12 @@ def _check_kernel(kernel, *, graph=None, dtype=None, reference_cache_dir=None,
     with _gpu_exec_guard():
         with _stage("validate"):
             if reference_cache_dir is not None:
-                inputs_by_name, reference = _load_reference(reference_cache_dir)
+                inputs_by_name, reference, mode = _load_reference(reference_cache_dir, with_mode=True)
             else:
                 inputs_by_name, reference, _ = build_inputs_and_reference(graph, dtype)
+                mode = compare_mode(graph)
             inputs = order_inputs_for_kernel(inputs_by_name, kernel)
-            _validate_kernel_outputs(kernel, inputs, reference, tolerance=tolerance)
+            _validate_kernel_outputs(kernel, inputs, reference, tolerance=tolerance, compare=mode)
         if benchmark is None:
             return None
         with _stage("bench"):

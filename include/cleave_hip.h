@@ -65,16 +65,21 @@ typedef struct chip_device_info {
                                      (python/cleave/runtime/gpu.py:15-38) */
 } chip_device_info;
 
-/* ABI version of the loaded library. */
+/* ABI version of the loaded library.  Has no counterpart in the reference
+ * (its boundary is Python objects, never a versioned binary interface). */
 int chip_abi_version(void);
 
-/* Last failure text on this thread ("" if none). Never NULL. */
+/* Last failure text on this thread ("" if none). Never NULL.  Carries what
+ * the reference gets as a Python exception out of its JIT and classifies at
+ * python/cleave/runtime/evaluate.py:107-133. */
 const char* chip_last_error(void);
 
-/* Number of visible HIP devices, or a negative chip_status. */
+/* Number of visible HIP devices, or a negative chip_status.  Stands in for
+ * the device enumeration behind python/cleave/runtime/gpu.py:15-38. */
 int chip_device_count(void);
 
-/* Fill `info` for device `dev`. */
+/* Fill `info` for device `dev`.  Stands in for get_cuda_device_properties and
+ * the attribute getters at python/cleave/arch/driver/cuda_driver.py:80-218. */
 int chip_device_info_get(int dev, chip_device_info* info);
 
 /* Compile HIP source text for `arch` (e.g. "gfx950") with hiprtc.
@@ -88,19 +93,28 @@ int chip_compile(const char* source, const char* name, const char* arch,
                  const char* const* opts, int nopts,
                  void** code, size_t* size, char** log);
 
-/* Release memory returned by chip_compile. */
+/* Release memory returned by chip_compile.  Has no counterpart in the
+ * reference (the JIT's kernel object owns its binary there). */
 void chip_free(void* p);
 
-/* Load a code object on the current device. */
+/* Load a code object on the current device.  Second half of what `tl.compile`
+ * returns at python/cleave/runtime/compile.py:30-34 (a loaded, callable
+ * kernel); kept separate so compile can run on a GPU-less host. */
 int chip_module_load(const void* code, size_t size, void** module);
 
-/* Unload a module and every function handle obtained from it. */
+/* Unload a module and every function handle obtained from it.  Stands in
+ * for dropping the JIT kernel in the worker's per-task cleanup
+ * (python/cleave/runtime/workers.py:93-101). */
 int chip_module_unload(void* module);
 
-/* Look up an `extern "C" __global__` entry by name. */
+/* Look up an `extern "C" __global__` entry by name: `main_kernel`, the entry
+ * the reference loads at python/cleave/runtime/compile.py:37-58. */
 int chip_get_function(void* module, const char* name, void** fn);
 
-/* Static resource usage of a kernel (for occupancy-aware ranking). */
+/* Static resource usage of a kernel (for occupancy-aware ranking and spill
+ * detection).  Has no counterpart in the reference, which learns of register
+ * or shared-memory overflow only from the launch failure markers at
+ * python/cleave/runtime/evaluate.py:96-104. */
 typedef struct chip_func_attr {
   int32_t num_regs;           /* VGPRs per lane */
   int32_t static_lds_bytes;
@@ -128,7 +142,10 @@ typedef struct chip_launch_desc {
   void** args;
 } chip_launch_desc;
 
-/* Enqueue `n` launches back to back on `stream`. */
+/* Enqueue `n` launches back to back on `stream`.  Stands in for the kernel
+ * call inside the reference's fused partial+combine `main_kernel`
+ * (python/cleave/codegen/split.py:78-125) and for `kernel(*args)` at
+ * python/cleave/runtime/timer.py:66-73. */
 int chip_launch_seq(const chip_launch_desc* seq, int n, void* stream);
 
 /* Time the sequence: `warmup` untimed passes, then `iters` passes between two

@@ -1,0 +1,161 @@
+"""Lowering of op-dict structures (the reference's stored superoptimizer output as data),
+operator recognition, the gfx950 schedule space, and what the emitter writes."""
+
+import json
+from pathlib import Path
+
+import pytest
+
+import cleave_amd.lang as cl
+from cleave_amd.codegen import HipCodeGen, parse_manifest
+from cleave_amd.core.errors import CodegenError, LoweringRejected, ScheduleRejected
+from cleave_amd.ir import recognize, to_ir
+from cleave_amd.lower import to_bundles
+from cleave_amd.lower.stages import partial_buffers, split_stages
+from cleave_amd.schedule import apply_tiling, search_tiling
+from cleave_amd.schedule.hint import TileDict
+from tests import _cases as C
+from tests._lowlevel import source_for, stage_graph
+
+STRUCT = Path(__file__).parent / "golden" / "graph_structures"
+
+
+def stored(name, **kw):
+    return to_ir(json.loads((STRUCT / name).read_text()), dtype="float16", **kw)
+
+
+def test_stored_split_k_matmul_is_read_through_its_split_ops():
+    low = recognize(stored("before_split_matmul_split_k_graph_structure.graph"))
+    assert low.family == "matmul" and low.split_dim == "K"
+    assert (low.problem["M"], low.problem["N"], low.problem["K"]) == (4, 8, 12)
+    assert sorted(low.split_axes.values()) == [0, 1]            # A split on its K axis (1), B on its K axis (0)
+
+
+def test_stored_reordered_rmsnorm_matmul_is_recognised():
+    """The superoptimizer's (x @ w) * rsqrt(sum(x*x)/K) form, symbolic extents mapped to real ones."""
+    low = recognize(stored("before_split_rmsnorm_matmul_graph_structure_valid_1.graph", symbol_map={12: 4096}))
+    assert low.family == "rmsnorm_matmul" and low.problem["K"] == 4096 and low.problem["eps"] == 0.0
+    assert not low.problem["gamma"] and set(low.operands) == {"A", "B"}
+
+
+def test_stored_split_gqa_is_attention_split_over_kv():
+    low = recognize(stored("before_split_gqa_graph_structure_valid_1.graph"))
+    p = low.problem
+    assert low.family == "attention" and low.split_dim == "SKV"
+    assert (p["units"], p["group"], p["sq"], p["skv"], p["head_dim"]) == (4, 2, 12, 16, 20)
+    assert p["scale"] == pytest.approx(1 / 8.0) and p["shift"] == -6.25 and not p["exact"]
+
+
+@pytest.mark.parametrize("name", ["before_split_rmsnorm_matmul_graph_structure_invalid_1.graph",
+                                  "before_split_rmsnorm_matmul_graph_structure_invalid_3.graph",
+                                  "before_split_gqa_graph_structure_invalid_2.graph",
+                                  "before_split_gqa_graph_structure_invalid_3.graph"])
+def test_stored_invalid_splits_are_refused(name):
+    with pytest.raises(LoweringRejected):
+        recognize(stored(name, symbol_map={12: 4096}))
+
+
+def test_cut_pair_structure_parses_but_is_not_a_single_operator():
+    pair = json.loads((STRUCT / "after_split_matmul_split_k_graph_structure.graph").read_text())
+    partial, combine = (to_ir(s, dtype="float16") for s in pair)
+    assert partial.op_kinds() == ["split", "split", "matmul"] and combine.op_kinds() == ["reduce_sum"]
+    with pytest.raises(LoweringRejected):
+        recognize(partial)      # its output still carries the split axis: a cut partial is not a whole operator
+
+
+@pytest.mark.parametrize("case,family", [("c1", "matmul"), ("c2", "rmsnorm_matmul"), ("c3", "attention"), ("c4", "mla")])
+def test_graded_programs_map_to_their_families(case, family):
+    fn, dt, _ = C.CASES[case]
+    g = stage_graph(fn.trace(dt, **C.FULL[case]))
+    assert g.lowered.family == family
+    if case == "c2":
+        assert g.lowered.problem["gamma"] and g.lowered.problem["eps"] == pytest.approx(1e-6)
+    if case == "c3":
+        assert g.lowered.problem["exact"] and (g.lowered.problem["units"], g.lowered.problem["group"]) == (64, 4)
+    if case == "c4":
+        assert g.lowered.problem["scale"] == pytest.approx(192 ** -0.5)
+
+
+def test_unrecognised_program_is_refused():
+    from cleave_amd.frontend import Program
+
+    p = Program("odd", cl.f16)
+    a = p.input("a", [8, 8])
+    p.output(a.exp().silu())
+    with pytest.raises(LoweringRejected, match="match no kernel family"):
+        stage_graph(p)
+
+
+def test_split_stages_and_partial_buffers():
+    g = stage_graph(C.gqa_decode_exact.trace(cl.f16, **C.FULL["c3"]))
+    partial, combine = split_stages(g, 16)
+    assert [o.shape for o in partial.outputs] == [(16, 256), (16, 256), (16, 256, 128)]
+    assert [p.name for p in combine.placeholders] == ["PlaceHolder_PM", "PlaceHolder_PL", "PlaceHolder_PO"]
+    assert partial_buffers(g.lowered, 16)[2][2] == "float32"
+    with pytest.raises(LoweringRejected, match="does not divide"):
+        split_stages(g, 3)
+    (bundle,) = to_bundles([C.matmul.trace(M=128, N=128, K=4096).to_graph_structure()], split_factors=[8],
+                           input_names=["x", "w"])
+    assert [s.role for s in bundle] == ["partial", "combine"] and bundle[0].outputs[0].shape == (8, 128, 128)
+
+
+def test_search_space_respects_gfx950_limits():
+    from cleave_amd.arch import GFX950
+
+    g = stage_graph(C.matmul.trace(cl.f16, M=4096, N=14336, K=4096))
+    cands = search_tiling(g, topk=10_000)
+    assert len(cands) > 50 and all(c.template == "gemm" for c in cands)
+    for c in cands:
+        t = c.tiling
+        assert t["BM"] % (16 * t["WM"]) == 0 and t["BN"] % (16 * t["WN"]) == 0 and t["BK"] in (32, 64)
+        assert c.lds_bytes <= GFX950.lds_bytes and c.n_threads % 64 == 0 and c.n_threads <= 1024
+        assert c.flat_graph is g
+    assert [c.score for c in cands] == sorted(c.score for c in cands)
+    # few rows: the weight-streaming template joins the pool
+    skinny = search_tiling(stage_graph(C.rmsnorm_matmul.trace(cl.f16, **C.FULL["c2"])), topk=10_000)
+    assert {"skinny", "gemm"} <= {c.template for c in skinny}
+    assert search_tiling(g, topk=3, accept=lambda c: c.tiling["BM"] == 256)[0].tiling["BM"] == 256
+    with pytest.raises(ScheduleRejected):
+        search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=4, HKV=4, SQ=1, SKV=64, D=48)))
+
+
+def test_emitted_signature_follows_the_naming_contract():
+    prog = C.rmsnorm_matmul.trace(cl.f16, **C.FULL["c2"])
+    m = parse_manifest(source_for(prog, template="skinny", tiling=dict(WAVES_N=1, WAVES_K=2)))
+    assert [p["name"] for p in m["params"]] == ["PlaceHolder_x", "PlaceHolder_gamma", "PlaceHolder_w", "OutputNode_0"]
+    assert m["out_idx"] == [-1] and m["launches"][0]["entry"] == "main_kernel" and m["launches"][0]["grid"][0] == "86"
+    fused = parse_manifest(source_for(prog, template="skinny", tiling=dict(WAVES_N=1, WAVES_K=2), split=8))
+    names = [p["name"] for p in fused["params"]]
+    assert names == ["PlaceHolder_x", "PlaceHolder_gamma", "PlaceHolder_w", "Partial_PACC_split", "Partial_PACC_combine",
+                     "Partial_PSS_split", "Partial_PSS_combine", "OutputNode_0"]
+    assert fused["params"][4]["alias"] == "Partial_PACC_split" and fused["params"][3]["role"] == "scratch"
+    assert [l["entry"] for l in fused["launches"]] == ["main_kernel", "main_kernel_combine"]
+    assert fused["launches"][0]["grid"][:2] == ["86", "8"]
+
+
+def test_paged_signature_matches_the_reference_operator():
+    from cleave_amd.dynamic.paging import PAGED_DECODE_SLAB, CombineTiling, DenseAttention, PagingSpec, build_split_decode
+
+    spec = PagingSpec(num_qo_heads=32, num_kv_heads=8, kind=PAGED_DECODE_SLAB, page_size=64)
+    dense = DenseAttention(16, 32, 128, 256, "bfloat16", "bfloat16", waves=4)
+    m = parse_manifest(HipCodeGen().gen(build_split_decode(spec, dense, 8, CombineTiling(split=8))))
+    names = [p["name"] for p in m["params"] if p["role"] != "scratch"]
+    assert names == ["PlaceHolder_Q", "PlaceHolder_K_CACHE", "PlaceHolder_V_CACHE", "PlaceHolder_KV_INDPTR",
+                     "PlaceHolder_KV_INDICES", "PlaceHolder_KV_LAST_PAGE_LEN", "sm_scale", "OutputNode_0", "OutputNode_1"]
+    by = {p["name"]: p for p in m["params"]}
+    assert by["PlaceHolder_K_CACHE"]["shape"] == ["num_pages", 64, 8, 128] and by["OutputNode_1"]["dtype"] == "float32"
+    assert by["Partial_PO_split"]["shape"] == [8, "batch", 32, 128] and m["dyn_dims"] == ["batch", "num_pages", "n_idx"]
+    assert m["launches"][0]["grid"] == ["(batch * 8) * 1", "8", "1"]
+
+
+def test_codegen_refuses_impossible_plans():
+    g = stage_graph(C.matmul.trace(cl.f16, M=128, N=128, K=4096))
+    with pytest.raises(CodegenError, match="multiple"):
+        HipCodeGen().gen(apply_tiling(TileDict("gemm", "main", dict(BM=64, BN=64, BK=64, WM=2, WN=2), flat_graph=g,
+                                               split_factor=None)).__class__(**{**apply_tiling(
+                                                   TileDict("gemm", "main", dict(BM=64, BN=64, BK=64, WM=2, WN=2),
+                                                            flat_graph=g)).__dict__, "problem": {**g.lowered.problem, "K": 4100}}))
+    with pytest.raises(CodegenError, match="no template"):
+        HipCodeGen().gen(apply_tiling(TileDict("nonesuch", "main", {}, flat_graph=g)))
+    with pytest.raises(CodegenError, match="manifest"):
+        parse_manifest("__global__ void k() {}")

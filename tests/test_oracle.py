@@ -1,0 +1,166 @@
+"""Pins of the numpy oracle: golden vectors (float64 closed forms), brute force on tiny inputs,
+invariants.  A dropped term, a wrong sign or index, or a transposed operand fails one of them."""
+
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import cleave_amd.lang as cl
+from cleave_amd.frontend import Program
+from oracle import paged_oracle, program_oracle as po
+from tests import _cases as C
+
+GOLD = Path(__file__).parent / "golden"
+
+
+def load(name):
+    return {k: v for k, v in np.load(GOLD / name).items()}
+
+
+def t(a, dtype=torch.float16):
+    return torch.tensor(np.asarray(a, dtype=np.float32)).to(dtype)
+
+
+def close(got, want, tol):
+    np.testing.assert_allclose(np.asarray(got, dtype=np.float64), want, rtol=tol, atol=tol)
+
+
+# ----------------------------------------------------------------------------- golden vectors
+def test_golden_matmul():
+    g = load("matmul.npz")
+    prog = C.matmul.trace(cl.f16, M=8, K=32, N=16)
+    close(po.evaluate(prog, [t(g["x"]), t(g["w"])], round_outputs=False)[0], g["y"], 1e-5)
+
+
+def test_golden_rmsnorm_matmul_with_gamma_and_eps():
+    g = load("rmsnorm_matmul.npz")
+    prog = C.rmsnorm_matmul.trace(cl.f16, M=4, K=64, N=24)
+    close(po.evaluate(prog, [t(g["x"]), t(g["gamma"]), t(g["w"])], round_outputs=False)[0], g["y"], 2e-5)
+    # and the rounded output is exactly the nearest float16 of the float32 result
+    y16 = po.evaluate(prog, [t(g["x"]), t(g["gamma"]), t(g["w"])])[0]
+    assert np.array_equal(y16, y16.astype(np.float16).astype(np.float32))
+
+
+def test_golden_gqa_attention_exact_and_shift_programs_agree():
+    g = load("gqa_attention.npz")
+    shapes = dict(HQ=6, HKV=2, SQ=3, SKV=40, D=16)
+    ins = [t(g["q"]), t(g["k"]), t(g["v"])]
+    exact = po.evaluate(C.gqa_decode_exact.trace(cl.f16, **shapes), ins, round_outputs=False)[0]
+    close(exact, g["o"], 2e-5)
+    shift = po.evaluate(C.gqa_decode_shift.trace(cl.f16, **shapes), ins, round_outputs=False)[0]
+    close(shift, g["o"], 2e-5)          # softmax is shift invariant
+
+
+def test_golden_mla_decode():
+    g = load("mla_decode.npz")
+    @cleave_amd_jit
+    def mla(q: cl.Tensor["B", "H", "D"], kv: cl.Tensor["B", "SKV", "D"], q_pe: cl.Tensor["B", "H", "PE"],
+            k_pe: cl.Tensor["B", "SKV", "PE"]):
+        return cl.softmax((q @ kv.mT + q_pe @ k_pe.mT) * (40 ** -0.5), dim=-1) @ kv
+    prog = mla.trace(cl.bf16, B=2, H=16, D=32, PE=8, SKV=20)
+    ins = [t(g[k], torch.bfloat16) for k in ("q", "kv", "q_pe", "k_pe")]
+    close(po.evaluate(prog, ins, round_outputs=False)[0], g["o"], 3e-5)
+
+
+def cleave_amd_jit(fn):
+    import cleave_amd
+
+    return cleave_amd.jit(fn)
+
+
+def test_golden_paged_decode_and_gather():
+    g = load("paged_decode.npz")
+    lens, page = g["lens"].tolist(), int(g["page"])
+    out, lse = paged_oracle.decode(g["q"], g["k_cache"], g["v_cache"], g["kv_indptr"], g["kv_indices"], lens, page,
+                                   float(g["scale"]), out_dtype="float32")
+    close(out, g["out"], 2e-5)
+    live = np.isfinite(g["lse"])
+    close(lse[live], g["lse"][live], 2e-5)
+    assert np.all(np.isneginf(lse[~live])) and np.all(out[1] == 0)      # the empty request
+    for b, n in enumerate(lens):
+        if n:
+            got = paged_oracle.gather(g["k_cache"], g["kv_indices"], int(g["kv_indptr"][b]), n, page)
+            assert np.array_equal(got, g[f"k{b}"])                       # the gather is bit exact
+
+
+# ----------------------------------------------------------------------------- brute force / invariants
+def test_every_record_kind_against_scalar_loops():
+    p = Program("p", cl.f32)
+    a, b = p.input("a", [3, 4]), p.input("b", [3, 1])
+    p.output(a - b), p.output(b - a), p.output(2.0 - a), p.output(a / b), p.output(3.0 / a)
+    p.output(a.max(-1, keepdim=True)), p.output(a.sum(0, keepdim=True)), p.output((a * a).sqrt())
+    p.output(a.silu()), p.output(a.exp()), p.output(a * 0.5 + 1.0)
+    rng = np.random.default_rng(0)
+    A, B = rng.uniform(0.5, 2, (3, 4)).astype(np.float32), rng.uniform(0.5, 2, (3, 1)).astype(np.float32)
+    got = po.evaluate(p, [A, B])
+    want = [A - B, B - A, 2 - A, A / B, 3 / A, A.max(-1, keepdims=True), A.sum(0, keepdims=True), np.abs(A),
+            A / (1 + np.exp(-A)), np.exp(A), A * 0.5 + 1]
+    for x, y in zip(got, want):
+        close(x, y.astype(np.float64), 1e-6)
+
+
+def test_grouped_matmul_is_repeat_interleave_not_tile():
+    rng = np.random.default_rng(1)
+    a, b = rng.normal(size=(6, 2, 4)).astype(np.float32), rng.normal(size=(2, 4, 5)).astype(np.float32)
+    got = po.grouped_matmul(a, b)
+    for h in range(6):
+        close(got[h], a[h].astype(np.float64) @ b[h // 3], 1e-5)       # head h pairs with kv head h // group
+    got_t = po.grouped_matmul(a, np.swapaxes(b, -1, -2).copy(), trans_b=True)
+    close(got_t, got, 1e-6)
+
+
+def test_bfloat16_rounding_matches_torch_bit_for_bit():
+    x = np.random.default_rng(2).normal(size=4096).astype(np.float32) * 37
+    x[:4] = [0.0, -0.0, 1.00390625, 3.3895314e38]                      # a tie and a near-overflow
+    want = torch.tensor(x).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(po.round_to_dtype(x, "bfloat16"), want)
+    assert np.array_equal(po.round_to_dtype(x, "float16"), torch.tensor(x).to(torch.float16).float().numpy())
+
+
+def test_page_permutation_leaves_paged_decode_unchanged():
+    lens = [5, 12, 7]
+    args = C.paged_workload(lens, page_size=4, num_pages=16, hq=4, hkv=2, d=8)
+    base = paged_oracle.decode(*args[:5], lens, 4, args[-1])
+    perm = torch.randperm(16, generator=torch.Generator().manual_seed(3))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(16)
+    moved = paged_oracle.decode(args[0], args[1][perm], args[2][perm], args[3], inv[args[4].long()], lens, 4, args[-1])
+    assert np.array_equal(base[0], moved[0]) and np.array_equal(base[1], moved[1])
+
+
+@pytest.mark.parametrize("n_pages,last,page,want", [(0, 0, 64, 0), (1, 17, 64, 17), (3, 64, 64, 192), (3, 1, 64, 129),
+                                                      (2, 999, 64, 128), (2, -5, 64, 64), (0, 9, 64, 0)])
+def test_valid_len_formula(n_pages, last, page, want):
+    assert paged_oracle.valid_len(n_pages, last, page) == want
+
+
+@pytest.mark.parametrize("n_tokens,tile,split", [(0, 64, 8), (1, 64, 8), (64 * 7 + 3, 64, 8), (16384, 32, 16), (100, 32, 32)])
+def test_every_kv_tile_is_owned_by_exactly_one_split(n_tokens, tile, split):
+    owned = []
+    for t0, trip in paged_oracle.split_ranges(n_tokens, tile, split):
+        owned += list(range(t0, t0 + trip))
+    assert owned == list(range(-(-n_tokens // tile)))
+
+
+def test_attend_lse_is_log2_of_the_partition_function():
+    rng = np.random.default_rng(4)
+    q, k, v = rng.normal(size=(2, 8)).astype(np.float32), rng.normal(size=(9, 2, 8)).astype(np.float32), \
+        rng.normal(size=(9, 2, 8)).astype(np.float32)
+    out, lse = paged_oracle.attend(q, k, v, 0.3)
+    for h in range(2):
+        s = (k[:, h].astype(np.float64) @ q[h]) * 0.3
+        assert abs(lse[h] - math.log2(np.exp(s).sum())) < 1e-5
+        close(out[h], (np.exp(s) / np.exp(s).sum()) @ v[:, h], 1e-5)
+
+
+def test_program_reference_and_oracle_agree_on_the_graded_programs():
+    """The frontend's own eager ``reference`` (torch) and the oracle (numpy) are independent
+    restatements; they must agree on every graded program."""
+    for name, (fn, dt, mk) in C.CASES.items():
+        prog = fn.trace(dt, **C.SMALL[name])
+        ins = mk(C.SMALL[name])
+        want = prog.reference(*ins)[0].float().numpy()
+        np.testing.assert_allclose(po.evaluate(prog, ins)[0], want, rtol=4e-3, atol=4e-3)
