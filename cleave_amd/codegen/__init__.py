@@ -219,7 +219,7 @@ class HipCodeGen:
     def _emit_gemm(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
         self._matmul_common(unit, plan, params, partial, combine, fused)
-        tile = dict(BM=64, BN=64, BK=32, WM=1, WN=1)
+        tile = dict(BM=64, BN=64, BK=64, WM=1, WN=1)
         tile.update(t)
         for k, v in tile.items():
             unit.define(f"CL_{k}", v)

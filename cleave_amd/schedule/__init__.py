@@ -56,7 +56,28 @@ def search_tiling(graph, topk: int = 10, force_fusion: bool = False, accept=None
             seen.add(c.key())
             c.flat_graph = graph
             unique.append(c)
-    return unique[:max(1, int(topk))]
+    return _cut(unique, max(1, int(topk)))
+
+
+def _cut(ranked, topk):
+    """The first ``topk`` of ``ranked``, except that every template in the pool keeps a share of
+    the slots (best-first within its share): the cost models of different templates are not
+    calibrated against each other well enough to let one of them crowd the other out."""
+    templates = []
+    for c in ranked:
+        if c.template not in templates:
+            templates.append(c.template)
+    if len(templates) < 2 or len(ranked) <= topk:
+        return ranked[:topk]
+    share = max(1, topk // len(templates))
+    keep = set()
+    for t in templates:
+        keep.update(id(c) for c in [c for c in ranked if c.template == t][:share])
+    for c in ranked:                      # fill what is left best-first
+        if len(keep) >= topk:
+            break
+        keep.add(id(c))
+    return [c for c in ranked if id(c) in keep][:topk]
 
 
 def _name(node_name: str) -> str:

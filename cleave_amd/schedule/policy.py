@@ -39,7 +39,7 @@ def _waves_time(blocks, per_cu, arch: Arch):
 
 # ----------------------------------------------------------------------------- GEMM
 def gemm_lds_bytes(bm, bn, bk, norm=False):
-    return 2 * (bm + bn) * (bk + 8) * 2 + (bm * 4 if norm else 0)
+    return 2 * (bm + bn) * bk * 2 + (bm * 4 if norm else 0)
 
 
 def gemm_candidates(low, role, factor, arch: Arch):
@@ -53,8 +53,8 @@ def gemm_candidates(low, role, factor, arch: Arch):
     norm = low.family == "rmsnorm_matmul"
     out = []
     shapes = (16, 32, 64, 128, 256)
-    for bm, bn, bk, (wm, wn) in itertools.product(shapes, shapes, (32, 64),
-                                                  ((1, 1), (1, 2), (2, 1), (2, 2), (1, 4), (4, 1), (2, 4), (4, 2))):
+    for bm, bn, bk, (wm, wn), depth in itertools.product(
+            shapes, shapes, (64,), ((1, 1), (1, 2), (2, 1), (2, 2), (1, 4), (4, 1), (2, 4), (4, 2)), (1, 2)):
         if bm % (16 * wm) or bn % (16 * wn) or kps % bk:
             continue
         if bm > max(16, 2 * M) or bn > max(16, 2 * N):
@@ -64,16 +64,22 @@ def gemm_candidates(low, role, factor, arch: Arch):
         acc_regs = tm * tn * 4
         if acc_regs > 256:
             continue
-        # loader granularity: K-minor tiles move 16-byte chunks, K-major ones 8x8 blocks
-        a_units = bm * (bk // 8) if not p["trans_A"] else (bm // 8) * (bk // 8)
-        b_units = bn * (bk // 8) if p["trans_B"] else (bn // 8) * (bk // 8)
         if p["trans_A"] and (bm % 8 or M % 8):
             continue
         if not p["trans_B"] and (bn % 8 or N % 8):
             continue
-        stage_regs = _ceil(a_units, threads) * (32 if p["trans_A"] else 4) \
-            + _ceil(b_units, threads) * (4 if p["trans_B"] else 32)
-        vgprs = acc_regs + stage_regs + (tm + tn) * 4 + 40
+        # staging registers per thread and step in flight: K-minor tiles move 16-byte chunks (4
+        # registers), K-major ones 8x8 blocks (32) or, when those would idle threads, 4x8 halves (16)
+        def stage(rows, k_major):
+            if not k_major:
+                return _ceil(rows * (bk // 8), threads) * 4
+            blocks = (rows // 8) * (bk // 8)
+            if rows % 64 == 0 and blocks < threads:
+                return _ceil(2 * blocks, threads) * 16
+            return _ceil(blocks, threads) * 32
+        stage_regs = depth * (stage(bm, p["trans_A"]) + stage(bn, not p["trans_B"]))
+        frag_regs = (min(tm, 3) + 2 * tn) * 4
+        vgprs = acc_regs + stage_regs + frag_regs + 40
         if vgprs > arch.vgprs_per_lane:
             continue
         lds = gemm_lds_bytes(bm, bn, bk, norm)
@@ -83,15 +89,18 @@ def gemm_candidates(low, role, factor, arch: Arch):
         per_cu = arch.blocks_per_cu(threads, lds, vgprs)
         if per_cu < 1:
             continue
+        if depth == 2 and (kps // bk < 4 or per_cu * threads > 512 and vgprs > 128):
+            continue
         passes = _waves_time(blocks, per_cu, arch)
-        # per-block cost: matrix-core cycles vs bytes pulled through L2, whichever is longer
-        mfma_clk = (bm * bn * kps * 2) / (1024.0 * min(4, wm * wn))
-        l2_clk = ((bm + bn) * kps * 2) / 48.0
-        lds_clk = (tm * 16 * wm * wn + tn * 16 * wm * wn) * kps * 2 / 128.0 * 0.5
-        block_clk = max(mfma_clk, l2_clk, lds_clk) + 2000
-        util = min(1.0, blocks / (per_cu * arch.compute_units)) if passes == 1 else 1.0
-        score = passes * block_clk * (1.0 + 0.15 * (1 - util))
-        tiling = dict(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn)
+        live = min(per_cu, _ceil(blocks, arch.compute_units))         # blocks a CU really holds
+        # one pass over the machine: the CU's matrix cores, its L1 path (about 24 B/clk sustained
+        # for these access shapes) and its LDS are shared by the blocks it holds
+        mfma_clk = live * (bm * bn * kps * 2) / 4096.0 / min(1.0, live * wm * wn / 8.0)
+        l1_clk = live * ((bm + bn) * kps * 2) / (24.0 * (1.6 if depth == 2 else 1.0))
+        lds_clk = live * (tm + tn) * 16 * wm * wn * kps * 2 / 256.0
+        pass_clk = max(mfma_clk, l1_clk, lds_clk) + 2500 + 1200 * (kps // bk) / max(1, min(live, 2))
+        score = passes * pass_clk
+        tiling = dict(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, GDEPTH=depth)
         out.append(TileDict("gemm", role, tiling, output_tile=[bm, bn], rstep_map={"k": bk}, n_threads=threads,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
     return out

@@ -26,8 +26,8 @@ def _check(program, make_inputs, shapes, **kw):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
-GEMM_TILES = [dict(BM=32, BN=32, BK=32, WM=1, WN=1), dict(BM=64, BN=64, BK=64, WM=2, WN=2),
-              dict(BM=128, BN=128, BK=32, WM=2, WN=2)]
+GEMM_TILES = [dict(BM=32, BN=32, BK=64, WM=1, WN=1), dict(BM=64, BN=64, BK=64, WM=2, WN=2),
+              dict(BM=128, BN=128, BK=64, WM=2, WN=2)]
 
 
 @pytest.mark.parametrize("tiling", GEMM_TILES, ids=lambda t: "x".join(str(v) for v in t.values()))
@@ -36,6 +36,18 @@ def test_matmul_gemm_small(tiling, split):
     fn, dt, mk = C.CASES["c1"]
     shapes = dict(M=96, N=136, K=512)
     _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=tiling, split=split)
+
+
+@pytest.mark.parametrize("tiling", [dict(BM=256, BN=256, BK=64, WM=2, WN=4, GDEPTH=1),
+                                    dict(BM=256, BN=128, BK=64, WM=4, WN=2, GDEPTH=2, GROUP_M=2),
+                                    dict(BM=128, BN=128, BK=64, WM=2, WN=2, GDEPTH=1, GROUP_M=3)],
+                         ids=lambda t: "x".join(str(v) for v in t.values()))
+def test_matmul_gemm_large_tiles(tiling):
+    """Ragged tile counts (3 x 4 or 5 x 7 tiles, not multiples of the XCD count or of GROUP_M)
+    exercise the workgroup renumbering and the clamped edge loads; K gives an odd step count."""
+    fn, dt, mk = C.CASES["c1"]
+    shapes = dict(M=600, N=776, K=448)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=tiling)
 
 
 @pytest.mark.parametrize("split", [None, 4, 8, 16])
@@ -71,8 +83,8 @@ def test_rmsnorm_matmul_c2_full(split):
 def test_rmsnorm_matmul_gemm_path():
     fn, dt, mk = C.CASES["c2"]
     shapes = dict(M=128, K=512, N=256)
-    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=32, WM=2, WN=2))
-    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=32, WM=2, WN=2), split=4)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=64, WM=2, WN=2))
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=64, WM=2, WN=2), split=4)
 
 
 @pytest.mark.parametrize("waves", [1, 2, 4])
