@@ -208,32 +208,34 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
     best = None
     tried = valid = 0
     saved = saved_choice(kernels_dir, "c5")
-    for waves in (1, 2, 4) if saved is None else ():
-        for split in (4, 8, 16):
-            dense = DenseAttention(16, 32, d, waves * 64, "float16", "float16", waves=waves)
-            src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split)))
-            loaded = _load_main_kernel_from_code(src)
-            k = _compile(loaded, loaded.manifest["out_idx"])
-            tried += 1
-            out, lse = k(*args)
-            torch.cuda.synchronize()
-            try:
-                torch.testing.assert_close(out.float(), want[0].float(), rtol=1e-2, atol=1e-2)
-                torch.testing.assert_close(lse, want[1], rtol=1e-2, atol=1e-2)
-            except AssertionError as e:
-                log(f"[c5] waves={waves} split={split} INVALID: {str(e).splitlines()[0]}")
-                continue
-            valid += 1
-            us = k.time(*args, warmup=2, iters=10) * 1e3
-            log(f"[c5] waves={waves} split={split}: {us:.1f} us")
-            if best is None or us < best[0]:
-                best = (us, waves, split, k, src)
+    configs = [dict(waves=w, split=sp) for w in (2, 4) for sp in (8, 16)]
+    configs += [dict(waves=hkv, split=8, chunk_pages=cp, prefetch=pf) for cp in (8, 16, -1) for pf in (1,)]
+    for cfg in configs if saved is None else ():
+        dense = DenseAttention(16, 32, d, cfg["waves"] * 64, "float16", "float16", waves=cfg["waves"],
+                               chunk_pages=cfg.get("chunk_pages", 0), prefetch=cfg.get("prefetch", 1))
+        src = HipCodeGen().gen(build_split_decode(spec, dense, cfg["split"], CombineTiling(split=cfg["split"])))
+        loaded = _load_main_kernel_from_code(src)
+        k = _compile(loaded, loaded.manifest["out_idx"])
+        tried += 1
+        out, lse = k(*args)
+        torch.cuda.synchronize()
+        try:
+            torch.testing.assert_close(out.float(), want[0].float(), rtol=1e-2, atol=1e-2)
+            torch.testing.assert_close(lse, want[1], rtol=1e-2, atol=1e-2)
+        except AssertionError as e:
+            log(f"[c5] {cfg} INVALID: {str(e).splitlines()[0]}")
+            continue
+        valid += 1
+        us = k.time(*args, warmup=2, iters=10) * 1e3
+        log(f"[c5] {cfg}: {us:.1f} us")
+        if best is None or us < best[0]:
+            best = (us, cfg, k, src)
     if saved is None:
-        _, waves, split, k, src = best
-        save_choice(kernels_dir, "c5", src, {"waves": waves, "split": split, "candidates": tried, "validated": valid})
+        _, cfg, k, src = best
+        save_choice(kernels_dir, "c5", src, {"cfg": cfg, "candidates": tried, "validated": valid})
     else:
         src, info = saved
-        waves, split, tried, valid = info["waves"], info["split"], info["candidates"], info["validated"]
+        cfg, tried, valid = info["cfg"], info["candidates"], info["validated"]
         k = compiled(src)
         out, lse = k(*args)
         torch.testing.assert_close(out.float(), want[0].float(), rtol=1e-2, atol=1e-2)
@@ -242,8 +244,9 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
     nbytes = sum(lens) * hkv * d * 2 * 2 + total_pages * 4 + 2 * 32 * hq * d * 2 + 32 * hq * 4 + 33 * 4 + 32 * 4
     flops = 4 * sum(lens) * hq * d
     res = {"op": "c5", "workload": f"paged GQA decode f16, 32 requests ({sum(lens)} tokens), page 64, 300k-page pool",
-           "best_us": round(us, 3), "dominant_kernel_us": round(dom, 3), "variant": f"split-kv={split}",
-           "plan": f"waves={waves}", "candidates": tried, "validated": valid,
+           "best_us": round(us, 3), "dominant_kernel_us": round(dom, 3),
+           "variant": f"chunked items of {cfg['chunk_pages']} pages" if cfg.get("chunk_pages") else f"split-kv={cfg['split']}",
+           "plan": " ".join(f"{a}={b}" for a, b in cfg.items()), "candidates": tried, "validated": valid,
            "hbm": roofline("hbm", nbytes, flops, us), "mfma": roofline("mfma", nbytes, flops, us),
            "roofline": roofline("hbm", nbytes, flops, dom, measured_traffic("c5")), "algorithmic_bytes": nbytes,
            "algorithmic_flops": flops}

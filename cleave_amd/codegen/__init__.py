@@ -143,6 +143,7 @@ class HipCodeGen:
             "role": plan.role, "family": plan.family, "dtype": plan.dtype, "label": plan.label,
             "split": plan.split_factor, "tiling": plan.tiling,
             "params": [p.to_json() for p in params], "dyn_dims": list(plan.dyn_dims),
+            "derived_dims": [list(d) for d in plan.extra.get("derived_dims", ())],
             "out_idx": list(range(-n_out, 0)), "launches": unit.launches,
         }
         head = [MANIFEST_BEGIN] + ["// " + line for line in json.dumps(manifest, indent=1).splitlines()] + [MANIFEST_END]
@@ -269,8 +270,11 @@ class HipCodeGen:
         names = self._by_name(params)
         ins = [q for q in params if q.role in ("input", "scalar")]
         outs = [q for q in params if q.role == "output"]
-        dyn = tuple(plan.dyn_dims)
+        derived = tuple(name for name, _ in plan.extra.get("derived_dims", ()))
+        dyn = tuple(plan.dyn_dims) + derived
         dyn_c = tuple((plan.problem.get("dim_names") or {}).keys()) or None
+        if dyn_c is not None:
+            dyn_c += derived
         splits = plan.split_factor or 1
         part_roles = ("PM", "PL", "PO")
         if partial:
@@ -291,6 +295,10 @@ class HipCodeGen:
                 sig, entry, suffix = ins + outs, ENTRY, ""
             else:
                 sig, entry, suffix = [names[op[f"{r}_COMBINE"]] for r in part_roles] + outs, COMBINE_ENTRY, "_COMBINE"
+                if plan.tiling.get("CHUNK_PAGES"):
+                    sig = [names[op["INDPTR"]]] + sig
+            if plan.tiling.get("CHUNK_PAGES"):
+                unit.define("CL_CARG_INDPTR", op["INDPTR"])
             for r in part_roles:
                 unit.define(f"CL_CARG_{r}", op[r + suffix])
             unit.define("CL_CARG_OUT", op["OUT"])
@@ -319,6 +327,8 @@ class HipCodeGen:
         unit.define("CL_ROWS", rows)
         unit.define("CL_WAVES", waves)
         unit.define("CL_PREFETCH", int(t.get("PREFETCH", 1)))
+        chunk_pages = bool(t.get("CHUNK_PAGES", 0)) and paged and (plan.split_factor or 1) > 1
+        unit.define("CL_CHUNK_PAGES", chunk_pages)
         unit.define("CL_PAGED", paged)
         unit.define("CL_PAGE_SIZE", p.get("page_size", 1))
         unit.define("CL_KV_HEADS", p.get("kv_heads", 1))
@@ -337,8 +347,12 @@ class HipCodeGen:
         if partial:
             from ..schedule.policy import attn_lds_bytes
 
-            unit.launch(ENTRY, (f"({units}) * {row_tiles}", splits, 1), waves * 64, attn_lds_bytes(waves, p["vdim"]),
-                        self._partial_args)
+            if chunk_pages:
+                items = f"ceildiv({p['dim_names']['n_idx']}, chunk_pages) + {batch_name}"
+                grid = (items, 1, 1)
+            else:
+                grid = (f"({units}) * {row_tiles}", splits, 1)
+            unit.launch(ENTRY, grid, waves * 64, attn_lds_bytes(waves, p["vdim"]), self._partial_args)
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv({grid_rows} * {p['vdim'] // 4}, 256)", 1, 1), 256, 0, args)

@@ -1,7 +1,45 @@
 // ---- split-KV combine shared by the decode-attention kernels -------------------------------
 // Partials are (split, row[, d]) f32 with m the running max in the log2 domain, l the sum of
 // weights relative to m, and O the unnormalised weighted values.
-#if CL_SPLITS > 1 && CL_EMIT_COMBINE
+#ifndef CL_CHUNK_PAGES
+#define CL_CHUNK_PAGES 0
+#endif
+#if CL_CHUNK_PAGES && CL_EMIT_COMBINE
+// Combine of chunked items: request b owns items b + p0/C .. b + (p1-1)/C (p0, p1 its page-table
+// range); partials are (item, query head[, d]).  One thread per (request, head, 4 d).
+extern "C" __global__ void __launch_bounds__(256)
+CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
+  const i64 total = (i64)CL_TOTAL_ROWS * (CL_VDIM / 4);
+  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const i64 row = idx / (CL_VDIM / 4);
+  const int d = (int)(idx % (CL_VDIM / 4)) * 4;
+  const int req = (int)(row / CL_Q_HEADS), qh = (int)(row % CL_Q_HEADS);
+  int p0 = CL_CARG_INDPTR[req], p1 = CL_CARG_INDPTR[req + 1];
+  p0 = p0 < 0 ? 0 : (p0 > n_idx ? n_idx : p0);
+  p1 = p1 < 0 ? 0 : (p1 > n_idx ? n_idx : p1);
+  const int first = req + p0 / chunk_pages;
+  const int count = p1 > p0 ? (p1 - 1) / chunk_pages - p0 / chunk_pages + 1 : 0;
+  float m = CL_NEG_BIG;
+  for (int s = 0; s < count; ++s) m = fmaxf(m, CL_CARG_PM[(i64)(first + s) * CL_Q_HEADS + qh]);
+  float l = 0.f;
+  f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < count; ++s) {
+    const i64 prow = (i64)(first + s) * CL_Q_HEADS + qh;
+    const float f = fast_exp2(CL_CARG_PM[prow] - m);
+    l += CL_CARG_PL[prow] * f;
+    o += *reinterpret_cast<const f32x4*>(CL_CARG_PO + prow * CL_VDIM + d) * f;
+  }
+  const float inv = 1.0f / fmaxf(l, 1.0e-30f);
+  elem4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = to_elem(o[i] * inv);
+  *reinterpret_cast<elem4*>(CL_CARG_OUT + row * CL_VDIM + d) = r;
+#if CL_EMIT_LSE
+  if (d == 0) CL_CARG_LSE[row] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
+#endif
+}
+#elif CL_SPLITS > 1 && CL_EMIT_COMBINE
 // Combine: out[row] = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).  One thread per (row, 4 d).
 extern "C" __global__ void __launch_bounds__(256)
 CL_COMBINE_NAME(CL_COMBINE_PARAMS) {

@@ -20,7 +20,15 @@
 //   CL_SCALE_LOG2E softmax scale * log2(e) (dense; paged passes sm_scale at run time)
 //   CL_EMIT_LSE  also write the base-2 log-sum-exp
 //   CL_PREFETCH  steps of K/V in flight ahead of the one being computed (1 or 2)
+//   CL_CHUNK_PAGES  paged only, 0 = off.  1: work is cut into items of at most `chunk_pages`
+//                pages (a run-time argument, 1..64, chosen by the host from the table length)
+//                instead of a fixed number of splits per request, and a workgroup holds one wave
+//                per kv head, so that the eight waves together stream whole contiguous token
+//                rows of the cache and a long request costs many items rather than long ones.
 
+#ifndef CL_CHUNK_PAGES
+#define CL_CHUNK_PAGES 0
+#endif
 #define ATT_STEP 32
 #define ATT_KJ (CL_HEAD_DIM / 32)            // score MFMAs per 16 tokens
 #define ATT_VC ((CL_VDIM + 127) / 128)       // 128-wide value chunks
@@ -34,12 +42,23 @@ struct AttUnit {
   int kv_len;           // valid tokens
   int rows;             // real rows in this tile (1..16)
   const int* pages;     // paged: this request's slice of the page table
+  int page_reg;         // chunked items: lane i holds the (clamped) id of the slice's page i
   int n_pages;          // paged: entries in that slice (>= 1 when kv_len > 0)
   int pool_pages;       // paged: pages in the cache; page ids are clamped below this
   i64 out_row;          // flattened (unit, row) index of the tile's first row
 };
 
-#if CL_PAGED
+#if CL_PAGED && CL_CHUNK_PAGES
+// An item's page ids were read once into one register per lane; a token's page id comes from
+// the lane that holds it.  A page-table load per token would sit in the same in-order load
+// queue as the K/V rows and make every prefetch wait for the rows of the step before it.
+CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) {
+  int pi = t / CL_PAGE_SIZE;
+  pi = pi < u.n_pages ? pi : u.n_pages - 1;
+  const i64 page = __builtin_amdgcn_ds_bpermute(pi << 2, u.page_reg);
+  return (page * CL_PAGE_SIZE + (t % CL_PAGE_SIZE)) * u.row_stride;
+}
+#elif CL_PAGED
 CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) {
   int pi = t / CL_PAGE_SIZE;
   pi = pi < u.n_pages ? pi : u.n_pages - 1;
@@ -84,18 +103,72 @@ CL_DEVICE void att_load(const AttUnit& u, int t0, int c, int g, AttTile& tile) {
   }
 }
 
+#if CL_CHUNK_PAGES
+// Work items in page-table order: a new item starts at every multiple of chunk_pages table
+// entries and at every request boundary, so item t = (chunk w) + (request b) for the one pair
+// with chunk w overlapping request b.  Request b owns items b + p0/C .. b + (p1-1)/C.
+static_assert(CL_PAGED && CL_ROWS <= 16 && CL_WAVES == CL_KV_HEADS, "chunked items: one wave per kv head");
+CL_DEVICE int att_clamp_ptr(int p, int n_idx) { return p < 0 ? 0 : (p > n_idx ? n_idx : p); }
+#endif
+
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(CL_WAVES * 64)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
+#if CL_CHUNK_PAGES
+  const int split = 0, tile_id = 0;
+  const int item = blockIdx.x;
+#else
   const int split = blockIdx.y;
   const int tile_id = blockIdx.x % ATT_ROW_TILES;
   const int unit = blockIdx.x / ATT_ROW_TILES;
+#endif
 
   AttUnit u;
   u.rows = CL_ROWS - 16 * tile_id < 16 ? CL_ROWS - 16 * tile_id : 16;
-#if CL_PAGED
+#if CL_CHUNK_PAGES
+  // the request whose items include `item`: the last b with b + indptr[b] / C <= item
+  int req = 0;
+  {
+    int hi_b = batch - 1;
+    while (req < hi_b) {
+      const int mid = (req + hi_b + 1) >> 1;
+      if (mid + att_clamp_ptr(CL_ARG_INDPTR[mid], n_idx) / chunk_pages <= item) req = mid;
+      else hi_b = mid - 1;
+    }
+  }
+  const int head = wave;
+  const int p0 = att_clamp_ptr(CL_ARG_INDPTR[req], n_idx), p1 = att_clamp_ptr(CL_ARG_INDPTR[req + 1], n_idx);
+  const int chunk = item - req;
+  const int lo = p0 > chunk * chunk_pages ? p0 : chunk * chunk_pages;
+  const int hi = p1 < (chunk + 1) * chunk_pages ? p1 : (chunk + 1) * chunk_pages;
+  if (hi <= lo) return;                               // an index no (chunk, request) pair maps to
+  {
+    int lastp = CL_PAGE_SIZE;
+#if CL_PAGE_SIZE > 1
+    if (hi == p1) {
+      lastp = CL_ARG_LAST[req];
+      lastp = lastp > 0 ? (lastp < CL_PAGE_SIZE ? lastp : CL_PAGE_SIZE) : 0;
+    }
+#endif
+    u.kv_len = (hi - lo - 1) * CL_PAGE_SIZE + lastp;
+  }
+  u.pages = CL_ARG_INDICES + lo;
+  u.n_pages = hi - lo;
+  u.pool_pages = num_pages;
+  {
+    int pid = u.pages[lane < u.n_pages ? lane : u.n_pages - 1];
+    pid = pid < num_pages - 1 ? pid : num_pages - 1;
+    u.page_reg = pid > 0 ? pid : 0;
+  }
+  u.row_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
+  u.k = CL_ARG_K + (i64)head * CL_HEAD_DIM;
+  u.v = CL_ARG_V + (i64)head * CL_VDIM;
+  u.out_row = (i64)req * CL_Q_HEADS + (i64)head * CL_ROWS;
+  u.q = CL_ARG_Q + u.out_row * CL_HEAD_DIM;
+  const float scale2 = sm_scale * 1.4426950408889634f;
+#elif CL_PAGED
   // unit = request * kv_heads + kv head.  The request's length follows the page-granular
   // CSR: every page but the last is full, the last holds kv_last_page_len tokens, and the
   // sum is clamped to the pages the request owns.
@@ -118,6 +191,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
   u.kv_len = kv_len;
   u.pages = CL_ARG_INDICES + p0;
+  u.page_reg = 0;
   u.n_pages = n_pages;
   u.pool_pages = num_pages;
   u.row_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
@@ -128,6 +202,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const float scale2 = sm_scale * 1.4426950408889634f;
 #else
   u.kv_len = CL_SKV;
+  u.page_reg = 0;
   u.pages = nullptr;
   u.n_pages = 0;
   u.pool_pages = 0;
@@ -141,10 +216,15 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 
   // This split's steps: ceil(n_steps / SPLITS) each; a trailing split may own none.
   const int n_steps = (u.kv_len + ATT_STEP - 1) / ATT_STEP;
+#if CL_CHUNK_PAGES
+  const int step_begin = 0, step_end = n_steps;      // the item is the unit of work: no further cut
+  (void)split;
+#else
   const int per_split = (n_steps + CL_SPLITS - 1) / CL_SPLITS;
   const int step_begin = split * per_split;
   int step_end = step_begin + per_split;
   step_end = step_end < n_steps ? step_end : n_steps;
+#endif
 
   // Query rows as the B operand: lane (c, g) holds Q[row c][32 j + 8 g .. +8]; padded rows are 0.
   elem8 qf[ATT_KJ];
@@ -171,27 +251,33 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // steps n+1 .. n+CL_PREFETCH are in flight.  The ring position is a compile-time constant of
   // the unrolled inner loop, so every tile stays in registers.
   AttTile ring[CL_PREFETCH + 1];
+#if CL_CHUNK_PAGES
+#define ATT_WSTRIDE 1                 // every wave walks all steps of the item for its own head
+  const int step0 = step_begin;
+#else
+#define ATT_WSTRIDE CL_WAVES
   const int step0 = step_begin + wave;
+#endif
   // Prefetch loads are issued unconditionally: a step past the end is clamped onto this wave's
   // last real step (an L2 hit, its tile is never consumed).  A branch around the loads would
   // make the hardware load counter differ between paths, and the waits the compiler then has
   // to insert drain the prefetch before every value product.
   int last_step = step0;
-  if (step_end > step0) last_step = step0 + ((step_end - 1 - step0) / CL_WAVES) * CL_WAVES;
+  if (step_end > step0) last_step = step0 + ((step_end - 1 - step0) / ATT_WSTRIDE) * ATT_WSTRIDE;
   if (step0 < step_end) {
 #pragma unroll
     for (int i = 0; i < CL_PREFETCH; ++i) {
-      int sidx = step0 + i * CL_WAVES;
+      int sidx = step0 + i * ATT_WSTRIDE;
       sidx = sidx < last_step ? sidx : last_step;
       att_load(u, sidx * ATT_STEP, c, g, ring[i]);
     }
   }
-  for (int base = step0; base < step_end; base += (CL_PREFETCH + 1) * CL_WAVES) {
+  for (int base = step0; base < step_end; base += (CL_PREFETCH + 1) * ATT_WSTRIDE) {
 #pragma unroll
     for (int r = 0; r <= CL_PREFETCH; ++r) {
-      const int step = base + r * CL_WAVES;
+      const int step = base + r * ATT_WSTRIDE;
       if (step >= step_end) break;
-      int ahead = step + CL_PREFETCH * CL_WAVES;
+      int ahead = step + CL_PREFETCH * ATT_WSTRIDE;
       ahead = ahead < last_step ? ahead : last_step;
       att_load(u, ahead * ATT_STEP, c, g, ring[(r + CL_PREFETCH) % (CL_PREFETCH + 1)]);
       const AttTile& cur = ring[r];
@@ -269,6 +355,21 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       }
   __syncthreads();
 
+#if CL_CHUNK_PAGES
+  // each wave owns one head: its rows leave through its own LDS slab, nothing is merged here
+  {
+    const i64 prow0 = (i64)item * CL_Q_HEADS + (i64)head * CL_ROWS;
+    for (int idx = lane; idx < CL_ROWS * (CL_VDIM / 4); idx += 64) {
+      const int row = idx / (CL_VDIM / 4), d = (idx % (CL_VDIM / 4)) * 4;
+      *reinterpret_cast<f32x4*>(CL_ARG_PO + (prow0 + row) * CL_VDIM + d) =
+          *reinterpret_cast<const f32x4*>(sh_o + (wave * 16 + row) * CL_VDIM + d);
+    }
+    if (lane < CL_ROWS) {
+      CL_ARG_PM[prow0 + lane] = sh_m[wave * 16 + lane];
+      CL_ARG_PL[prow0 + lane] = sh_l[wave * 16 + lane];
+    }
+  }
+#else
   for (int idx = threadIdx.x; idx < 16 * CL_VDIM; idx += CL_WAVES * 64) {
     const int row = idx / CL_VDIM, d = idx % CL_VDIM;
     if (row >= u.rows) continue;
@@ -298,6 +399,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
 #endif
   }
+#endif  // CL_CHUNK_PAGES
 }
 #endif  // CL_EMIT_PARTIAL
 

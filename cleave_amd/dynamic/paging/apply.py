@@ -38,6 +38,11 @@ class DenseAttention:
     accum_dtype: str = "float32"
     waves: int = 4
     split: int | None = None
+    prefetch: int = 1
+    # Non-zero: split-KV work is cut into items of at most this many pages (one wave per kv head,
+    # `waves` is then the kv-head count) instead of `split` equal parts per request.  -1 lets the
+    # launch choose the size from the page-table length so that one item lands on each compute unit.
+    chunk_pages: int = 0
 
 
 def read_dense_attention(plan: KernelPlan) -> DenseAttention:
@@ -126,9 +131,29 @@ def _paged_problem(spec: PagingSpec, dense: DenseAttention) -> dict:
 def _plan(spec, dense, role, params, operands, split=None) -> KernelPlan:
     dyn = (spec.batch_dim, spec.pages_dim, spec.index_dim)
     label = f"kv={dense.kv_tile} q={dense.query_rows} thr={dense.n_threads}"
-    return KernelPlan(template="attn_decode", role=role, family="attention", dtype=dense.dtype,
-                      problem=_paged_problem(spec, dense), tiling={"WAVES": dense.waves}, params=params,
+    tiling = {"WAVES": dense.waves, "PREFETCH": dense.prefetch}
+    extra = {}
+    if dense.chunk_pages and split:
+        tiling.update(WAVES=spec.num_kv_heads, CHUNK_PAGES=dense.chunk_pages)
+        extra["derived_dims"] = [("chunk_pages", chunk_pages_expr(spec, dense.chunk_pages))]
+    return KernelPlan(template="attn_decode", role=role, family="attention", dtype=dense.dtype, extra=extra,
+                      problem=_paged_problem(spec, dense), tiling=tiling, params=params,
                       operands=operands, split_factor=split, dyn_dims=dyn, n_threads=dense.n_threads, label=label)
+
+
+MAX_CHUNK_PAGES = 64      # an item's page ids live in one register per lane of a wave
+
+
+def chunk_pages_expr(spec, chunk_pages: int) -> str:
+    """The launch-time expression for the item size: the fixed value, or for -1 the size that
+    spreads the table over the machine's compute units (each request boundary adds an item)."""
+    if chunk_pages > 0:
+        return str(min(chunk_pages, MAX_CHUNK_PAGES))
+    from ...core.target import current_target
+
+    cus = current_target().arch.compute_units
+    return (f"max(1, min({MAX_CHUNK_PAGES}, ceildiv({spec.index_dim}, "
+            f"max(1, {cus} - {spec.batch_dim}))))")
 
 
 def apply_paging(plan: KernelPlan, spec) -> KernelPlan:
@@ -153,13 +178,26 @@ def build_split_decode(spec, dense: DenseAttention, split: int, comb: CombineTil
     b, h, d = spec.batch_dim, spec.num_qo_heads, dense.head_dim
     # split-major partials: one request's splits sit one stride apart
     # (python/cleave/dynamic/paging/tensor_maps.py:41-69)
-    bufs = [("PM", (split, b, h)), ("PL", (split, b, h)), ("PO", (split, b, h, d))]
+    if dense.chunk_pages:
+        if dense.chunk_pages < -1 or dense.chunk_pages > MAX_CHUNK_PAGES or dense.query_rows > 16 \
+                or spec.num_kv_heads > 16:
+            raise UnsupportedTiling(f"chunked items need chunk_pages in 1..{MAX_CHUNK_PAGES} (or -1), one 16-row "
+                                    "query tile and at most 16 kv heads")
+        # one partial per work item: a new item at every chunk_pages table entries and every request
+        items = f"ceildiv({spec.index_dim}, chunk_pages) + {b}"
+        bufs = [("PM", (items, h)), ("PL", (items, h)), ("PO", (items, h, d))]
+    else:
+        bufs = [("PM", (split, b, h)), ("PL", (split, b, h)), ("PO", (split, b, h, d))]
     part_outs = [ParamSpec(f"OutputNode_{i}", "float32", shape, "output") for i, (_, shape) in enumerate(bufs)]
     part_ops = {**operands, **{name: p.name for (name, _), p in zip(bufs, part_outs)}}
     partial = _plan(spec, dense, "partial", params + part_outs, part_ops, split)
     comb_ins = [ParamSpec(f"PlaceHolder_{name}", "float32", shape, "input") for name, shape in bufs]
     outs, out_ops = _paged_outputs(spec, dense)
     comb_ops = {**{name: p.name for (name, _), p in zip(bufs, comb_ins)}, **out_ops}
+    if dense.chunk_pages:         # the combine finds a request's items from the page-table offsets
+        indptr = next(q for q in params if q.name == operands["INDPTR"])
+        comb_ins.append(indptr)
+        comb_ops["INDPTR"] = indptr.name
     combine = _plan(spec, dense, "combine", comb_ins + outs, comb_ops, split)
     return [partial, combine]
 

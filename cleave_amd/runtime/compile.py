@@ -172,6 +172,10 @@ class CompiledKernel:
                 if not isinstance(want, int) and not str(want).isidentifier():
                     if eval_extent(want, dims) != int(got):
                         raise ValueError(f"{p.name}: extent {want} should be {eval_extent(want, dims)}, got {got}")
+        # extents the generator derives from the inferred ones (a work-item size chosen from the
+        # table length, say): evaluated in order, passed to the kernels like any other extent
+        for name, expr in self.manifest.get("derived_dims", ()):
+            dims[name] = eval_extent(expr, dims)
         missing = [d for d in self.dyn_dims if d not in dims]
         if missing:
             raise ValueError(f"run-time dims {missing} could not be inferred from the arguments")
