@@ -164,8 +164,7 @@ template <int COLS> struct GmPickTransposed<COLS, true> { typedef GmTransposedHa
 // LDS reads issued under the cover of row `i` of 32-wide k block `s` (see GM_COMPUTE).
 constexpr int gm_reads_after(int s, int i) {
   int n = 0;
-  if (GM_TM > 2 && i + 2 < GM_TM) ++n;
-  if (s == 0 && i + 2 >= GM_TM && i + 2 - GM_TM < (GM_TM < 2 ? GM_TM : 2)) ++n;
+  if (s * GM_TM + i + 2 < 2 * GM_TM) ++n;
   if (s == 0)
     for (int j = 0; j < GM_TN; ++j)
       if (j % GM_TM == i) ++n;
@@ -299,22 +298,22 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     elem8 af[2][GM_TM], bf[2][GM_TN];                                                                     \
     _Pragma("unroll") for (int j = 0; j < GM_TN; ++j) bf[0][j] = GM_BFRAG(0, j);                         \
     af[0][0] = GM_AFRAG(0, 0);                                                                            \
-    if (GM_TM > 1) af[0][1 % GM_TM] = GM_AFRAG(0, 1 % GM_TM);                                             \
+    af[1 / GM_TM][1 % GM_TM] = GM_AFRAG(1 / GM_TM, 1 % GM_TM);                                            \
     _Pragma("unroll") for (int s = 0; s < 2; ++s) {                                                      \
       _Pragma("unroll") for (int i = 0; i < GM_TM; ++i) {                                                \
         /* rows of the MFMA result follow its first operand: feeding B first leaves each lane */         \
         /* with four consecutive columns of one row of C */                                              \
         _Pragma("unroll") for (int j = 0; j < GM_TN; ++j) acc[i][j] = mfma16(bf[s][j], af[s][i], acc[i][j]); \
-        if (GM_TM > 2 && i + 2 < GM_TM) af[s][(i + 2) % GM_TM] = GM_AFRAG(s, (i + 2) % GM_TM);            \
-        if (s == 0 && i + 2 >= GM_TM && i + 2 - GM_TM < (GM_TM < 2 ? GM_TM : 2))                          \
-          af[1][(i + 2 - GM_TM) % GM_TM] = GM_AFRAG(1, (i + 2 - GM_TM) % GM_TM);                          \
+        /* the A fragments form one sequence over both k blocks, read two ahead of their use */          \
+        if (s * GM_TM + i + 2 < 2 * GM_TM)                                                                \
+          af[(s * GM_TM + i + 2) / GM_TM][(i + 2) % GM_TM] = GM_AFRAG((s * GM_TM + i + 2) / GM_TM, (i + 2) % GM_TM); \
         if (s == 0) {                                                                                     \
           _Pragma("unroll") for (int j = 0; j < GM_TN; ++j)                                              \
             if (j % GM_TM == i) bf[1][j] = GM_BFRAG(1, j);                                                \
         }                                                                                                 \
       }                                                                                                   \
     }                                                                                                     \
-    __builtin_amdgcn_sched_group_barrier(0x100, GM_TN + (GM_TM > 1 ? 2 : 1), 0);                          \
+    __builtin_amdgcn_sched_group_barrier(0x100, GM_TN + 2, 0);                                            \
     gm_sched_rows<0, 0>();                                                                                \
   }
 

@@ -27,7 +27,10 @@ def _check(program, make_inputs, shapes, **kw):
 
 
 GEMM_TILES = [dict(BM=32, BN=32, BK=64, WM=1, WN=1), dict(BM=64, BN=64, BK=64, WM=2, WN=2),
-              dict(BM=128, BN=128, BK=64, WM=2, WN=2)]
+              dict(BM=128, BN=128, BK=64, WM=2, WN=2),
+              # one 16-row operand tile per wave along M (and along both axes)
+              dict(BM=16, BN=32, BK=64, WM=1, WN=2, GDEPTH=2), dict(BM=16, BN=16, BK=64, WM=1, WN=1, GDEPTH=1),
+              dict(BM=32, BN=32, BK=64, WM=2, WN=2, GDEPTH=2), dict(BM=16, BN=64, BK=64, WM=1, WN=1)]
 
 
 @pytest.mark.parametrize("tiling", GEMM_TILES, ids=lambda t: "x".join(str(v) for v in t.values()))

@@ -15,7 +15,7 @@ from oracle import paged_oracle, program_oracle
 from tests import _cases as C
 
 pytestmark = pytest.mark.gpu
-SHAPES = dict(M=128, N=128, K=256)
+SHAPES = dict(M=128, N=128, K=512)   # K / 8 splits is still a whole 64-wide step
 FAST = dict(schedule=P.ScheduleConfig(topk=3), eval=P.EvalConfig(warmup=2, iters=20, max_parallel=2))
 
 
