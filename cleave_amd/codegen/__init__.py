@@ -362,12 +362,21 @@ class HipCodeGen:
         total_rows = p["batch"] * p["heads"]
         emit_lse = bool(p.get("emit_lse"))
         self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], total_rows, emit_lse)
-        waves = int(t.get("WAVES", 4))
-        if p["heads"] % (16 * waves):
-            raise CodegenError(f"{p['heads']} heads do not divide into {waves} waves of 16")
+        waves, hg = int(t.get("WAVES", 4)), int(t.get("HG", 1))
+        if p["heads"] % (16 * hg * waves):
+            raise CodegenError(f"{p['heads']} heads do not divide into {waves} waves of {16 * hg}")
+        if p["ckv"] % 64 or p["kpe"] % 64:
+            raise CodegenError("the MLA template stages 64-feature panels: latent and rope widths must be multiples of 64")
         for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_SKV", p["skv"]),
-                     ("CL_WAVES", waves), ("CL_BATCH", p["batch"])):
+                     ("CL_WAVES", waves), ("CL_HG", hg), ("CL_BATCH", p["batch"])):
             unit.define(k, v)
+        if "LDS_AHEAD" in t:
+            unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
+        for k in t:
+            if k.startswith("DBG_"):
+                unit.define(f"CL_{k}", 1)
+        # split partials of this family are stored in the element type (normalised per split)
+        unit.define("CL_PO_ELEM", 1)
         unit.define("CL_SCALE_LOG2E", _f(float(p["scale"]) * LOG2E))
         for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE")):
             if role in op:
@@ -377,11 +386,11 @@ class HipCodeGen:
         if partial:
             from ..schedule.policy import mla_lds_bytes
 
-            grid = (p["batch"] * (p["heads"] // (16 * waves)), splits, 1)
+            grid = (p["batch"] * (p["heads"] // (16 * hg * waves)), splits, 1)
             unit.launch(ENTRY, grid, waves * 64, mla_lds_bytes(p["ckv"], p["kpe"]), self._partial_args)
         if combine:
             entry, args = self._combine_args
-            unit.launch(entry, (-(-(total_rows * (p["ckv"] // 4)) // 256), 1, 1), 256, 0, args)
+            unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)
 
 
 def parse_manifest(source: str) -> dict:

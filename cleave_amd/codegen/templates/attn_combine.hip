@@ -4,6 +4,9 @@
 #ifndef CL_CHUNK_PAGES
 #define CL_CHUNK_PAGES 0
 #endif
+#ifndef CL_PO_ELEM
+#define CL_PO_ELEM 0
+#endif
 #if CL_CHUNK_PAGES && CL_EMIT_COMBINE
 // Combine of chunked items: request b owns items b + p0/C .. b + (p1-1)/C (p0, p1 its page-table
 // range); partials are (item, query head[, d]).  One thread per (request, head, 4 d).
@@ -35,6 +38,47 @@ CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) r[i] = to_elem(o[i] * inv);
   *reinterpret_cast<elem4*>(CL_CARG_OUT + row * CL_VDIM + d) = r;
+#if CL_EMIT_LSE
+  if (d == 0) CL_CARG_LSE[row] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
+#endif
+}
+#elif CL_SPLITS > 1 && CL_EMIT_COMBINE && CL_PO_ELEM
+// Combine of partials whose values are stored in the element type (normalised per split, m the
+// split's log-sum-exp, l = 1, or 0 with zero values for an empty split): the same rule as below,
+// out[row] = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m).
+// One thread per (row, 8 d): 16-byte loads.
+extern "C" __global__ void __launch_bounds__(256)
+CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
+  const i64 total = (i64)CL_TOTAL_ROWS * (CL_VDIM / 8);
+  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const i64 row = idx / (CL_VDIM / 8);
+  const int d = (int)(idx % (CL_VDIM / 8)) * 8;
+  float ms[CL_SPLITS];
+  float m = CL_NEG_BIG;
+#pragma unroll
+  for (int s = 0; s < CL_SPLITS; ++s) {
+    ms[s] = CL_CARG_PM[(i64)s * CL_TOTAL_ROWS + row];
+    m = fmaxf(m, ms[s]);
+  }
+  float l = 0.f;
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+#pragma unroll
+  for (int s = 0; s < CL_SPLITS; ++s) {
+    const i64 prow = (i64)s * CL_TOTAL_ROWS + row;
+    const float f = fast_exp2(ms[s] - m);
+    l += CL_CARG_PL[prow] * f;
+    const elem8 v = as_elem8(ld16(CL_CARG_PO + prow * CL_VDIM + d));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] += to_f32(v[i]) * f;
+  }
+  const float inv = 1.0f / fmaxf(l, 1.0e-30f);
+  elem8 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = to_elem(o[i] * inv);
+  st16(CL_CARG_OUT + row * CL_VDIM + d, as_u32x4(r));
 #if CL_EMIT_LSE
   if (d == 0) CL_CARG_LSE[row] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
 #endif

@@ -53,15 +53,16 @@ CL_DEVICE u32x4 as_u32x4(elem8 v) { return __builtin_bit_cast(u32x4, v); }
 // In-register 8x8 transpose of 16-bit elements.  in[e] holds row e (eight columns); out[j]
 // receives column j (eight rows).  Row-major global tensors hand a lane eight neighbours of
 // the *minor* axis per 16-byte load, while a matrix-core operand wants eight neighbours of
-// the contraction axis: this turns one into the other without touching LDS.
+// the contraction axis: this turns one into the other without touching LDS (32 byte-permutes).
 CL_DEVICE void transpose8x8(const u32x4 (&in)[8], u32x4 (&out)[8]) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {      // column pair (2q, 2q+1) lives in dword q of every row
 #pragma unroll
     for (int p = 0; p < 4; ++p) {    // row pair (2p, 2p+1) becomes dword p of the output
+      // one byte-permute each: bytes 0-3 of the selector's source pair are x, bytes 4-7 are y
       u32 x = in[2 * p][q], y = in[2 * p + 1][q];
-      out[2 * q][p] = (x & 0xffffu) | (y << 16);
-      out[2 * q + 1][p] = (x >> 16) | (y & 0xffff0000u);
+      out[2 * q][p] = __builtin_amdgcn_perm(y, x, 0x05040100u);      // (x & 0xffff) | (y << 16)
+      out[2 * q + 1][p] = __builtin_amdgcn_perm(y, x, 0x07060302u);  // (x >> 16) | (y & 0xffff0000)
     }
   }
 }

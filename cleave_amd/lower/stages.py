@@ -37,7 +37,7 @@ def to_ir(structure, symbol_map=None, dtype="float16", out_dtype=None, input_nam
 def partial_buffers(low: Lowered, factor: int) -> list:
     """``[(name, shape, dtype)]`` of what a split partial writes and its combine reads, split-major
     like the reference's ``(split, batch, heads[, D])`` layout
-    (``python/cleave/dynamic/paging/tensor_maps.py:41-69``); always f32 here."""
+    (``python/cleave/dynamic/paging/tensor_maps.py:41-69``); f32 except the MLA value partials."""
     p = low.problem
     if low.family in ("matmul", "rmsnorm_matmul"):
         batch = max(p["batch_A"], p["batch_B"])
@@ -48,7 +48,12 @@ def partial_buffers(low: Lowered, factor: int) -> list:
     if low.family == "attention":
         rows, width = p["units"] * p["group"] * p["sq"], p["vdim"]
     elif low.family == "mla":
+        # every split covers all heads of a batch entry, so the value partials are as large as
+        # `factor` outputs: they are kept in the element type, normalised per split, with the
+        # split's log-sum-exp in PM and PL = 1 (the reference's partials are in the element type too)
         rows, width = p["batch"] * p["heads"], p["ckv"]
+        return [("PM", (factor, rows), "float32"), ("PL", (factor, rows), "float32"),
+                ("PO", (factor, rows, width), low.dtype)]
     else:
         raise LoweringRejected(f"family {low.family!r} has no split form")
     return [("PM", (factor, rows), "float32"), ("PL", (factor, rows), "float32"),

@@ -88,9 +88,11 @@ def publish_reference(reference_cache_dir, graph, dtype, device: str = "cuda"):
 
 
 def compare_mode(graph) -> str:
-    """How a stage's raw outputs are compared.  Softmax partials (m, l, O) are unnormalised sums
-    whose low-order bits depend on the order the running maximum was met in, so they are
-    compared as (m, l, O / l): the quantities the combine actually consumes."""
+    """How a stage's raw outputs are compared.  Softmax partials (m, l, O) are sums relative to a
+    reference point m that a kernel is free to choose (the running maximum, a maximum raised
+    only in coarse steps, or the log-sum-exp itself with l = 1 and normalised values), so they
+    are compared as (m + log2 l, O / l): the quantities that do not depend on that choice and
+    that the combine actually consumes."""
     low = getattr(graph, "lowered", None)
     if low is not None and getattr(graph, "role", "main") == "partial" and low.family in ("attention", "mla"):
         return "softmax_partial"
@@ -100,8 +102,11 @@ def compare_mode(graph) -> str:
 def _comparable(outputs, mode):
     if mode != "softmax_partial":
         return list(outputs)
+    import torch
+
     pm, pl, po = (t.float() for t in outputs)
-    return [pm, pl, po / pl.clamp_min(1e-30).unsqueeze(-1)]
+    lse = torch.where(pl > 0, pm + torch.log2(pl.clamp_min(1e-30)), torch.full_like(pm, -1.0e30))
+    return [lse, po / pl.clamp_min(1e-30).unsqueeze(-1)]
 
 
 def _load_reference(reference_cache_dir, device: str = "cuda", with_mode: bool = False):

@@ -204,12 +204,14 @@ def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
 
 # ----------------------------------------------------------------------------- MLA decode
 def mla_lds_bytes(ckv, kpe):
-    return 2 * (32 * (ckv + kpe + 8) + ckv * (32 + 8)) * 2
+    """Two stages of the token-major tile ((ckv + kpe) / 64 panels of 32 x 64) and of the
+    feature-major copy (ckv / 2 rows of 64), two bytes per element."""
+    return 2 * (((ckv + kpe) // 64) * 32 * 64 + (ckv // 2) * 64) * 2
 
 
 def mla_ok(low) -> bool:
     p = low.problem
-    return p["heads"] % 16 == 0 and p["ckv"] % 32 == 0 and p["kpe"] % 32 == 0 and p["ckv"] % 16 == 0
+    return p["heads"] % 16 == 0 and p["ckv"] % 64 == 0 and p["kpe"] % 64 == 0
 
 
 def mla_candidates(low, role, factor, arch: Arch):
@@ -219,28 +221,36 @@ def mla_candidates(low, role, factor, arch: Arch):
     if lds > arch.lds_bytes:
         return []
     out = []
-    groups16 = p["heads"] // 16
-    for waves in (1, 2, 4, 8):
-        if groups16 % waves:
+    d = p["ckv"] + p["kpe"]
+    for waves, hg in itertools.product((1, 2, 4, 8), (1, 2)):
+        heads_per_block = 16 * hg * waves
+        if p["heads"] % heads_per_block:
             continue
-        vgprs = (p["ckv"] + p["kpe"]) // 32 * 4 + p["ckv"] // 16 * 4 + 40 + 48
+        # Q fragments and accumulators of a wave's heads stay in registers for the whole split
+        # (plus a step's staging registers, the ring of LDS operand reads and the softmax state)
+        vgprs = hg * (d // 32 * 4 + p["ckv"] // 16 * 4) + 36 + 32 + 48
         if vgprs > arch.vgprs_per_lane:
             continue
-        blocks = p["batch"] * (groups16 // waves) * splits
+        blocks = p["batch"] * (p["heads"] // heads_per_block) * splits
         per_cu = arch.blocks_per_cu(waves * 64, lds, vgprs)
         if per_cu < 1:
             continue
         passes = _waves_time(blocks, per_cu, arch)
         steps = _ceil(_ceil(p["skv"], 32), splits)
-        # per step and wave: 2*(D/32) + ckv/16 matrix-core issues of 16 clocks; LDS operand reads
-        # of every wave share one 128 B/clk port
-        mfma_clk = (2 * (p["ckv"] + p["kpe"]) // 32 + p["ckv"] // 16) * 16 * _ceil(waves, 4)
-        lds_clk = waves * (32 * (p["ckv"] + p["kpe"]) + 32 * p["ckv"]) * 2 / 128.0
-        load_clk = 32 * (p["ckv"] + p["kpe"]) * 2 / 24.0
-        step_clk = max(mfma_clk, lds_clk, load_clk) + 200
+        # per step: every wave reads the whole tile and its transposed copy from LDS once (one
+        # 128 B/clk port per CU) and issues hg matrix ops of 16 clocks per 1 KiB operand read;
+        # the staging writes both images once per workgroup
+        operand_reads = 2 * (d // 32) + p["ckv"] // 16
+        mfma_clk = operand_reads * hg * 16 * _ceil(waves, 4)
+        lds_clk = (waves * operand_reads * 1024 + 32 * (d + p["ckv"]) * 2) / 128.0
+        load_clk = 32 * d * 2 / 24.0
+        step_clk = max(mfma_clk, lds_clk, load_clk) + 400
         util = min(1.0, blocks / (per_cu * arch.compute_units))
-        score = passes * steps * step_clk * (1.0 + 0.3 * (1 - util)) + 3000
-        out.append(TileDict("mla_decode", role, dict(WAVES=waves), output_tile=[16 * waves, p["ckv"]],
+        # split partials go out and come back once (element type): 2 * splits * rows * ckv * 2 bytes
+        partial_clk = (4 * splits * p["batch"] * p["heads"] * p["ckv"]) / (arch.hbm_gbps * 1e3 * 0.6) * 2400 \
+            if splits > 1 else 0.0
+        score = passes * steps * step_clk * (1.0 + 0.3 * (1 - util)) + 3000 + partial_clk
+        out.append(TileDict("mla_decode", role, dict(WAVES=waves, HG=hg), output_tile=[heads_per_block, p["ckv"]],
                             rstep_map={"kv": 32}, n_threads=waves * 64, split_factor=factor, score=score,
                             lds_bytes=lds, est_vgprs=vgprs))
     return out

@@ -122,9 +122,31 @@ def test_mla_decode_small(split):
     _check(fn.trace(dt, **C.SMALL["c4"]), mk, C.SMALL["c4"], template="mla_decode", tiling=dict(WAVES=1), split=split)
     shapes = dict(B=2, H=64, D=512, PE=64, SKV=160)
     _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=4), split=split)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=2, HG=2), split=split)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=1, HG=2), split=split)
 
 
-@pytest.mark.parametrize("split", [4, 8])
-def test_mla_decode_c4_full(split):
+def test_mla_decode_rising_maximum():
+    """Scores that keep growing along the KV axis force the running maximum up in steps of
+    more than 8 (log2 domain) several times per split: the deferred rescale must stay exact."""
     fn, dt, mk = C.CASES["c4"]
-    _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=dict(WAVES=4), split=split)
+    shapes = dict(B=1, H=32, D=512, PE=64, SKV=512)
+    prog = fn.trace(dt, **shapes)
+    q, kv, q_pe, k_pe = mk(shapes, device="cpu")
+    ramp = torch.linspace(0.2, 6.0, shapes["SKV"]).reshape(1, -1, 1)
+    kv = (kv.float() * 0.2 + ramp * torch.sign(q.float().mean(dim=(1,), keepdim=True))).to(kv.dtype)
+    ins = [q, kv, q_pe, k_pe]
+    want = po.evaluate(prog, ins)[0]
+    for tiling, split in ((dict(WAVES=2, HG=1), None), (dict(WAVES=1, HG=2), 2)):
+        kernel = kernel_for(prog, template="mla_decode", tiling=tiling, split=split)
+        print(f"case mla rising maximum {tiling} split={split}", flush=True)
+        got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("tiling,split", [(dict(WAVES=4, HG=1), 8), (dict(WAVES=8, HG=1), 16), (dict(WAVES=4, HG=2), 16),
+                                          (dict(WAVES=4, HG=2), 4)],
+                         ids=lambda v: "x".join(str(x) for x in v.values()) if isinstance(v, dict) else str(v))
+def test_mla_decode_c4_full(tiling, split):
+    fn, dt, mk = C.CASES["c4"]
+    _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=tiling, split=split)
