@@ -114,7 +114,7 @@ class HipCodeGen:
         """Partial and combine in one unit: the partial's outputs become scratch parameters."""
         if partial.role != "partial" or combine.role != "combine":
             raise CodegenError("a fused pair is [partial, combine]")
-        if partial.template != combine.template and not {partial.template, combine.template} <= {"gemm", "skinny"}:
+        if partial.template != combine.template and not {partial.template, combine.template} <= {"gemm", "gemm_dma", "skinny"}:
             raise CodegenError(f"partial ({partial.template}) and combine ({combine.template}) templates differ")
         params = [p for p in partial.params if p.role in ("input", "scalar")]
         operands = dict(partial.operands)
@@ -235,6 +235,30 @@ class HipCodeGen:
             grid = (-(-p["N"] // tile["BN"]), -(-p["M"] // tile["BM"]), batch * splits)
             lds = gemm_lds_bytes(tile["BM"], tile["BN"], tile["BK"], plan.family == "rmsnorm_matmul")
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, lds, self._partial_args)
+        if combine:
+            entry, args, total = self._combine_args
+            unit.launch(entry, (-(-(total // 4) // 256), 1, 1), 256, 0, args)
+
+    def _emit_gemm_dma(self, unit, plan, params, partial, combine, fused):
+        p, t = plan.problem, plan.tiling
+        if plan.family != "matmul":
+            raise CodegenError("the direct-to-LDS matmul template has no fused RMSNorm form")
+        self._matmul_common(unit, plan, params, partial, combine, fused)
+        tile = dict(BM=128, BN=128, BK=64, WM=2, WN=2)
+        tile.update(t)
+        for k, v in tile.items():
+            unit.define(f"CL_{k}", v)
+        splits = plan.split_factor or 1
+        batch = max(p["batch_A"], p["batch_B"])
+        unit.templates.append("gemm_dma.hip")
+        if partial:
+            if tile["BK"] != 64 or p["K"] % (splits * 64):
+                raise CodegenError(f"K={p['K']} is not a multiple of splits*64={splits * 64}")
+            if (not p["trans_B"] and p["N"] % 8) or (p["trans_A"] and p["M"] % 8) or p["K"] % 8:
+                raise CodegenError("16-byte global chunks need the minor extent of each operand to be a multiple of 8")
+            grid = (-(-p["N"] // tile["BN"]), -(-p["M"] // tile["BM"]), batch * splits)
+            # the tile images are static LDS arrays of the kernel: no dynamic LDS at launch
+            unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, 0, self._partial_args)
         if combine:
             entry, args, total = self._combine_args
             unit.launch(entry, (-(-(total // 4) // 256), 1, 1), 256, 0, args)

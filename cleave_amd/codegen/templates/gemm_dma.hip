@@ -1,0 +1,324 @@
+// ---- LDS-tiled MFMA matmul with direct global->LDS loads: C[M, N] = A[M, K] * B[K, N] ---------
+//
+// A workgroup owns a BM x BN tile of C and walks K in steps of 64.  Both operand tiles go from
+// global memory straight into LDS (global_load_lds, 16 bytes per lane, no register staging, no
+// LDS store instructions); a lane chooses which 16-byte chunk it fetches, so the LDS image can
+// be swizzled although a wave's 1 KiB lands in lane order.  Two stages: while the matrix cores
+// work on one, the loads of the next step fill the other; one barrier per step.
+//
+// Tile images in LDS (the 16-byte chunk index of a row is XORed with a function of the row so
+// that the operand reads are free of bank conflicts):
+//   K-minor operand (A as (M,K), B as (N,K)):  [rows][64]   operand fragment = one ds_read_b128
+//   K-major operand (B as (K,N), A as (K,M)):  [64][cols]   operand fragment = two transposing
+//       reads (ds_read_b64_tr_b16): within 16 lanes, lane 4a+b receives element b of the 8-byte
+//       pieces addressed by lanes a, 4+a, 8+a, 12+a; the sixteen lanes address a 4(k) x 16(col)
+//       patch (lane j: row j/4, columns 4 (j%4)..+3), so lane c ends up with four consecutive k
+//       of column c.
+//
+//   CL_M CL_N CL_K  CL_BM CL_BN  CL_WM x CL_WN waves  CL_TRANS_A / CL_TRANS_B  CL_BATCH_A/B
+//   CL_SPLITS (split-K: f32 partial tiles to CL_ARG_PACC[split])  CL_GROUP_M (tile order patch)
+
+#define GD_WAVES (CL_WM * CL_WN)
+#define GD_THREADS (GD_WAVES * 64)
+#define GD_TM (CL_BM / CL_WM / 16)
+#define GD_TN (CL_BN / CL_WN / 16)
+#define GD_BK 64
+#define GD_BATCH (CL_BATCH_A > CL_BATCH_B ? CL_BATCH_A : CL_BATCH_B)
+#ifndef CL_GROUP_M
+#define CL_GROUP_M 4
+#endif
+#define GD_XCDS 8
+static_assert(CL_BK == 64, "K steps are 64 wide (128-byte K-minor rows)");
+static_assert((GD_TM & (GD_TM - 1)) == 0 && (GD_TN & (GD_TN - 1)) == 0, "wave tiles are powers of two");
+static_assert(CL_BM % 16 == 0 && CL_BN % 16 == 0, "tiles are multiples of 16");
+
+typedef __attribute__((address_space(3))) void gd_lds_void;
+typedef __attribute__((address_space(1))) const void gd_gbl_void;
+typedef short gd_s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) gd_s16x4 gd_lds_s16x4;
+
+// operand extents along the non-contraction axis and their LDS images (two stages each)
+#define GD_A_ELEMS (CL_BM * GD_BK)
+#define GD_B_ELEMS (CL_BN * GD_BK)
+__shared__ __attribute__((aligned(1024))) elem_t gd_a0[GD_A_ELEMS];
+__shared__ __attribute__((aligned(1024))) elem_t gd_a1[GD_A_ELEMS];
+__shared__ __attribute__((aligned(1024))) elem_t gd_b0[GD_B_ELEMS];
+__shared__ __attribute__((aligned(1024))) elem_t gd_b1[GD_B_ELEMS];
+
+// ---- K-minor image: row r at r * 64, chunk ch at slot ch ^ swz(r) ------------------------------
+CL_DEVICE int gd_swz_kmin(int row) { return ((row >> 1) ^ (row >> 3)) & 7; }
+
+// ---- K-major image: k row at k * COLS, chunk ch at slot ch ^ f(k); f is even so that the two
+// chunks of a 32-byte patch row stay neighbours.  The eight k rows a half wave reads together
+// (k = 4 t + i + 8 g', i < 4, g' < 2) get eight different bank positions.
+template <int COLS>
+CL_DEVICE int gd_swz_kmaj(int k) {
+  if (COLS >= 128) return 2 * ((k & 3) | (((k >> 3) & 1) << 2));
+  if (COLS == 64) return 2 * (((k >> 1) & 1) | (((k >> 3) & 1) << 1));
+  return 0;
+}
+
+// One operand of the product: how its tile is fetched and how fragments are read.
+//   EXT      tile extent along the operand's own axis (BM for A, BN for B)
+//   KMAJOR   stored with K as the major axis
+template <int EXT, bool KMAJOR>
+struct GdOperand {
+  static constexpr int CPR = EXT / 8;                          // K-major: chunks per k row
+  static constexpr int UNITS = EXT * GD_BK * 2 / 1024;         // 1 KiB wave loads per tile
+  static constexpr int PER = (UNITS + GD_WAVES - 1) / GD_WAVES;
+  u32 goff[PER];     // this lane's byte offset (from the tile's first element at k = 0) per unit
+
+  // ext0: first row/column of the tile, lim: tensor extent along that axis, pitch: elements
+  CL_METHOD void init(int ext0, int lim, int pitch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int u = wave + i * GD_WAVES;
+      if (!KMAJOR) {
+        const int r = 8 * u + (lane >> 3);
+        const int chunk = (lane & 7) ^ gd_swz_kmin(r);
+        int row = ext0 + r;
+        row = row < lim ? row : lim - 1;                        // rows past the edge repeat the last one
+        goff[i] = (u32)(((row - ext0) * pitch + 8 * chunk) * 2);
+      } else {
+        constexpr int RPU = 64 / CPR > 0 ? 64 / CPR : 1;        // k rows per unit
+        const int k = u * RPU + lane / CPR;
+        const int chunk = (lane % CPR) ^ gd_swz_kmaj<EXT>(k);
+        int col = ext0 + 8 * chunk;
+        col = col < lim - 8 ? col : lim - 8;                    // chunks past the edge repeat the last one
+        goff[i] = (u32)((k * pitch + (col - ext0)) * 2);
+      }
+    }
+  }
+
+  // issue this wave's loads of one K step; `base`: the tile's first element of this step (uniform)
+  CL_METHOD void issue(const elem_t* base, elem_t* lds) const {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: the LDS target goes to M0
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int u = wave + i * GD_WAVES;
+      if (UNITS % GD_WAVES == 0 || u < UNITS)
+        __builtin_amdgcn_global_load_lds((gd_gbl_void*)(reinterpret_cast<const char*>(base) + goff[i]),
+                                         (gd_lds_void*)(lds + u * 512), 16, 0, 0);
+    }
+  }
+};
+
+// fragment readers --------------------------------------------------------------------------------
+// K-minor: `off0` = element offset of (row ext_w + c, chunk g) for the wave's first 16-row tile
+CL_DEVICE elem8 gd_read_kmin(const elem_t* tile, int off0, int i, int s) {
+  // row 16 i + c: swizzle(16 i + c) = swizzle(c-part) ^ (2 i & 7); k block s: chunk + 4 s
+  return *reinterpret_cast<const elem8*>(tile + 16 * i * 64 + (off0 ^ (s * 32) ^ (((2 * i) & 7) << 3)));
+}
+// K-major: `off0` = element offset of this lane's 8-byte piece for tile j = 0, k block 0, t = 0
+template <int COLS>
+CL_DEVICE elem8 gd_read_kmaj(const elem_t* tile, int off0, int j, int s) {
+  const gd_lds_s16x4* p0 = (const gd_lds_s16x4*)(tile + ((off0 ^ (j << 4)) + (32 * s) * COLS));
+  const gd_lds_s16x4* p1 = (const gd_lds_s16x4*)(tile + ((off0 ^ (j << 4)) + (32 * s + 4) * COLS));
+  const gd_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(const_cast<gd_lds_s16x4*>(p0));
+  const gd_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(const_cast<gd_lds_s16x4*>(p1));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(elem8, v);
+}
+
+// LDS read instructions per fragment, and the reads issued under the cover of row `i` of k block
+// `s` in GD_COMPUTE
+#define GD_A_READS (CL_TRANS_A ? 2 : 1)
+#define GD_B_READS (CL_TRANS_B ? 1 : 2)
+constexpr int gd_reads_after(int s, int i) {
+  int n = 0;
+  if (s * GD_TM + i + 2 < 2 * GD_TM) n += GD_A_READS;
+  if (s == 0)
+    for (int j = 0; j < GD_TN; ++j)
+      if (j % GD_TM == i) n += GD_B_READS;
+  return n;
+}
+template <int S, int I>
+CL_DEVICE void gd_sched_rows() {
+  __builtin_amdgcn_sched_group_barrier(0x008, GD_TN, 0);
+  constexpr int n = gd_reads_after(S, I);
+  if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);
+  if constexpr (I + 1 < GD_TM) gd_sched_rows<S, I + 1>();
+  else if constexpr (S == 0) gd_sched_rows<1, 0>();
+}
+
+#if CL_EMIT_PARTIAL
+extern "C" __global__ void __launch_bounds__(GD_THREADS)
+CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int wm = wave / CL_WN, wn = wave % CL_WN;
+  // Workgroups are handed to the XCDs round-robin in launch order.  Renumber them so that the
+  // ones an XCD runs at the same time are neighbours in C: launch id L -> the (L / 8)-th tile of
+  // XCD (L % 8)'s contiguous share, tiles ordered in patches of CL_GROUP_M row-tiles.
+  constexpr int tiles_m = (CL_M + CL_BM - 1) / CL_BM, tiles_n = (CL_N + CL_BN - 1) / CL_BN;
+  constexpr int tiles = tiles_m * tiles_n;
+  int tile_id = blockIdx.y * tiles_n + blockIdx.x;
+  {
+    const int xcd = tile_id % GD_XCDS, nth = tile_id / GD_XCDS;
+    constexpr int share = tiles / GD_XCDS, extra = tiles % GD_XCDS;
+    tile_id = xcd * share + (xcd < extra ? xcd : extra) + nth;
+  }
+  constexpr int group_m = CL_GROUP_M < tiles_m ? CL_GROUP_M : tiles_m;
+  const int band = tile_id / (group_m * tiles_n);
+  const int band_rows = (tiles_m - band * group_m) < group_m ? (tiles_m - band * group_m) : group_m;
+  const int in_band = tile_id - band * group_m * tiles_n;
+  const int m0 = (band * group_m + in_band % band_rows) * CL_BM, n0 = (in_band / band_rows) * CL_BN;
+  const int batch = blockIdx.z / CL_SPLITS, split = blockIdx.z % CL_SPLITS;
+  constexpr int k_per_split = CL_K / CL_SPLITS;
+  const int k_begin = split * k_per_split;
+  constexpr int KT = k_per_split / GD_BK;
+
+  const elem_t* A = CL_ARG_A + (i64)(batch / (GD_BATCH / CL_BATCH_A)) * CL_M * CL_K;
+  const elem_t* B = CL_ARG_B + (i64)(batch / (GD_BATCH / CL_BATCH_B)) * CL_K * CL_N;
+
+  // ---- operand movers: tile origin at K step 0 and the uniform advance per step ---------------
+  GdOperand<CL_BM, CL_TRANS_A != 0> opa;
+  GdOperand<CL_BN, CL_TRANS_B == 0> opb;
+#if CL_TRANS_A
+  opa.init(m0, CL_M, CL_M);                                   // A stored (K, M)
+  const elem_t* a_base = A + (i64)k_begin * CL_M + m0;
+  constexpr i64 a_step = (i64)GD_BK * CL_M;
+#else
+  opa.init(m0, CL_M, CL_K);                                   // A stored (M, K)
+  const elem_t* a_base = A + (i64)m0 * CL_K + k_begin;
+  constexpr i64 a_step = GD_BK;
+#endif
+#if CL_TRANS_B
+  opb.init(n0, CL_N, CL_K);                                   // B stored (N, K)
+  const elem_t* b_base = B + (i64)n0 * CL_K + k_begin;
+  constexpr i64 b_step = GD_BK;
+#else
+  opb.init(n0, CL_N, CL_N);                                   // B stored (K, N)
+  const elem_t* b_base = B + (i64)k_begin * CL_N + n0;
+  constexpr i64 b_step = (i64)GD_BK * CL_N;
+#endif
+
+  // ---- this lane's fragment offsets -------------------------------------------------------------
+  const int am = wm * (CL_BM / CL_WM), bn = wn * (CL_BN / CL_WN);   // wave origin inside the tile
+#if CL_TRANS_A
+  const int a_f = gd_swz_kmaj<CL_BM>(8 * g + (c >> 2));
+  const int a_off = (8 * g + (c >> 2)) * CL_BM + 8 * (((am / 8) ^ a_f) + ((c & 3) >> 1)) + 4 * (c & 1);
+#define GD_AFRAG(tile, i, s) gd_read_kmaj<CL_BM>(tile, a_off, i, s)
+#else
+  const int a_off = (am + c) * 64 + ((g ^ gd_swz_kmin(am + c)) << 3);
+#define GD_AFRAG(tile, i, s) gd_read_kmin(tile, a_off, i, s)
+#endif
+#if CL_TRANS_B
+  const int b_off = (bn + c) * 64 + ((g ^ gd_swz_kmin(bn + c)) << 3);
+#define GD_BFRAG(tile, j, s) gd_read_kmin(tile, b_off, j, s)
+#else
+  const int b_f = gd_swz_kmaj<CL_BN>(8 * g + (c >> 2));
+  const int b_off = (8 * g + (c >> 2)) * CL_BN + 8 * (((bn / 8) ^ b_f) + ((c & 3) >> 1)) + 4 * (c & 1);
+#define GD_BFRAG(tile, j, s) gd_read_kmaj<CL_BN>(tile, b_off, j, s)
+#endif
+
+  f32x4 acc[GD_TM][GD_TN];
+#pragma unroll
+  for (int i = 0; i < GD_TM; ++i)
+#pragma unroll
+    for (int j = 0; j < GD_TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // Matrix-core work of one step on one stage, software-pipelined: the B fragments of a 32-wide
+  // k block stay in registers, the A fragments stream two ahead of their use, and the next k
+  // block's B fragments arrive spread over the rows of the current one.  Rows of the MFMA result
+  // follow its first operand, so feeding B first leaves each lane with four consecutive columns
+  // of one row of C.  The group barriers pin the order "GD_TN matrix ops, then the reads issued
+  // under their cover" so that no LDS latency is waited for with the matrix cores idle.
+#define GD_COMPUTE(a_tile, b_tile)                                                                  \
+  {                                                                                                 \
+    elem8 af[2][GD_TM], bf[2][GD_TN];                                                               \
+    _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) bf[0][j] = GD_BFRAG(b_tile, j, 0);           \
+    af[0][0] = GD_AFRAG(a_tile, 0, 0);                                                              \
+    af[1 / GD_TM][1 % GD_TM] = GD_AFRAG(a_tile, 1 % GD_TM, 1 / GD_TM);                              \
+    _Pragma("unroll") for (int s = 0; s < 2; ++s) {                                                \
+      _Pragma("unroll") for (int i = 0; i < GD_TM; ++i) {                                          \
+        _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) acc[i][j] = mfma16(bf[s][j], af[s][i], acc[i][j]); \
+        if (s * GD_TM + i + 2 < 2 * GD_TM)                                                          \
+          af[(s * GD_TM + i + 2) / GD_TM][(i + 2) % GD_TM] =                                        \
+              GD_AFRAG(a_tile, (i + 2) % GD_TM, (s * GD_TM + i + 2) / GD_TM);                       \
+        if (s == 0) {                                                                               \
+          _Pragma("unroll") for (int j = 0; j < GD_TN; ++j)                                        \
+            if (j % GD_TM == i) bf[1][j] = GD_BFRAG(b_tile, j, 1);                                  \
+        }                                                                                           \
+      }                                                                                             \
+    }                                                                                               \
+    __builtin_amdgcn_sched_group_barrier(0x100, GD_B_READS * GD_TN + 2 * GD_A_READS, 0);            \
+    gd_sched_rows<0, 0>();                                                                          \
+  }
+  // everything this wave loaded has landed; after the barrier, everything every wave loaded
+#define GD_STEP_END()                           \
+  __builtin_amdgcn_s_waitcnt(0x0F70);           \
+  __syncthreads();
+  // the loads of a step are issued before the matrix work they overlap with, and stay there
+#ifdef CL_DBG_NODMA
+#define GD_ISSUE(kt, a_lds, b_lds)
+#else
+#define GD_ISSUE(kt, a_lds, b_lds)                              \
+  opa.issue(a_base + (i64)(kt) * a_step, a_lds);                \
+  opb.issue(b_base + (i64)(kt) * b_step, b_lds);                \
+  __builtin_amdgcn_sched_barrier(0);
+#endif
+#ifdef CL_DBG_NOCOMPUTE
+#undef GD_COMPUTE
+#define GD_COMPUTE(a_tile, b_tile)
+#endif
+
+  // Two steps per trip, one on each stage, with no branch inside: the loads issued in the second
+  // half are clamped onto the last step (for an even step count the final trip fetches that step
+  // once more into the idle stage, which nobody reads).
+  GD_ISSUE(0, gd_a0, gd_b0)
+  GD_STEP_END()
+  for (int kt = 0; kt + 1 < KT; kt += 2) {
+    GD_ISSUE(kt + 1, gd_a1, gd_b1)
+    GD_COMPUTE(gd_a0, gd_b0)
+    GD_STEP_END()
+    GD_ISSUE((kt + 2 < KT ? kt + 2 : KT - 1), gd_a0, gd_b0)
+    GD_COMPUTE(gd_a1, gd_b1)
+    GD_STEP_END()
+  }
+  if constexpr (KT % 2 == 1) GD_COMPUTE(gd_a0, gd_b0)     // an odd number of steps ends on stage 0
+
+  // ---- epilogue: acc[i][j][r] = C[m0 + am + 16 i + c][n0 + bn + 16 j + 4 g + r] ----------------
+#pragma unroll
+  for (int i = 0; i < GD_TM; ++i) {
+    const int m = m0 + am + 16 * i + c;
+    if (m >= CL_M) continue;
+#pragma unroll
+    for (int j = 0; j < GD_TN; ++j) {
+      const int n = n0 + bn + 16 * j + 4 * g;
+      if (n >= CL_N) continue;
+#if CL_SPLITS > 1
+      *reinterpret_cast<f32x4*>(CL_ARG_PACC + (((i64)split * GD_BATCH + batch) * CL_M + m) * CL_N + n) = acc[i][j];
+#else
+      elem4 y;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[i][j][r]);
+      *reinterpret_cast<elem4*>(CL_ARG_OUT + ((i64)batch * CL_M + m) * CL_N + n) = y;
+#endif
+    }
+  }
+}
+#endif  // CL_EMIT_PARTIAL
+
+#if CL_SPLITS > 1 && CL_EMIT_COMBINE
+// Combine: C = sum_s P[s].  Four columns per thread.
+extern "C" __global__ void __launch_bounds__(256)
+CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
+  const i64 rows = (i64)GD_BATCH * CL_M;
+  const i64 total = rows * (CL_N / 4);
+  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const i64 row = idx / (CL_N / 4);
+  const int n = (int)(idx % (CL_N / 4)) * 4;
+  f32x4 a = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < CL_SPLITS; ++s)
+    a += *reinterpret_cast<const f32x4*>(CL_CARG_PACC + ((i64)s * rows + row) * CL_N + n);
+  elem4 y;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) y[r] = to_elem(a[r]);
+  *reinterpret_cast<elem4*>(CL_CARG_OUT + row * CL_N + n) = y;
+}
+#endif

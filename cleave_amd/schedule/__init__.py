@@ -26,6 +26,7 @@ def _candidates(graph, arch):
             cands += policy.skinny_candidates(low, role, factor, arch)
         if not (fam == "rmsnorm_matmul" and low.problem["trans_A"]):
             cands += policy.gemm_candidates(low, role, factor, arch)
+        cands += policy.gemm_dma_candidates(low, role, factor, arch)
         return cands
     if fam == "attention":
         if not policy.attn_ok(low):

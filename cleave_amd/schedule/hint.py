@@ -7,7 +7,7 @@ from dataclasses import dataclass, field
 
 @dataclass(eq=False)
 class TileDict:
-    template: str                 # gemm | skinny | attn_decode | mla_decode
+    template: str                 # gemm | gemm_dma | skinny | attn_decode | mla_decode
     role: str                     # main | partial | combine
     tiling: dict                  # template parameters (BM/BN/BK/WM/WN, WAVES, ...)
     output_tile: list = field(default_factory=list)

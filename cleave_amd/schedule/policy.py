@@ -106,6 +106,62 @@ def gemm_candidates(low, role, factor, arch: Arch):
     return out
 
 
+def gemm_dma_candidates(low, role, factor, arch: Arch):
+    """Tilings of the direct-to-LDS matmul (plain matmul only: a fused norm needs the operand in
+    registers on its way to LDS).  No staging registers, so the budget is accumulators plus two
+    k blocks of operand fragments; tiles whose accumulators would fill a whole register class
+    (256) are left out: the compiler then shuffles them on every step."""
+    p = low.problem
+    if low.family != "matmul":
+        return []
+    splits = factor or 1
+    M, N, K = p["M"], p["N"], p["K"]
+    if K % (splits * 64) or (not p["trans_B"] and N % 8) or (p["trans_A"] and M % 8):
+        return []
+    kps = K // splits
+    batch = max(p["batch_A"], p["batch_B"])
+    out = []
+    shapes = (16, 32, 64, 128, 256)
+    for bm, bn, (wm, wn) in itertools.product(
+            shapes, shapes, ((1, 1), (1, 2), (2, 1), (2, 2), (1, 4), (4, 1), (2, 4), (4, 2))):
+        if bm % (16 * wm) or bn % (16 * wn):
+            continue
+        if bm > max(16, 2 * M) or bn > max(16, 2 * N):
+            continue
+        threads = wm * wn * 64
+        tm, tn = bm // wm // 16, bn // wn // 16
+        if tm & (tm - 1) or tn & (tn - 1) or tm * tn * 4 > 128:
+            continue
+        # every wave must own whole 1 KiB load units of both tiles or none
+        units_a, units_b = bm // 8, bn // 8
+        vgprs = tm * tn * 4 + (tm + tn) * 6 + -(-units_a // (wm * wn)) + -(-units_b // (wm * wn)) + 24
+        if vgprs > arch.vgprs_per_lane:
+            continue
+        lds = gemm_lds_bytes(bm, bn, 64)
+        if lds > arch.lds_bytes:
+            continue
+        blocks = _ceil(M, bm) * _ceil(N, bn) * batch * splits
+        per_cu = arch.blocks_per_cu(threads, lds, vgprs)
+        if per_cu < 1:
+            continue
+        passes = _waves_time(blocks, per_cu, arch)
+        live = min(per_cu, _ceil(blocks, arch.compute_units))
+        mfma_clk = live * (bm * bn * kps * 2) / 4096.0 / min(1.0, live * wm * wn / 8.0)
+        # LDS -> register traffic: about 32 B/clk per SIMD for 16-byte reads, two thirds of that for
+        # the transposing reads of a K-major operand
+        a_rate = 21.0 if p["trans_A"] else 32.0
+        b_rate = 32.0 if p["trans_B"] else 21.0
+        waves_per_simd = max(1.0, live * wm * wn / 4.0)
+        lds_clk = waves_per_simd * kps * 2 * 16 * (tm / a_rate + tn / b_rate)
+        fetch_clk = live * ((bm + bn) * kps * 2) / 24.0
+        pass_clk = max(mfma_clk, lds_clk, fetch_clk) + 2500 + 1500 * (kps // 64) / max(1, min(live, 2))
+        score = passes * pass_clk
+        tiling = dict(BM=bm, BN=bn, BK=64, WM=wm, WN=wn)
+        out.append(TileDict("gemm_dma", role, tiling, output_tile=[bm, bn], rstep_map={"k": 64}, n_threads=threads,
+                            split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+    return out
+
+
 # ----------------------------------------------------------------------------- few-row matmul
 def skinny_ok(low) -> bool:
     p = low.problem

@@ -53,6 +53,22 @@ def test_matmul_gemm_large_tiles(tiling):
     _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=tiling)
 
 
+DMA_TILES = [dict(BM=16, BN=16, BK=64, WM=1, WN=1), dict(BM=32, BN=64, BK=64, WM=1, WN=2),
+             dict(BM=64, BN=64, BK=64, WM=2, WN=2), dict(BM=128, BN=128, BK=64, WM=2, WN=2),
+             dict(BM=256, BN=128, BK=64, WM=4, WN=2), dict(BM=128, BN=256, BK=64, WM=2, WN=4, GROUP_M=2),
+             dict(BM=256, BN=256, BK=64, WM=2, WN=2)]
+
+
+@pytest.mark.parametrize("tiling", DMA_TILES, ids=lambda t: "x".join(str(v) for v in t.values()))
+@pytest.mark.parametrize("split", [None, 3])
+def test_matmul_gemm_dma(tiling, split):
+    """Direct-to-LDS matmul: ragged tile counts on both axes (edge rows and column chunks are
+    clamped), an odd number of K steps per split (the two-stage loop ends on either stage)."""
+    fn, dt, mk = C.CASES["c1"]
+    shapes = dict(M=600, N=776, K=576)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling, split=split)
+
+
 @pytest.mark.parametrize("split", [None, 4, 8, 16])
 def test_matmul_c1_full(split):
     fn, dt, mk = C.CASES["c1"]
