@@ -386,13 +386,18 @@ class HipCodeGen:
         total_rows = p["batch"] * p["heads"]
         emit_lse = bool(p.get("emit_lse"))
         self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], total_rows, emit_lse)
-        waves, hg = int(t.get("WAVES", 4)), int(t.get("HG", 1))
-        if p["heads"] % (16 * hg * waves):
-            raise CodegenError(f"{p['heads']} heads do not divide into {waves} waves of {16 * hg}")
+        waves, hg, stages = int(t.get("WAVES", 4)), int(t.get("HG", 1)), int(t.get("STAGES", 3))
+        vsplit = int(t.get("VSPLIT", 1))
+        if waves not in (1, 2, 4, 8):
+            raise CodegenError("the MLA template runs 1, 2, 4 or 8 waves per workgroup")
+        if waves % vsplit or p["heads"] % (16 * hg * waves // vsplit) or (p["ckv"] // 16) % (4 * vsplit):
+            raise CodegenError(f"{p['heads']} heads / {p['ckv']} features do not divide into {waves} waves of "
+                               f"{16 * hg} heads sharing a head set by {vsplit}")
         if p["ckv"] % 64 or p["kpe"] % 64:
-            raise CodegenError("the MLA template stages 64-feature panels: latent and rope widths must be multiples of 64")
+            raise CodegenError("the MLA template loads 64-feature panels: latent and rope widths must be multiples of 64")
         for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_SKV", p["skv"]),
-                     ("CL_WAVES", waves), ("CL_HG", hg), ("CL_BATCH", p["batch"])):
+                     ("CL_WAVES", waves), ("CL_HG", hg), ("CL_STAGES", stages), ("CL_VSPLIT", vsplit),
+                     ("CL_BATCH", p["batch"])):
             unit.define(k, v)
         if "LDS_AHEAD" in t:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
@@ -408,10 +413,9 @@ class HipCodeGen:
         splits = plan.split_factor or 1
         unit.templates += ["mla_decode.hip", "attn_combine.hip"]
         if partial:
-            from ..schedule.policy import mla_lds_bytes
-
-            grid = (p["batch"] * (p["heads"] // (16 * hg * waves)), splits, 1)
-            unit.launch(ENTRY, grid, waves * 64, mla_lds_bytes(p["ckv"], p["kpe"]), self._partial_args)
+            grid = (p["batch"] * (p["heads"] // (16 * hg * waves // vsplit)), splits, 1)
+            # the LDS images are a static array of the kernel: no dynamic LDS at launch
+            unit.launch(ENTRY, grid, waves * 64, 0, self._partial_args)
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)

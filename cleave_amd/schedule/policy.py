@@ -259,10 +259,9 @@ def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
 
 
 # ----------------------------------------------------------------------------- MLA decode
-def mla_lds_bytes(ckv, kpe):
-    """Two stages of the token-major tile ((ckv + kpe) / 64 panels of 32 x 64) and of the
-    feature-major copy (ckv / 2 rows of 64), two bytes per element."""
-    return 2 * (((ckv + kpe) // 64) * 32 * 64 + (ckv // 2) * 64) * 2
+def mla_lds_bytes(ckv, kpe, stages=3):
+    """`stages` token-major images of a 32-token step: (ckv + kpe) / 64 panels of 32 x 64 elements."""
+    return stages * ((ckv + kpe) // 64) * 32 * 64 * 2
 
 
 def mla_ok(low) -> bool:
@@ -273,18 +272,25 @@ def mla_ok(low) -> bool:
 def mla_candidates(low, role, factor, arch: Arch):
     p = low.problem
     splits = factor or 1
-    lds = mla_lds_bytes(p["ckv"], p["kpe"])
-    if lds > arch.lds_bytes:
-        return []
     out = []
     d = p["ckv"] + p["kpe"]
-    for waves, hg in itertools.product((1, 2, 4, 8), (1, 2)):
-        heads_per_block = 16 * hg * waves
+    for waves, (hg, vsplit), stages in itertools.product((1, 2, 4, 8), ((1, 1), (2, 2)), (2, 3, 4)):
+        # 32 heads per wave only with the value features shared out over a wave pair: the
+        # accumulators of 32 heads x all features would fill a whole register class
+        if waves % vsplit or (p["ckv"] // 16) % (4 * vsplit):
+            continue
+        heads_per_block = 16 * hg * waves // vsplit
         if p["heads"] % heads_per_block:
             continue
+        lds = mla_lds_bytes(p["ckv"], p["kpe"], stages)
+        if lds > arch.lds_bytes:
+            continue
+        units_per = (d // 64) * 4 // min(waves, 4)
+        if (stages - 2) * units_per >= 64:        # the wait for a step's loads counts the younger ones
+            continue
         # Q fragments and accumulators of a wave's heads stay in registers for the whole split
-        # (plus a step's staging registers, the ring of LDS operand reads and the softmax state)
-        vgprs = hg * (d // 32 * 4 + p["ckv"] // 16 * 4) + 36 + 32 + 48
+        # (plus the ring of LDS operand reads and the softmax state); loads use no registers
+        vgprs = hg * (d // 32 * 4 + p["ckv"] // 16 * 4 // vsplit + 4) + 32 + 24
         if vgprs > arch.vgprs_per_lane:
             continue
         blocks = p["batch"] * (p["heads"] // heads_per_block) * splits
@@ -293,22 +299,26 @@ def mla_candidates(low, role, factor, arch: Arch):
             continue
         passes = _waves_time(blocks, per_cu, arch)
         steps = _ceil(_ceil(p["skv"], 32), splits)
-        # per step: every wave reads the whole tile and its transposed copy from LDS once (one
-        # 128 B/clk port per CU) and issues hg matrix ops of 16 clocks per 1 KiB operand read;
-        # the staging writes both images once per workgroup
-        operand_reads = 2 * (d // 32) + p["ckv"] // 16
-        mfma_clk = operand_reads * hg * 16 * _ceil(waves, 4)
-        lds_clk = (waves * operand_reads * 1024 + 32 * (d + p["ckv"]) * 2) / 128.0
-        load_clk = 32 * d * 2 / 24.0
-        step_clk = max(mfma_clk, lds_clk, load_clk) + 400
+        # per step and wave: the score operands are 1 KiB reads at about 32 B/clk and SIMD, the
+        # value operands transposing reads at about two thirds of that; each feeds hg matrix ops
+        score_reads, value_reads = 2 * (d // 32), p["ckv"] // 16 // vsplit
+        mfma_clk = (score_reads + value_reads + 1) * hg * 18
+        lds_clk = (score_reads * 32 + value_reads * 48) * 0.45     # measured: LDS reads hide under the matrix ops
+        simd_share = max(1.0, per_cu * waves / 4.0)
+        # measured: the matrix ops of a step plus about 1500 clocks that nothing overlaps (barrier,
+        # load issue, the softmax between the two products); per workgroup of heads_per_block heads
+        step_clk = (max(mfma_clk, lds_clk) * simd_share / per_cu + 1500) * (64.0 / heads_per_block)
         util = min(1.0, blocks / (per_cu * arch.compute_units))
+        # a step's loads have (stages - 1) steps of matrix work to arrive in
+        latency_clk = 4000.0 / (stages - 1)
+        step_clk = max(step_clk, latency_clk)
         # split partials go out and come back once (element type): 2 * splits * rows * ckv * 2 bytes
         partial_clk = (4 * splits * p["batch"] * p["heads"] * p["ckv"]) / (arch.hbm_gbps * 1e3 * 0.6) * 2400 \
             if splits > 1 else 0.0
-        score = passes * steps * step_clk * (1.0 + 0.3 * (1 - util)) + 3000 + partial_clk
-        out.append(TileDict("mla_decode", role, dict(WAVES=waves, HG=hg), output_tile=[heads_per_block, p["ckv"]],
-                            rstep_map={"kv": 32}, n_threads=waves * 64, split_factor=factor, score=score,
-                            lds_bytes=lds, est_vgprs=vgprs))
+        score = passes * steps * step_clk * (1.0 + 0.3 * (1 - util)) + 8000 + partial_clk
+        out.append(TileDict("mla_decode", role, dict(WAVES=waves, HG=hg, VSPLIT=vsplit, STAGES=stages),
+                            output_tile=[heads_per_block, p["ckv"]], rstep_map={"kv": 32}, n_threads=waves * 64,
+                            split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
     return out
 
 

@@ -140,6 +140,9 @@ def test_mla_decode_small(split):
     _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=4), split=split)
     _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=2, HG=2), split=split)
     _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=1, HG=2), split=split)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=4, HG=2, VSPLIT=2), split=split)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(WAVES=2, HG=1, VSPLIT=2, STAGES=2),
+           split=split)
 
 
 def test_mla_decode_rising_maximum():
@@ -153,15 +156,16 @@ def test_mla_decode_rising_maximum():
     kv = (kv.float() * 0.2 + ramp * torch.sign(q.float().mean(dim=(1,), keepdim=True))).to(kv.dtype)
     ins = [q, kv, q_pe, k_pe]
     want = po.evaluate(prog, ins)[0]
-    for tiling, split in ((dict(WAVES=2, HG=1), None), (dict(WAVES=1, HG=2), 2)):
+    for tiling, split in ((dict(WAVES=2, HG=1), None), (dict(WAVES=1, HG=2), 2), (dict(WAVES=2, HG=2, VSPLIT=2), 2)):
         kernel = kernel_for(prog, template="mla_decode", tiling=tiling, split=split)
         print(f"case mla rising maximum {tiling} split={split}", flush=True)
         got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
         np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("tiling,split", [(dict(WAVES=4, HG=1), 8), (dict(WAVES=8, HG=1), 16), (dict(WAVES=4, HG=2), 16),
-                                          (dict(WAVES=4, HG=2), 4)],
+@pytest.mark.parametrize("tiling,split", [(dict(WAVES=4, HG=1), 8), (dict(WAVES=4, HG=1, STAGES=4), 16),
+                                          (dict(WAVES=2, HG=1, STAGES=2), 4), (dict(WAVES=4, HG=2, VSPLIT=2), 8),
+                                          (dict(WAVES=8, HG=1), 16)],
                          ids=lambda v: "x".join(str(x) for x in v.values()) if isinstance(v, dict) else str(v))
 def test_mla_decode_c4_full(tiling, split):
     fn, dt, mk = C.CASES["c4"]
