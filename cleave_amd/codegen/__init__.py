@@ -266,7 +266,7 @@ class HipCodeGen:
     def _emit_skinny(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
         self._matmul_common(unit, plan, params, partial, combine, fused)
-        tile = dict(WAVES_N=1, WAVES_K=1)
+        tile = dict(WAVES_N=1, WAVES_K=1, PREFETCH=2)
         tile.update(t)
         for k, v in tile.items():
             unit.define(f"CL_{k}", v)

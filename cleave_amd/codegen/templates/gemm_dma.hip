@@ -46,7 +46,8 @@ __shared__ __attribute__((aligned(1024))) elem_t gd_b0[GD_B_ELEMS];
 __shared__ __attribute__((aligned(1024))) elem_t gd_b1[GD_B_ELEMS];
 
 // ---- K-minor image: row r at r * 64, chunk ch at slot ch ^ swz(r) ------------------------------
-CL_DEVICE int gd_swz_kmin(int row) { return ((row >> 1) ^ (row >> 3)) & 7; }
+// (row & 6: measured at the full rate of a linear read for the operand shape, lane = row l % 16, chunk l / 16)
+CL_DEVICE int gd_swz_kmin(int row) { return row & 6; }
 
 // ---- K-major image: k row at k * COLS, chunk ch at slot ch ^ f(k); f is even so that the two
 // chunks of a 32-byte patch row stay neighbours.  The eight k rows a half wave reads together
@@ -107,8 +108,8 @@ struct GdOperand {
 // fragment readers --------------------------------------------------------------------------------
 // K-minor: `off0` = element offset of (row ext_w + c, chunk g) for the wave's first 16-row tile
 CL_DEVICE elem8 gd_read_kmin(const elem_t* tile, int off0, int i, int s) {
-  // row 16 i + c: swizzle(16 i + c) = swizzle(c-part) ^ (2 i & 7); k block s: chunk + 4 s
-  return *reinterpret_cast<const elem8*>(tile + 16 * i * 64 + (off0 ^ (s * 32) ^ (((2 * i) & 7) << 3)));
+  // row 16 i + c has the swizzle of row c; k block s: chunk + 4 s
+  return *reinterpret_cast<const elem8*>(tile + 16 * i * 64 + (off0 ^ (s * 32)));
 }
 // K-major: `off0` = element offset of this lane's 8-byte piece for tile j = 0, k block 0, t = 0
 template <int COLS>

@@ -17,25 +17,49 @@
 //   CL_SPLITS          K splits across workgroups (grid.y)
 //   CL_NORM            0 plain, 1 RMSNorm epilogue; CL_GAMMA: 1 when a (K) weight multiplies X
 //   CL_EPS             epsilon inside the rsqrt
+//   CL_PREFETCH        steps of loads in flight ahead of the one being computed (1..3)
 
 #define SK_MT ((CL_M + 15) / 16)
 #define SK_COLS 128
 #define SK_STEP 32
 #define SK_THREADS (CL_WAVES_N * CL_WAVES_K * 64)
 
+#ifndef CL_PREFETCH
+#define CL_PREFETCH 2
+#endif
+// Everything one 32-row step needs, as loaded: the lane's 8x8 block of W, its X fragments
+// (lane (c, g) holds X[16 mt + c][k0 + 8 g .. +8]) and the matching gamma chunk.  X and gamma
+// travel with the W block on purpose: a small load issued on its own in the loop would sit
+// behind the W prefetches in the in-order load queue and make every step wait for them.
 struct SkTile {
   u32x4 w[8];
+  u32x4 x[SK_MT];
+#if CL_NORM && CL_GAMMA
+  u32x4 gm;
+#endif
 };
 
-CL_DEVICE void sk_load_w(const elem_t* __restrict__ W, int k0, int ncol, int g, SkTile& t) {
+CL_DEVICE void sk_load(const elem_t* __restrict__ W, const elem_t* __restrict__ X, const elem_t* __restrict__ G,
+                       int k0, int ncol, int c, int g, SkTile& t) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) t.w[e] = ld16(W + (i64)(k0 + 8 * g + e) * CL_N + ncol);
+#pragma unroll
+  for (int mt = 0; mt < SK_MT; ++mt) {
+    const int m = 16 * mt + c;
+    t.x[mt] = ld16(X + (i64)(m < CL_M ? m : CL_M - 1) * CL_K + k0 + 8 * g);   // rows past M: masked when used
+  }
+#if CL_NORM && CL_GAMMA
+  t.gm = ld16(G + k0 + 8 * g);
+#else
+  (void)G;
+#endif
 }
 
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(SK_THREADS)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // (readfirstlane: everything derived from the wave index is uniform and stays in scalar registers)
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int wn = wave % CL_WAVES_N, wk = wave / CL_WAVES_N;
   const int split = blockIdx.y;
@@ -67,45 +91,88 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
   for (int mt = 0; mt < SK_MT; ++mt) ss[mt] = 0.f;
 
-  SkTile cur, nx1, nx2;
-  if (s_begin < s_end) sk_load_w(CL_ARG_W, s_begin * SK_STEP, ncol, g, cur);
-  if (s_begin + 1 < s_end) sk_load_w(CL_ARG_W, (s_begin + 1) * SK_STEP, ncol, g, nx1);
-  for (int s = s_begin; s < s_end; ++s) {
-    const int k0 = s * SK_STEP;
-    if (s + 2 < s_end) sk_load_w(CL_ARG_W, (s + 2) * SK_STEP, ncol, g, nx2);
-
-    // X fragments (A operand): lane (c, g) holds X[16 mt + c][k0 + 8 g .. +8]
-    elem8 xa[SK_MT];
-#pragma unroll
-    for (int mt = 0; mt < SK_MT; ++mt) {
-      const int m = 16 * mt + c;
-      const bool live = m < CL_M;
-      u32x4 raw = ld16(CL_ARG_X + (i64)(live ? m : 0) * CL_K + k0 + 8 * g);
-      if (!live) raw = (u32x4){0u, 0u, 0u, 0u};
-      elem8 x = as_elem8(raw);
+  // Ring of CL_PREFETCH + 1 register tiles: while step n is in the matrix cores the loads of
+  // steps n+1 .. n+CL_PREFETCH are in flight.
+#if CL_NORM && CL_GAMMA
+  const elem_t* gamma_ptr = CL_ARG_GAMMA;
+#else
+  const elem_t* gamma_ptr = nullptr;
+#endif
+  SkTile ring[CL_PREFETCH + 1];
+  // one step on the tile `cur`: row sums of squares, gamma, 8x8 transpose of W, eight MFMAs per row tile
+#define SK_CONSUME(cur)                                                                   \
+  {                                                                                       \
+    elem8 xa[SK_MT];                                                                      \
+    _Pragma("unroll") for (int mt = 0; mt < SK_MT; ++mt) {                                \
+      u32x4 raw = (cur).x[mt];                                                            \
+      if (16 * mt + c >= CL_M) raw = (u32x4){0u, 0u, 0u, 0u};                             \
+      elem8 x = as_elem8(raw);                                                            \
+      SK_NORM_X(x, mt, cur)                                                               \
+      xa[mt] = x;                                                                         \
+    }                                                                                     \
+    u32x4 wt[8];                                                                          \
+    transpose8x8((cur).w, wt);                                                            \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j)                                         \
+      _Pragma("unroll") for (int mt = 0; mt < SK_MT; ++mt)                                \
+        acc[mt][j] = mfma16(xa[mt], as_elem8(wt[j]), acc[mt][j]);                         \
+  }
 #if CL_NORM
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float xf = to_f32(x[i]);
-        ss[mt] += xf * xf;
-      }
 #if CL_GAMMA
-      elem8 gm = as_elem8(ld16(CL_ARG_GAMMA + k0 + 8 * g));
-#pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] = to_elem(to_f32(x[i]) * to_f32(gm[i]));
+#define SK_GAMMA_X(x, cur)                                                                \
+  {                                                                                       \
+    const elem8 gm = as_elem8((cur).gm);                                                  \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i) x[i] = to_elem(to_f32(x[i]) * to_f32(gm[i])); \
+  }
+#else
+#define SK_GAMMA_X(x, cur)
 #endif
+#define SK_NORM_X(x, mt, cur)                                                             \
+  _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                         \
+    const float xf = to_f32(x[i]);                                                        \
+    ss[mt] += xf * xf;                                                                    \
+  }                                                                                       \
+  SK_GAMMA_X(x, cur)
+#else
+#define SK_NORM_X(x, mt, cur)
 #endif
-      xa[mt] = x;
-    }
 
-    u32x4 wt[8];
-    transpose8x8(cur.w, wt);
+  if constexpr (steps_total % (CL_SPLITS * CL_WAVES_K) == 0 && steps_per_wave <= 32) {
+    // every wave has exactly steps_per_wave steps: the whole walk is straight-line code, each
+    // load issued CL_PREFETCH steps ahead of its use and none past the end
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int i = 0; i < CL_PREFETCH && i < steps_per_wave; ++i)
+      sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, (s_begin + i) * SK_STEP, ncol, c, g, ring[i % (CL_PREFETCH + 1)]);
 #pragma unroll
-      for (int mt = 0; mt < SK_MT; ++mt) acc[mt][j] = mfma16(xa[mt], as_elem8(wt[j]), acc[mt][j]);
-    cur = nx1;
-    nx1 = nx2;
+    for (int i = 0; i < steps_per_wave; ++i) {
+      if (i + CL_PREFETCH < steps_per_wave)
+        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, (s_begin + i + CL_PREFETCH) * SK_STEP, ncol, c, g,
+                ring[(i + CL_PREFETCH) % (CL_PREFETCH + 1)]);
+      SK_CONSUME(ring[i % (CL_PREFETCH + 1)])
+    }
+  } else {
+    // Ragged ranges: prefetch loads are issued unconditionally, a step past the end clamped onto
+    // the wave's last step (an L2 hit, never consumed), so the load counter is the same on every
+    // path and the waits stay exact.
+    const int last_step = s_end - 1;
+    if (s_begin < s_end) {
+#pragma unroll
+      for (int i = 0; i < CL_PREFETCH; ++i) {
+        int sidx = s_begin + i;
+        sidx = sidx < last_step ? sidx : last_step;
+        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, sidx * SK_STEP, ncol, c, g, ring[i]);
+      }
+    }
+    for (int base = s_begin; base < s_end; base += CL_PREFETCH + 1) {
+#pragma unroll
+      for (int r = 0; r <= CL_PREFETCH; ++r) {
+        const int s = base + r;
+        if (s >= s_end) break;
+        int ahead = s + CL_PREFETCH;
+        ahead = ahead < last_step ? ahead : last_step;
+        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, ahead * SK_STEP, ncol, c, g, ring[(r + CL_PREFETCH) % (CL_PREFETCH + 1)]);
+        SK_CONSUME(ring[r])
+      }
+    }
   }
 
   // ---- reduce across the waves that share a column slab ------------------------------------
