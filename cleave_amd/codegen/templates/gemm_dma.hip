@@ -25,7 +25,7 @@
 #define GD_BK 64
 #define GD_BATCH (CL_BATCH_A > CL_BATCH_B ? CL_BATCH_A : CL_BATCH_B)
 #ifndef CL_GROUP_M
-#define CL_GROUP_M 4
+#define CL_GROUP_M 8
 #endif
 #define GD_XCDS 8
 static_assert(CL_BK == 64, "K steps are 64 wide (128-byte K-minor rows)");

@@ -7,6 +7,8 @@ import numpy as np
 import pytest
 import torch
 
+import cleave_amd
+import cleave_amd.lang as cl
 from oracle import program_oracle as po
 from tests import _cases as C
 from tests._lowlevel import kernel_for
@@ -67,6 +69,47 @@ def test_matmul_gemm_dma(tiling, split):
     fn, dt, mk = C.CASES["c1"]
     shapes = dict(M=600, N=776, K=576)
     _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling, split=split)
+
+
+def test_matmul_gemm_dma_bf16():
+    shapes = dict(M=192, N=256, K=384)
+    prog = C.matmul.trace(cl.bf16, **shapes)
+    ins = [t.to(torch.bfloat16) for t in C.inputs_c1(shapes, seed=7)]
+    want = po.evaluate(prog, ins)[0]
+    for tiling, split in ((dict(BM=64, BN=128, BK=64, WM=2, WN=2), None), (dict(BM=32, BN=64, BK=64, WM=1, WN=2), 2)):
+        kernel = kernel_for(prog, template="gemm_dma", tiling=tiling, split=split)
+        print(f"case matmul bf16 gemm_dma {tiling} split={split}", flush=True)
+        got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@cleave_amd.jit
+def matmul_nt(x: cl.Tensor["M", "K"], w: cl.Tensor["N", "K"]):
+    return x @ w.mT
+
+
+@cleave_amd.jit
+def matmul_tn(x: cl.Tensor["K", "M"], w: cl.Tensor["K", "N"]):
+    return x.mT @ w
+
+
+@pytest.mark.parametrize("template,tiling", [("gemm_dma", dict(BM=64, BN=64, BK=64, WM=2, WN=2)),
+                                             ("gemm_dma", dict(BM=128, BN=256, BK=64, WM=2, WN=4)),
+                                             ("gemm", dict(BM=64, BN=64, BK=64, WM=2, WN=2))],
+                         ids=["dma64", "dma128x256", "staged64"])
+def test_matmul_transposed_operands(template, tiling):
+    """B stored (N, K) (both operands K-minor) and A stored (K, M) (both K-major): the other two
+    combinations of the 16-byte and the transposing fragment readers."""
+    g = torch.Generator(device="cpu").manual_seed(11)
+    M, N, K = 200, 328, 320
+    for fn, shapes_in in ((matmul_nt, ((M, K), (N, K))), (matmul_tn, ((K, M), (K, N)))):
+        prog = fn.trace(cl.f16, M=M, N=N, K=K)
+        ins = [((torch.rand(*shp, generator=g) * 2 - 1) / K ** 0.5).to(torch.float16) for shp in shapes_in]
+        want = po.evaluate(prog, ins)[0]
+        kernel = kernel_for(prog, template=template, tiling=tiling)
+        print(f"case {prog.name} {template} {tiling}", flush=True)
+        got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("split", [None, 4, 8, 16])
