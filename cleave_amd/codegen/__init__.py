@@ -215,7 +215,12 @@ class HipCodeGen:
                 unit.define("CL_CARG_PSS", op["PSS" + suffix])
             unit.define("CL_CARG_OUT", op["OUT"])
             args = unit.signature("CL_COMBINE_PARAMS", "CL_COMBINE_NAME", entry, sig, ())
-            self._combine_args = (entry, args, batch * p["M"] * p["N"])
+            # columns per thread: the most that still leaves the chip a few hundred workgroups
+            total = batch * p["M"] * p["N"]
+            cols = next((c for c in (4, 2, 1) if p["N"] % c == 0 and total // c // 256 >= 256), 1)
+            unit.define("CL_COMBINE_ROWS", batch * p["M"])
+            unit.define("CL_COMBINE_COLS", cols)
+            self._combine_args = (entry, args, -(-(total // cols) // 256))
 
     def _emit_gemm(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
@@ -236,8 +241,9 @@ class HipCodeGen:
             lds = gemm_lds_bytes(tile["BM"], tile["BN"], tile["BK"], plan.family == "rmsnorm_matmul")
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, lds, self._partial_args)
         if combine:
-            entry, args, total = self._combine_args
-            unit.launch(entry, (-(-(total // 4) // 256), 1, 1), 256, 0, args)
+            entry, args, blocks = self._combine_args
+            unit.templates.append("matmul_combine.hip")
+            unit.launch(entry, (blocks, 1, 1), 256, 0, args)
 
     def _emit_gemm_dma(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
@@ -260,8 +266,9 @@ class HipCodeGen:
             # the tile images are static LDS arrays of the kernel: no dynamic LDS at launch
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, 0, self._partial_args)
         if combine:
-            entry, args, total = self._combine_args
-            unit.launch(entry, (-(-(total // 4) // 256), 1, 1), 256, 0, args)
+            entry, args, blocks = self._combine_args
+            unit.templates.append("matmul_combine.hip")
+            unit.launch(entry, (blocks, 1, 1), 256, 0, args)
 
     def _emit_skinny(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
@@ -281,8 +288,9 @@ class HipCodeGen:
             lds = skinny_lds_bytes(-(-p["M"] // 16), tile["WAVES_N"], tile["WAVES_K"])
             unit.launch(ENTRY, grid, tile["WAVES_N"] * tile["WAVES_K"] * 64, lds, self._partial_args)
         if combine:
-            entry, args, total = self._combine_args
-            unit.launch(entry, (-(-(total // 8) // 256), 1, 1), 256, 0, args)
+            entry, args, blocks = self._combine_args
+            unit.templates.append("matmul_combine.hip")
+            unit.launch(entry, (blocks, 1, 1), 256, 0, args)
 
     # ------------------------------------------------------------------ attention families
     def _attn_common(self, unit, plan, params, partial, combine, fused, vdim, total_rows, emit_lse):
@@ -401,6 +409,8 @@ class HipCodeGen:
             unit.define(k, v)
         if "LDS_AHEAD" in t:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
+        if "OCC" in t:
+            unit.define("CL_OCC", int(t["OCC"]))
         for k in t:
             if k.startswith("DBG_"):
                 unit.define(f"CL_{k}", 1)

@@ -302,24 +302,3 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 }
 #endif  // CL_EMIT_PARTIAL
-
-#if CL_SPLITS > 1 && CL_EMIT_COMBINE
-// Combine: C = sum_s P[s].  Four columns per thread.
-extern "C" __global__ void __launch_bounds__(256)
-CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
-  const i64 rows = (i64)GD_BATCH * CL_M;
-  const i64 total = rows * (CL_N / 4);
-  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const i64 row = idx / (CL_N / 4);
-  const int n = (int)(idx % (CL_N / 4)) * 4;
-  f32x4 a = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int s = 0; s < CL_SPLITS; ++s)
-    a += *reinterpret_cast<const f32x4*>(CL_CARG_PACC + ((i64)s * rows + row) * CL_N + n);
-  elem4 y;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) y[r] = to_elem(a[r]);
-  *reinterpret_cast<elem4*>(CL_CARG_OUT + row * CL_N + n) = y;
-}
-#endif

@@ -28,6 +28,7 @@
 //   CL_WAVES  waves per workgroup (1, 2, 4 or 8)       CL_HG   16-head groups per wave (1 or 2)
 //   CL_SPLITS KV splits                                CL_BATCH  batch entries
 //   CL_SCALE_LOG2E  softmax scale * log2(e)            CL_STAGES LDS images (2..4)
+//   CL_OCC     workgroups meant to share a compute unit (register cap)
 //   CL_VSPLIT  waves sharing one head set, each accumulating 1 / VSPLIT of the value features (the
 //              accumulators of 32 heads x 512 features would fill a whole register class)
 //   CL_PO_ELEM  1: split partials are normalised values in the element type with m = log-sum-exp
@@ -154,7 +155,13 @@ CL_DEVICE void ml_issue_from(const MlLoader& ld, const elem_t* lat_rows, const e
 #endif
 
 #if CL_EMIT_PARTIAL
-extern "C" __global__ void __launch_bounds__(ML_THREADS)
+#ifndef CL_OCC
+#define CL_OCC 1
+#endif
+// CL_OCC workgroups share a compute unit (the second launch bound caps the registers so that
+// CL_OCC * WAVES / 4 waves fit a SIMD): their barriers are independent, so one's waits overlap
+// the other's matrix work
+extern "C" __global__ void __launch_bounds__(ML_THREADS, (CL_OCC * CL_WAVES + 3) / 4)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   ML_STAMP(0)
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);

@@ -255,40 +255,3 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 }
 #endif  // CL_EMIT_PARTIAL
-
-#if CL_SPLITS > 1 && CL_EMIT_COMBINE
-// Combine: Y[m][n] = (sum_s P[s][m][n]) * rsqrt(sum_s ss[s][m] / K + eps).  Eight columns per thread.
-extern "C" __global__ void __launch_bounds__(256)
-CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
-  const i64 total = (i64)CL_M * (CL_N / 8);
-  const i64 idx = (i64)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const int m = (int)(idx / (CL_N / 8));
-  const int n = (int)(idx % (CL_N / 8)) * 8;
-  f32x4 a = (f32x4){0.f, 0.f, 0.f, 0.f}, b = a;
-#if CL_NORM
-  float tot = 0.f;
-#endif
-#pragma unroll
-  for (int s = 0; s < CL_SPLITS; ++s) {
-    const float* p = CL_CARG_PACC + ((i64)s * CL_M + m) * CL_N + n;
-    a += *reinterpret_cast<const f32x4*>(p);
-    b += *reinterpret_cast<const f32x4*>(p + 4);
-#if CL_NORM
-    tot += CL_CARG_PSS[(i64)s * CL_M + m];
-#endif
-  }
-#if CL_NORM
-  const float rs = fast_rsqrt(tot * (1.0f / CL_K) + CL_EPS);
-#else
-  const float rs = 1.0f;
-#endif
-  elem8 y;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    y[i] = to_elem(a[i] * rs);
-    y[4 + i] = to_elem(b[i] * rs);
-  }
-  st16(CL_CARG_OUT + (i64)m * CL_N + n, as_u32x4(y));
-}
-#endif
