@@ -1,7 +1,8 @@
 """Shipped dynamic operators: the spec that names each one's inputs and the tiling it is
 built at (``python/cleave/dynamic/registry.py:37-231``).  Of the reference's nine operators
-the paged GQA decode family is built here; the others are recognised by the frontend and
-refused by the access layer until their templates exist."""
+the three paged GQA decode ones are built here (page size 1 with 8 and 4 kv heads, page size 64);
+the prefill and MLA ones are recognised by the frontend and refused by the access layer until
+their templates exist."""
 
 from __future__ import annotations
 
@@ -63,6 +64,16 @@ class DynamicOperator:
 
 
 OPERATORS = {op.name: op for op in (
+    # page size 1: the row-gather layer (one table entry per token); the kv4 operator has eight
+    # query rows per kv head, the kv8 one four: both fit one 16-row tile
+    DynamicOperator(
+        "gqa_paged_decode_h32_kv8_d128_ps1", PagingSpec(num_qo_heads=32, num_kv_heads=8),
+        dict(query_rows=16, kv_tile=32, head_dim=128, waves=4), (32, 8, 128),
+        _wl.WORKLOADS["gqa_paged_decode_h32_kv8_d128_ps1"], page_size=1),
+    DynamicOperator(
+        "gqa_paged_decode_h32_kv4_d128_ps1", PagingSpec(num_qo_heads=32, num_kv_heads=4, grid_order=("head", "batch")),
+        dict(query_rows=16, kv_tile=32, head_dim=128, waves=4), (32, 4, 128),
+        _wl.WORKLOADS["gqa_paged_decode_h32_kv4_d128_ps1"], page_size=1),
     DynamicOperator(
         "gqa_paged_decode_h32_kv8_d128_ps64",
         PagingSpec(num_qo_heads=32, num_kv_heads=8, kind=PAGED_DECODE_SLAB, page_size=64, grid_order=("head", "batch"),

@@ -14,7 +14,18 @@ import random
 import zlib
 
 WORKLOADS = {
+    "gqa_paged_decode_h32_kv8_d128_ps1": ((1, 11, 10), (16, 1069, 1034), (16, 81390, 12942), (64, 68237, 58966)),
+    "gqa_paged_decode_h32_kv4_d128_ps1": ((1, 8, 7), (16, 1070, 1020), (16, 32348, 23079), (64, 61535, 61519)),
     "gqa_paged_decode_h32_kv8_d128_ps64": ((4, 349, 212), (16, 1686, 1033), (32, 15178, 14103), (128, 52033, 47438)),
+}
+
+# Geomean latency over exactly those axes on the reference's own back end, as recorded in its
+# checked-in baseline (``tests/perf/baselines/h100-80gb-hbm3.json``, NVIDIA H100 80GB HBM3, bf16):
+# microseconds per axis in the order above.  Quoted beside this back end's numbers, never a target.
+REFERENCE_H100_US = {
+    "gqa_paged_decode_h32_kv8_d128_ps1": (2.4898, 5.2114, 59.4166, 137.0866),
+    "gqa_paged_decode_h32_kv4_d128_ps1": (2.4530, 5.0890, 80.3984, 131.4043),
+    "gqa_paged_decode_h32_kv8_d128_ps64": (74.0303, 149.6087, 1667.6903, 4817.6807),
 }
 
 

@@ -125,3 +125,40 @@ def paged_workload(lens, page_size=64, num_pages=None, hq=32, hkv=8, d=128, seed
     v_cache = (torch.randn(num_pages, page_size, hkv, d, generator=g) * pool_scale).to(dtype)
     args = [q, k_cache, v_cache, indptr, kv_indices, last]
     return [a.to(device) for a in args] + [float(d) ** -0.5]
+
+
+_batch, _num_pages, _n_idx = cl.dims("batch num_pages n_idx", dynamic=True)
+_kv_len = cl.Dim("kv_len", dynamic=True, hint=4096)
+
+
+def paged_decode_op(hq=32, hkv=8, d=128, page=64, dtype=cl.f16, name=None):
+    """The paged GQA decode operator as a ``@jit`` program (the reference's registry form:
+    with a last-page-length input only when pages hold more than one token)."""
+    name = name or f"gqa_paged_decode_h{hq}_kv{hkv}_d{d}_ps{page}"
+
+    def body(q, k_cache, v_cache, pages):
+        k, v = cl.paged_gather(k_cache, pages), cl.paged_gather(v_cache, pages)
+        qg = q.view(_batch, hkv, hq // hkv, d)
+        return qg, k, v
+
+    if page > 1:
+        def op(q, k_cache, v_cache, kv_indptr, kv_indices, kv_last_page_len, sm_scale):
+            pages = cl.PageTable(kv_indptr, kv_indices, last_page_len=kv_last_page_len, length=_kv_len)
+            qg, k, v = body(q, k_cache, v_cache, pages)
+            p, lse = cl.softmax((qg @ k.mT) * sm_scale, dim=-1, return_lse=True)
+            return (p @ v).view(_batch, hq, d), lse.view(_batch, hq)
+    else:
+        def op(q, k_cache, v_cache, kv_indptr, kv_indices, sm_scale):
+            pages = cl.PageTable(kv_indptr, kv_indices, length=_kv_len)
+            qg, k, v = body(q, k_cache, v_cache, pages)
+            p, lse = cl.softmax((qg @ k.mT) * sm_scale, dim=-1, return_lse=True)
+            return (p @ v).view(_batch, hq, d), lse.view(_batch, hq)
+    # the annotations are built here rather than written on the signature: this module defers
+    # annotation evaluation, and the extents are arguments of this factory
+    ann = {"q": cl.Tensor[_batch, hq, d], "k_cache": cl.Tensor[_num_pages, page, hkv, d],
+           "v_cache": cl.Tensor[_num_pages, page, hkv, d], "kv_indptr": cl.Tensor[_batch + 1, cl.i32],
+           "kv_indices": cl.Tensor[_n_idx, cl.i32], "sm_scale": cl.Scalar[cl.f32]}
+    if page > 1:
+        ann["kv_last_page_len"] = cl.Tensor[_batch, cl.i32] | None
+    op.__annotations__ = ann
+    return cleave_amd.jit(name=name, dtype=dtype)(op)

@@ -127,3 +127,26 @@ def test_compile_dynamic_paged_decode(cache_root):
     _close(out, want_o)
     live = np.isfinite(want_l)
     np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("name", ["gqa_paged_decode_h32_kv4_d128_ps1", "gqa_paged_decode_h32_kv8_d128_ps1"])
+def test_registry_row_gather_operators(cache_root, name):
+    """The shipped page-size-1 decode operators (one table entry per token), bf16, searched and
+    validated over their captured workload axes; then one call against the numpy oracle."""
+    from cleave_amd.dynamic import OPERATORS
+
+    op = OPERATORS[name]
+    hq, hkv, d = op.dims[:3]
+    fn = C.paged_decode_op(hq, hkv, d, 1, dtype=cl.bf16, name=name)
+    kernel = cleave_amd.compile(fn, schedule=P.ScheduleConfig(topk=1), split=cl.Split("kv_len", (4,)), max_workloads=2)
+    rep = kernel.report
+    assert rep.best() is not None and len(rep.correct) >= 2 and rep.n_workloads == len(op.workloads)
+    lens = [37, 0, 300, 1]
+    args = C.paged_workload(lens, page_size=1, num_pages=400, hq=hq, hkv=hkv, d=d, dtype=torch.bfloat16, device="cuda")
+    args = args[:5] + args[6:]                      # no last-page-length input at page size 1
+    out, lse = kernel(*args)
+    want_o, want_l = paged_oracle.decode(*[a.cpu() if isinstance(a, torch.Tensor) else a for a in args[:5]], lens, 1,
+                                         args[-1])
+    _close(out, want_o)
+    live = np.isfinite(want_l)
+    np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
