@@ -325,4 +325,66 @@ int chip_time_launches(const chip_launch_desc* seq, int n, void* stream, int war
   return rc;
 }
 
+int chip_time_graph(const chip_launch_desc* seq, int n, void* stream, int warmup, int batch, int rounds, int nsets,
+                    void*** arg_sets, float* ms_per_iter) {
+  if (!seq || n <= 0 || !ms_per_iter) return fail(CHIP_ERR_INVALID, "chip_time_graph: bad sequence or output");
+  if (batch <= 0 || rounds <= 0 || warmup < 0)
+    return fail(CHIP_ERR_INVALID, "chip_time_graph: batch and rounds must be > 0 and warmup >= 0");
+  if (nsets > 1 && !arg_sets) return fail(CHIP_ERR_INVALID, "chip_time_graph: nsets > 1 needs arg_sets");
+  hipStream_t caller = static_cast<hipStream_t>(stream);
+  // Work queued on the caller's stream comes first; capture and replay then run on a stream of
+  // this call's own (the legacy default stream cannot be captured), at the default priority.
+  HIP_TRY(hipStreamSynchronize(caller));
+  hipStream_t s = nullptr;
+  HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+  int rc = CHIP_OK;
+  auto pass = [&](int it) -> int {
+    for (int i = 0; i < n; ++i) {
+      void** args = seq[i].args;
+      if (nsets > 1) args = arg_sets[(size_t)(it % nsets) * n + i];
+      int r = launch_one(seq[i], args, s);
+      if (r) return r;
+    }
+    return CHIP_OK;
+  };
+  auto step = [&](const char* what, hipError_t e) {
+    if (rc == CHIP_OK && e != hipSuccess) rc = hip_fail(what, e);
+  };
+  for (int it = 0; rc == CHIP_OK && it < warmup; ++it) rc = pass(it);
+  step("hipStreamSynchronize", hipStreamSynchronize(s));
+  if (rc == CHIP_OK) {
+    // only kernel launches are recorded: no memset or copy nodes
+    step("hipStreamBeginCapture", hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    if (rc == CHIP_OK) {
+      int prc = CHIP_OK;
+      for (int it = 0; prc == CHIP_OK && it < batch; ++it) prc = pass(warmup + it);
+      hipError_t e = hipStreamEndCapture(s, &graph);   // always end the capture, also after a failed launch
+      if (prc != CHIP_OK) rc = prc;
+      step("hipStreamEndCapture", e);
+    }
+  }
+  if (rc == CHIP_OK) step("hipGraphInstantiate", hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+  if (rc == CHIP_OK) step("hipGraphLaunch", hipGraphLaunch(exec, s));          // one untimed replay
+  step("hipStreamSynchronize", hipStreamSynchronize(s));
+  if (rc == CHIP_OK) step("hipEventCreate", hipEventCreate(&t0));
+  if (rc == CHIP_OK) step("hipEventCreate", hipEventCreate(&t1));
+  if (rc == CHIP_OK) step("hipEventRecord", hipEventRecord(t0, s));
+  for (int r = 0; rc == CHIP_OK && r < rounds; ++r) step("hipGraphLaunch", hipGraphLaunch(exec, s));
+  if (rc == CHIP_OK) step("hipEventRecord", hipEventRecord(t1, s));
+  if (rc == CHIP_OK) step("hipEventSynchronize", hipEventSynchronize(t1));
+  float ms = 0.f;
+  if (rc == CHIP_OK) step("hipEventElapsedTime", hipEventElapsedTime(&ms, t0, t1));
+  (void)hipStreamSynchronize(s);
+  if (t0) (void)hipEventDestroy(t0);
+  if (t1) (void)hipEventDestroy(t1);
+  if (exec) (void)hipGraphExecDestroy(exec);
+  if (graph) (void)hipGraphDestroy(graph);
+  (void)hipStreamDestroy(s);
+  if (rc == CHIP_OK) *ms_per_iter = ms / ((float)rounds * (float)batch);
+  return rc;
+}
+
 }  // extern "C"

@@ -246,11 +246,13 @@ class CompiledKernel:
             return None
         return outs[0] if len(outs) == 1 else outs
 
-    def time(self, *args, warmup: int = 4, iters: int = 100, rotate=None, only=None) -> float:
+    def time(self, *args, warmup: int = 4, iters: int = 100, rotate=None, only=None, graph_batch: int = 0) -> float:
         """Milliseconds per call measured with HIP events inside the native library.  ``rotate``:
         further argument tuples (same signature) cycled through call by call, so a working set
         larger than the 256 MB last-level cache keeps every call reading HBM.  ``only``: indices
-        of the launches to time (e.g. ``[0]`` for the partial kernel of a fused pair alone)."""
+        of the launches to time (e.g. ``[0]`` for the partial kernel of a fused pair alone).
+        ``graph_batch`` > 0: time replays of a HIP graph holding that many calls (the reference's
+        way of timing) instead of an eager launch loop."""
         import torch
 
         sets = [args] + list(rotate or [])
@@ -259,6 +261,9 @@ class CompiledKernel:
         for a in sets:
             bound, dims, device = self._bind(a)
             held.append(self._materialise(bound, dims, device))
+            if self.out_idx is not None:
+                for t in held[-1]:
+                    t.zero_()      # the outputs are this call's own: whatever they hold afterwards, the timed launches wrote
             with torch.cuda.device(device):
                 descs, keep = self._descs(bound, dims)
             if not descs:
@@ -269,7 +274,9 @@ class CompiledKernel:
             all_keep.append(keep)
         with torch.cuda.device(device):
             stream = torch.cuda.current_stream(device).cuda_stream
-            ms = shim.time_launches(all_descs[0], stream, warmup, iters, all_keep if len(sets) > 1 else None)
+            ms = shim.time_launches(all_descs[0], stream, warmup, iters, all_keep if len(sets) > 1 else None,
+                                    graph_batch=graph_batch)
+        self.last_timed_outputs = held[0]      # what the timed launches of the first argument set wrote
         return ms
 
 

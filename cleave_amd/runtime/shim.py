@@ -25,6 +25,7 @@ EXPORTS = (
     "chip_abi_version", "chip_last_error", "chip_device_count", "chip_device_info_get",
     "chip_compile", "chip_free", "chip_module_load", "chip_module_unload", "chip_get_function",
     "chip_function_attributes", "chip_launch", "chip_launch_seq", "chip_time_launches",
+    "chip_time_graph",
 )
 
 # Options every kernel is compiled with.  Packed-fp32 instruction selection is switched off:
@@ -124,6 +125,8 @@ def _declare(lib):
     lib.chip_launch_seq.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p]
     lib.chip_time_launches.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p, c.c_int, c.c_int, c.c_int,
                                        c.POINTER(c.POINTER(c.c_void_p)), c.POINTER(c.c_float)]
+    lib.chip_time_graph.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int,
+                                    c.POINTER(c.POINTER(c.c_void_p)), c.POINTER(c.c_float)]
 
 
 def last_error() -> str:
@@ -270,10 +273,11 @@ def launch_seq(descs, stream: int):
     _check(load().chip_launch_seq(arr, len(descs), ctypes.c_void_p(stream or 0)), "chip_launch_seq")
 
 
-def time_launches(descs, stream: int, warmup: int, iters: int, arg_sets=None) -> float:
+def time_launches(descs, stream: int, warmup: int, iters: int, arg_sets=None, graph_batch: int = 0) -> float:
     """Milliseconds per pass of the launch sequence, measured with HIP events on ``stream``.
     ``arg_sets``: optional list (one entry per rotation set) of lists of ``PackedArgs`` (one
-    per launch in ``descs``)."""
+    per launch in ``descs``).  ``graph_batch`` > 0: capture that many passes into one HIP graph
+    and time replays of it (at least ``iters`` passes in total) instead of an eager launch loop."""
     arr = (LaunchDesc * len(descs))(*descs)
     ms = ctypes.c_float()
     nsets, sets_ptr = 0, None
@@ -284,6 +288,11 @@ def time_launches(descs, stream: int, warmup: int, iters: int, arg_sets=None) ->
             raise ValueError("each argument set needs one PackedArgs per launch")
         sets_arr = (ctypes.POINTER(ctypes.c_void_p) * len(flat))(*flat)
         sets_ptr = ctypes.cast(sets_arr, ctypes.POINTER(ctypes.POINTER(ctypes.c_void_p)))
+    if graph_batch:
+        rounds = max(1, -(-int(iters) // int(graph_batch)))
+        _check(load().chip_time_graph(arr, len(descs), ctypes.c_void_p(stream or 0), int(warmup), int(graph_batch),
+                                      rounds, nsets, sets_ptr, ctypes.byref(ms)), "chip_time_graph")
+        return float(ms.value)
     _check(load().chip_time_launches(arr, len(descs), ctypes.c_void_p(stream or 0), int(warmup), int(iters),
                                      nsets, sets_ptr, ctypes.byref(ms)), "chip_time_launches")
     return float(ms.value)

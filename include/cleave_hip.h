@@ -160,6 +160,19 @@ int chip_time_launches(const chip_launch_desc* seq, int n, void* stream,
                        int warmup, int iters, int nsets, void*** arg_sets,
                        float* ms_per_iter);
 
+/* The same measurement taken the way the reference takes it
+ * (`capture_launch_graph` / `replay_rounds`, python/cleave/runtime/timer.py:14-73):
+ * `warmup` eager passes, then `batch` passes of the sequence are captured into
+ * one HIP graph (kernel nodes only) and the graph is replayed `rounds` times
+ * between two hipEvents; *ms_per_iter = elapsed / (rounds * batch).  Capture and
+ * replay run on a stream this call creates (default priority) after draining
+ * `stream`, because the legacy default stream cannot be captured; the call
+ * returns with that stream drained and destroyed.  Argument rotation as in
+ * chip_time_launches (pass i of the batch uses set i % nsets). */
+int chip_time_graph(const chip_launch_desc* seq, int n, void* stream,
+                    int warmup, int batch, int rounds, int nsets,
+                    void*** arg_sets, float* ms_per_iter);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,7 +29,8 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) >= 13 and {"chip_compile", "chip_launch", "chip_launch_seq", "chip_time_launches"} <= set(names)
+    assert len(names) >= 14 and {"chip_compile", "chip_launch", "chip_launch_seq", "chip_time_launches",
+                                 "chip_time_graph"} <= set(names)
     lib = shim.load()
     for n in names:
         assert hasattr(lib, n), f"libcleave_hip.so does not export {n}"

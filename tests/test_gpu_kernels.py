@@ -213,3 +213,27 @@ def test_mla_decode_rising_maximum():
 def test_mla_decode_c4_full(tiling, split):
     fn, dt, mk = C.CASES["c4"]
     _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=tiling, split=split)
+
+
+def test_graph_replay_timer_matches_eager_results_and_time():
+    """The graph-replay timer (a fused partial + combine pair captured ``graph_batch`` times):
+    every replayed batch must leave the eager result in the output, with the program's own eager
+    launches and synchronisations between the timings, and both timers must agree on the time."""
+    fn, dt, mk = C.CASES["c2"]
+    shapes = C.FULL["c2"]
+    prog = fn.trace(dt, **shapes)
+    kernel = kernel_for(prog, template="skinny", tiling=dict(WAVES_N=1, WAVES_K=4), split=4)
+    args = [t.cuda() for t in mk(shapes, device="cpu")]
+    other = [t.cuda() for t in mk(shapes, seed=7)]
+    want = kernel(*args).clone()
+    torch.cuda.synchronize()
+    eager_ms = kernel.time(*args, warmup=3, iters=50)
+    times = []
+    for r in range(4):
+        print(f"case graph timer replay {r}", flush=True)
+        ms = kernel.time(*args, warmup=1, iters=60, graph_batch=20, rotate=[other] if r % 2 else None)
+        times.append(ms)
+        torch.cuda.synchronize()
+        assert torch.equal(kernel.last_timed_outputs[0], want)
+        assert torch.equal(kernel(*args), want)            # eager work between the replays
+    assert all(0 < t < 5 * eager_ms for t in times) and min(times) < 1.5 * eager_ms
