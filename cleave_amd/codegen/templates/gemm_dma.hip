@@ -28,6 +28,12 @@
 #define CL_GROUP_M 8
 #endif
 #define GD_XCDS 8
+#ifndef CL_SPREAD_LOADS
+#define CL_SPREAD_LOADS 0
+#endif
+#ifndef CL_ASM_LOADS
+#define CL_ASM_LOADS 0
+#endif
 static_assert(CL_BK == 64, "K steps are 64 wide (128-byte K-minor rows)");
 static_assert((GD_TM & (GD_TM - 1)) == 0 && (GD_TN & (GD_TN - 1)) == 0, "wave tiles are powers of two");
 static_assert(CL_BM % 16 == 0 && CL_BN % 16 == 0, "tiles are multiples of 16");
@@ -92,16 +98,31 @@ struct GdOperand {
     }
   }
 
-  // issue this wave's loads of one K step; `base`: the tile's first element of this step (uniform)
-  CL_METHOD void issue(const elem_t* base, elem_t* lds) const {
+  // issue this wave's i-th load of one K step; `base`: the tile's first element of this step (uniform)
+  CL_METHOD void issue_unit(int i, const elem_t* base, elem_t* lds) const {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: the LDS target goes to M0
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int u = wave + i * GD_WAVES;
-      if (UNITS % GD_WAVES == 0 || u < UNITS)
-        __builtin_amdgcn_global_load_lds((gd_gbl_void*)(reinterpret_cast<const char*>(base) + goff[i]),
-                                         (gd_lds_void*)(lds + u * 512), 16, 0, 0);
+    const int u = wave + i * GD_WAVES;
+    if (UNITS % GD_WAVES == 0 || u < UNITS) {
+#if CL_ASM_LOADS
+      // Written as assembly the load is not counted by the compiler: with the builtin in a loop
+      // its bookkeeping of LDS traffic degrades to "wait for every LDS read" (lgkmcnt(0)) before
+      // each matrix op that takes a fragment.  The kernel's own vmcnt(0) at the end of a step
+      // covers these loads.  (Measured: no faster on the large matmul, so the builtin, whose
+      // waits the compiler derives itself, stays the default.)
+      const unsigned lds_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)(lds + u * 512);
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                   :: "v"(reinterpret_cast<const char*>(base) + goff[i]), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
+                   : "memory");
+#else
+      __builtin_amdgcn_global_load_lds((gd_gbl_void*)(reinterpret_cast<const char*>(base) + goff[i]),
+                                       (gd_lds_void*)(lds + u * 512), 16, 0, 0);
+#endif
     }
+  }
+  // ... all of them
+  CL_METHOD void issue(const elem_t* base, elem_t* lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) issue_unit(i, base, lds);
   }
 };
 
@@ -227,7 +248,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // follow its first operand, so feeding B first leaves each lane with four consecutive columns
   // of one row of C.  The group barriers pin the order "GD_TN matrix ops, then the reads issued
   // under their cover" so that no LDS latency is waited for with the matrix cores idle.
-#define GD_COMPUTE(a_tile, b_tile)                                                                  \
+#define GD_COMPUTE(a_tile, b_tile, NEXT)                                                            \
   {                                                                                                 \
     elem8 af[2][GD_TM], bf[2][GD_TN];                                                               \
     _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) bf[0][j] = GD_BFRAG(b_tile, j, 0);           \
@@ -235,6 +256,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     af[1 / GD_TM][1 % GD_TM] = GD_AFRAG(a_tile, 1 % GD_TM, 1 / GD_TM);                              \
     _Pragma("unroll") for (int s = 0; s < 2; ++s) {                                                \
       _Pragma("unroll") for (int i = 0; i < GD_TM; ++i) {                                          \
+        NEXT(s * GD_TM + i)                                                                         \
         _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) acc[i][j] = mfma16(bf[s][j], af[s][i], acc[i][j]); \
         if (s * GD_TM + i + 2 < 2 * GD_TM)                                                          \
           af[(s * GD_TM + i + 2) / GD_TM][(i + 2) % GD_TM] =                                        \
@@ -243,43 +265,81 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           _Pragma("unroll") for (int j = 0; j < GD_TN; ++j)                                        \
             if (j % GD_TM == i) bf[1][j] = GD_BFRAG(b_tile, j, 1);                                  \
         }                                                                                           \
+        GD_ROW_END()                                                                                \
       }                                                                                             \
     }                                                                                               \
-    __builtin_amdgcn_sched_group_barrier(0x100, GD_B_READS * GD_TN + 2 * GD_A_READS, 0);            \
-    gd_sched_rows<0, 0>();                                                                          \
+    GD_STEP_SCHED()                                                                                 \
   }
+#if CL_SPREAD_LOADS
+// every row of matrix ops closes with a scheduling barrier: the order of the source (this row's
+// loads of the next step, its matrix ops, the fragment reads for two rows on) is the order of the
+// instruction stream
+#define GD_ROW_END() __builtin_amdgcn_sched_barrier(0);
+#define GD_STEP_SCHED()
+#else
+#define GD_ROW_END()
+#define GD_STEP_SCHED()                                                                             \
+    __builtin_amdgcn_sched_group_barrier(0x100, GD_B_READS * GD_TN + 2 * GD_A_READS, 0);            \
+    gd_sched_rows<0, 0>();
+#endif
   // everything this wave loaded has landed; after the barrier, everything every wave loaded
 #define GD_STEP_END()                           \
   __builtin_amdgcn_s_waitcnt(0x0F70);           \
   __syncthreads();
-  // the loads of a step are issued before the matrix work they overlap with, and stay there
+  // The loads of the next step.  A wave that issues a load while the path from L2 into the
+  // compute unit (64 bytes per clock) is busy stands still, matrix ops and all; every wave
+  // issuing its whole share at the top of a step stops the matrix cores for the length of the
+  // transfer.  CL_SPREAD_LOADS: row r of a step's matrix work is preceded by the r-th slice of
+  // the wave's loads instead (measured: no faster on the large matmul; off by default).
 #ifdef CL_DBG_NODMA
 #define GD_ISSUE(kt, a_lds, b_lds)
+#define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)
 #else
 #define GD_ISSUE(kt, a_lds, b_lds)                              \
   opa.issue(a_base + (i64)(kt) * a_step, a_lds);                \
   opb.issue(b_base + (i64)(kt) * b_step, b_lds);                \
   __builtin_amdgcn_sched_barrier(0);
+#define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)                                                         \
+  {                                                                                                 \
+    constexpr int ua_ = decltype(opa)::PER, ub_ = decltype(opb)::PER;                               \
+    constexpr int per_row_ = (ua_ + ub_ + 2 * GD_TM - 1) / (2 * GD_TM);                             \
+    _Pragma("unroll") for (int q_ = (r) * per_row_; q_ < ((r) + 1) * per_row_; ++q_) {             \
+      if (q_ < ua_) opa.issue_unit(q_, a_base + (i64)(kt) * a_step, a_lds);                         \
+      else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, b_base + (i64)(kt) * b_step, b_lds);        \
+    }                                                                                               \
+  }
 #endif
 #ifdef CL_DBG_NOCOMPUTE
 #undef GD_COMPUTE
-#define GD_COMPUTE(a_tile, b_tile)
+#define GD_COMPUTE(a_tile, b_tile, NEXT)
 #endif
+#define GD_NO_NEXT(r)
 
   // Two steps per trip, one on each stage, with no branch inside: the loads issued in the second
   // half are clamped onto the last step (for an even step count the final trip fetches that step
   // once more into the idle stage, which nobody reads).
   GD_ISSUE(0, gd_a0, gd_b0)
   GD_STEP_END()
+#if CL_SPREAD_LOADS
+#define GD_NEXT_1(r) GD_ISSUE_SLICE(r, kt + 1, gd_a1, gd_b1)
+#define GD_NEXT_0(r) GD_ISSUE_SLICE(r, (kt + 2 < KT ? kt + 2 : KT - 1), gd_a0, gd_b0)
   for (int kt = 0; kt + 1 < KT; kt += 2) {
-    GD_ISSUE(kt + 1, gd_a1, gd_b1)
-    GD_COMPUTE(gd_a0, gd_b0)
+    GD_COMPUTE(gd_a0, gd_b0, GD_NEXT_1)
     GD_STEP_END()
-    GD_ISSUE((kt + 2 < KT ? kt + 2 : KT - 1), gd_a0, gd_b0)
-    GD_COMPUTE(gd_a1, gd_b1)
+    GD_COMPUTE(gd_a1, gd_b1, GD_NEXT_0)
     GD_STEP_END()
   }
-  if constexpr (KT % 2 == 1) GD_COMPUTE(gd_a0, gd_b0)     // an odd number of steps ends on stage 0
+#else
+  for (int kt = 0; kt + 1 < KT; kt += 2) {
+    GD_ISSUE(kt + 1, gd_a1, gd_b1)
+    GD_COMPUTE(gd_a0, gd_b0, GD_NO_NEXT)
+    GD_STEP_END()
+    GD_ISSUE((kt + 2 < KT ? kt + 2 : KT - 1), gd_a0, gd_b0)
+    GD_COMPUTE(gd_a1, gd_b1, GD_NO_NEXT)
+    GD_STEP_END()
+  }
+#endif
+  if constexpr (KT % 2 == 1) GD_COMPUTE(gd_a0, gd_b0, GD_NO_NEXT)     // an odd number of steps ends on stage 0
 
   // ---- epilogue: acc[i][j][r] = C[m0 + am + 16 i + c][n0 + bn + 16 j + 4 g + r] ----------------
 #pragma unroll
