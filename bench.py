@@ -281,7 +281,7 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
 
 # ----------------------------------------------------------------------------- shipped paged operators
 def run_dynamic(names=None):
-    """The registry's paged GQA decode operators (bf16) over their captured workload axes:
+    """The registry's paged decode operators (GQA and MLA, bf16) over their captured workload axes:
     ``compile`` searches tilings and split-KV pairs, validates every candidate on every workload
     against the torch reference and times the valid ones; with a split pair and a single kernel
     it calibrates which to run per workload.  Reported: the best geomean, per-workload times of
@@ -301,8 +301,11 @@ def run_dynamic(names=None):
     for name, op in OPERATORS.items():
         if names and name not in names:
             continue
-        hq, hkv, d = op.dims[:3]
-        fn = C.paged_decode_op(hq, hkv, d, op.page_size, dtype=cl.bf16, name=name)
+        if op.is_mla:
+            fn = C.mla_paged_decode_op(*op.dims[:3], dtype=cl.bf16, name=name)
+        else:
+            hq, hkv, d = op.dims[:3]
+            fn = C.paged_decode_op(hq, hkv, d, op.page_size, dtype=cl.bf16, name=name)
         t0 = time.perf_counter()
         with contextlib.redirect_stdout(sys.stderr):
             kernel = cleave_amd.compile(fn, schedule=P.ScheduleConfig(topk=3), split=cl.Split("kv_len", (4, 8, 16)),
@@ -370,6 +373,7 @@ def main():
     ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
+    ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")
     ap.add_argument("--kernels", default=None, metavar="DIR",
                     help="save each op's selected kernel source under DIR; when DIR already holds one, time it "
                          "without searching (so a profiler sees only the timed launches)")
@@ -393,8 +397,8 @@ def main():
             results[name] = run_copy(max(10, args.steps // 4), max(2, args.warmup // 4))
             continue
         if name == "dyn":
-            results[name] = {"op": "dyn", "workload": "registry paged GQA decode operators over their captured axes",
-                             "operators": run_dynamic()}
+            results[name] = {"op": "dyn", "workload": "registry paged decode operators (GQA, MLA) over their captured axes",
+                             "operators": run_dynamic([n for n in args.dyn_ops.split(",") if n] or None)}
             continue
         if name == "c5":
             results[name] = run_paged(max(10, args.steps // 4), max(2, args.warmup // 4), not args.no_cpu, args.kernels)

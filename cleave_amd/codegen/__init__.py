@@ -391,6 +391,8 @@ class HipCodeGen:
 
     def _emit_mla_decode(self, unit, plan, params, partial, combine, fused):
         p, t, op = plan.problem, plan.tiling, plan.operands
+        if p.get("paged"):
+            return self._emit_mla_paged(unit, plan, params, partial, combine, fused)
         total_rows = p["batch"] * p["heads"]
         emit_lse = bool(p.get("emit_lse"))
         self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], total_rows, emit_lse)
@@ -432,6 +434,35 @@ class HipCodeGen:
             entry, args = self._combine_args
             unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)
 
+
+    def _emit_mla_paged(self, unit, plan, params, partial, combine, fused):
+        """Paged MLA decode (token table, page size 1): one wave per (work item, 16 heads); work
+        items are requests (single kernel) or table slices of at most ``chunk_pages`` entries
+        (split form, folded by the chunked combine)."""
+        p, t, op = plan.problem, plan.tiling, plan.operands
+        batch_name = p["dim_names"]["batch"]
+        emit_lse = bool(p.get("emit_lse"))
+        self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], f"(batch * {p['heads']})", emit_lse)
+        if p["heads"] % 16 or p["ckv"] % 64 or p["kpe"] % 64:
+            raise CodegenError("paged MLA decode needs heads % 16 == 0 and latent / rope widths that are multiples of 64")
+        chunked = (plan.split_factor or 1) > 1
+        if chunked and not t.get("CHUNK_PAGES"):
+            raise CodegenError("the split form of paged MLA decode is the chunked one (CHUNK_PAGES)")
+        for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_CHUNKED", chunked),
+                     ("CL_CHUNK_PAGES", chunked), ("CL_Q_HEADS", p["heads"])):
+            unit.define(k, v)
+        if "LDS_AHEAD" in t:
+            unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
+        for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE"),
+                            ("INDPTR", "CL_ARG_INDPTR"), ("INDICES", "CL_ARG_INDICES")):
+            unit.define(macro, op[role])
+        unit.templates += ["mla_paged_decode.hip", "attn_combine.hip"]
+        if partial:
+            items = f"ceildiv({p['dim_names']['n_idx']}, chunk_pages) + {batch_name}" if chunked else batch_name
+            unit.launch(ENTRY, (items, p["heads"] // 16, 1), 64, 0, self._partial_args)
+        if combine:
+            entry, args = self._combine_args
+            unit.launch(entry, (f"ceildiv(({batch_name} * {p['heads']}) * {p['ckv'] // 4}, 256)", 1, 1), 256, 0, args)
 
     def _emit_mla_decode_xw(self, unit, plan, partial, combine, total_rows):
         """The 64-heads-per-workgroup kernel: score product shared out by (token half, head half),

@@ -1,0 +1,306 @@
+// ---- paged MLA decode: per request, out = softmax((q kv^T + q_pe k_pe^T) * sm_scale) kv with the
+// latent (kv) and rope (k_pe) rows gathered through a token table (page size 1) ----------------
+//
+// One wave per work item and 16-head group.  An item is a request (single kernel) or, with
+// CL_CHUNKED, a slice of at most `chunk_pages` table entries of one request (a new item starts
+// at every multiple of chunk_pages entries and at every request boundary, as in the chunked GQA
+// decode; the combine folds a request's items).  The wave walks its tokens in steps of 32: the
+// latent and rope rows of a step go from global memory straight into LDS (16 bytes per lane, the
+// row of every lane looked up in the table) as the token-major image of the dense MLA kernel:
+//   tile  [D/64][32][64]   64-feature panels, 128-byte token rows, 16-byte chunk ^ (token & 6)
+// two images, the next step's rows in flight while the matrix cores work on the current one.
+// Table entries are read 256 at a time into four registers per lane (entry 64 k + lane in
+// register k) one window ahead; a lane fetches the entry of the row it loads with a cross-lane
+// read.  Scores, softmax and value product are the dense kernel's (16 heads per wave, Q fragments
+// resident, fixed softmax reference raised outside the hot loop).
+//
+//   CL_HEADS (multiple of 16)  CL_CKV  CL_KPE (multiples of 64)  CL_CHUNKED
+//   run-time: batch, num_pages, n_idx [, chunk_pages]; scalar sm_scale (> 0 or not: the
+//   maximum is taken over scaled scores)
+
+#define MP_STEP 32
+#define MP_D (CL_CKV + CL_KPE)
+#define MP_PANEL (MP_STEP * 64)
+#define MP_PANELS (MP_D / 64)
+#define MP_LAT_PANELS (CL_CKV / 64)
+#define MP_TILE (MP_PANELS * MP_PANEL)
+#define MP_KJ (MP_D / 32)
+#define MP_FB (CL_CKV / 16)
+#define MP_WINDOW 256                          // table entries held in registers at a time
+#define MP_RESCALE_STEP 8.0f
+#ifndef CL_LDS_AHEAD
+#define CL_LDS_AHEAD 8
+#endif
+static_assert(CL_CKV % 64 == 0 && CL_KPE % 64 == 0, "latent and rope widths are whole 64-feature panels");
+static_assert(CL_HEADS % 16 == 0, "16 heads per wave");
+
+__shared__ __attribute__((aligned(1024))) elem_t mp_tiles[2 * MP_TILE];
+
+typedef short mp_s16x4 __attribute__((ext_vector_type(4)));
+typedef short mp_s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) mp_s16x4 mp_lds_s16x4;
+
+CL_DEVICE int mp_swz(int token) { return token & 6; }
+CL_DEVICE int mp_clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// 16 bytes per lane, global -> LDS: the wave's 64 lanes fill 1 KiB starting at LDS byte address
+// `lds_byte` + OFF (wave-uniform), lane l from `gptr` + OFF.  Not counted by the compiler: the
+// kernel waits for it itself.
+template <int OFF>
+CL_DEVICE void mp_dma16(const void* gptr, unsigned lds_byte) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory");
+}
+
+// panels P.. of row group RG (token rows 8 RG + lane / 8 of the step) from this lane's row
+template <int P>
+CL_DEVICE void mp_issue_row_group(const char* lat_src, const char* pe_src, unsigned group_byte) {
+  if constexpr (P < MP_PANELS) {
+    constexpr int OFF = 128 * (P < MP_LAT_PANELS ? P : P - MP_LAT_PANELS);
+    mp_dma16<OFF>(P < MP_LAT_PANELS ? lat_src : pe_src, group_byte + (unsigned)(P * MP_PANEL * 2) - OFF);
+    mp_issue_row_group<P + 1>(lat_src, pe_src, group_byte);
+  }
+}
+
+#if CL_EMIT_PARTIAL
+extern "C" __global__ void __launch_bounds__(64)
+CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
+  const int lane = threadIdx.x & 63;
+  const int c = lane & 15, g = lane >> 4;
+  const int head0 = 16 * blockIdx.y;
+#if CL_CHUNKED
+  const int item = blockIdx.x;
+  // the request whose items include `item`: the last b with b + indptr[b] / C <= item
+  int req = 0;
+  {
+    int hi_b = batch - 1;
+    while (req < hi_b) {
+      const int mid = (req + hi_b + 1) >> 1;
+      if (mid + mp_clamp(CL_ARG_INDPTR[mid], 0, n_idx) / chunk_pages <= item) req = mid;
+      else hi_b = mid - 1;
+    }
+  }
+  const int p0 = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx), p1 = mp_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx);
+  const int chunk = item - req;
+  const int lo = p0 > chunk * chunk_pages ? p0 : chunk * chunk_pages;
+  const int hi = p1 < (chunk + 1) * chunk_pages ? p1 : (chunk + 1) * chunk_pages;
+  if (hi <= lo) return;                               // an index no (chunk, request) pair maps to
+#else
+  const int req = blockIdx.x;
+  const int lo = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx);
+  int hi = mp_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx);
+  hi = hi > lo ? hi : lo;
+#endif
+  const int n_tok = hi - lo;
+  const int n_steps = (n_tok + MP_STEP - 1) / MP_STEP;
+  const float scale_log2e = sm_scale * 1.4426950408889634f;
+  const i64 qrow = (i64)req * CL_HEADS + head0 + c;
+  const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)mp_tiles;
+
+  float m_run = CL_NEG_BIG;            // softmax reference point of head c (log2 domain), uniform over g
+  f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};  // every component: sum of the weights of head c
+  f32x4 acc[MP_FB];                    // acc[fb][r] = O[head c][16 fb + 4 g + r]
+#pragma unroll
+  for (int fb = 0; fb < MP_FB; ++fb) acc[fb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  if (n_steps > 0) {
+    elem8 ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ones[i] = to_elem(1.0f);
+
+    // table entries of a 256-entry window: register k holds entry 64 k + lane (positions past the
+    // item's end repeat its last entry; ids outside the pool are clamped into it)
+    auto load_window = [&](int w, int (&ids)[4]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        int pos = lo + w * MP_WINDOW + 64 * k + lane;
+        pos = pos < hi - 1 ? pos : hi - 1;
+        ids[k] = mp_clamp(CL_ARG_INDICES[pos], 0, num_pages - 1);
+      }
+    };
+    int ids_cur[4], ids_next[4];
+    load_window(0, ids_cur);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) ids_next[k] = ids_cur[k];
+
+    // the rows of step s (its window's entries in `ids`) into image s % 2: lane l loads token row
+    // 8 rg + l / 8 of the step, the chunk that belongs in slot l % 8 of that row
+    auto issue_step = [&](int s, const int (&ids)[4]) __attribute__((always_inline)) {
+      const int in_window = s % (MP_WINDOW / MP_STEP);
+      const int k = in_window >> 1;
+      const int held = k == 0 ? ids[0] : k == 1 ? ids[1] : k == 2 ? ids[2] : ids[3];
+      const unsigned stage_byte = tiles_byte + (unsigned)((s & 1) * MP_TILE * 2);
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int r = 8 * rg + (lane >> 3);
+        const int src_lane = 32 * (in_window & 1) + r;
+        const int id = __builtin_amdgcn_ds_bpermute(src_lane << 2, held);
+        const int chunk = (lane & 7) ^ mp_swz(r);
+        const char* lat_src = reinterpret_cast<const char*>(CL_ARG_KV) + ((i64)id * CL_CKV + 8 * chunk) * 2;
+        const char* pe_src = reinterpret_cast<const char*>(CL_ARG_KPE) + ((i64)id * CL_KPE + 8 * chunk) * 2;
+        mp_issue_row_group<0>(lat_src, pe_src, stage_byte + (unsigned)(rg * 1024));
+      }
+    };
+    issue_step(0, ids_cur);
+
+    // Q fragments (B operand of the score product): lane (c, g) holds q[head c][32 j + 8 g .. +8]
+    elem8 qf[MP_KJ];
+#pragma unroll
+    for (int j = 0; j < MP_KJ; ++j) {
+      const int col = 32 * j + 8 * g;
+      const elem_t* src = col < CL_CKV ? CL_ARG_Q + qrow * CL_CKV + col : CL_ARG_QPE + qrow * CL_KPE + (col - CL_CKV);
+      qf[j] = as_elem8(ld16(src));
+    }
+
+    // this lane's operand offsets inside an image (elements):
+    //   score operand: token row c of a 16-token half, chunk g of a 32-feature block
+    //   value operand: its 8-byte piece of the 4 (token) x 16 (feature) patch of lane group g
+    const int a_lo = c * 64 + ((g ^ mp_swz(c)) << 3);
+    const int vtok = 4 * g + (c >> 2);
+    const int v_lo = vtok * 64 + (((((c & 3) >> 1)) ^ mp_swz(vtok)) << 3) + 4 * (c & 1);
+
+    // Softmax as in the dense kernel: weights are exp2(score - m_run) against a fixed reference,
+    // row sums by one more matrix op against ones, nothing crosses lanes in the hot loop; a
+    // score more than MP_RESCALE_STEP above the reference leaves the loop before the step is
+    // consumed, the cold block raises the reference, rescales (l, O) and re-enters at the step.
+    int step = 0;
+    bool front_done = false;           // the loads of `step` have been waited for and the next ones issued
+    for (;;) {
+      bool raise_any = false;
+      float mxl = CL_NEG_BIG;
+      while (step < n_steps) {
+        if (!front_done) {
+          // everything in flight is step `step` (and table entries read a window ahead): wait, then
+          // send the next step's rows into the other image (its last readers were the matrix
+          // ops of step - 1, all issued)
+          __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+          __syncthreads();
+          if (step % (MP_WINDOW / MP_STEP) == 0 && (step / (MP_WINDOW / MP_STEP) + 1) * MP_WINDOW < n_tok)
+            load_window(step / (MP_WINDOW / MP_STEP) + 1, ids_next);
+          if (step + 1 < n_steps) {
+            if ((step + 1) % (MP_WINDOW / MP_STEP) == 0) {
+#pragma unroll
+              for (int k = 0; k < 4; ++k) ids_cur[k] = ids_next[k];
+            }
+            issue_step(step + 1, ids_cur);
+          }
+          front_done = true;
+        }
+        const elem_t* tile = mp_tiles + (step & 1) * MP_TILE;
+
+        // scores^T: rows = tokens 16 h + (0..15), columns = heads
+        f32x4 st[2];
+        st[0] = st[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < MP_KJ; ++j) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const elem8 a = *reinterpret_cast<const elem8*>(tile + (j >> 1) * MP_PANEL + 16 * h * 64 +
+                                                            (a_lo ^ ((4 * (j & 1)) << 3)));
+            st[h] = mfma16(a, qf[j], st[h]);
+          }
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, CL_LDS_AHEAD, 0);
+#pragma unroll
+        for (int n = 0; n < 2 * MP_KJ - CL_LDS_AHEAD; ++n) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, CL_LDS_AHEAD, 0);
+
+        // scaled scores; tokens past the item's end weigh nothing
+        const int t0 = step * MP_STEP;
+        float v = CL_NEG_BIG;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            st[h][r] = t0 + 16 * h + 4 * g + r < n_tok ? st[h][r] * scale_log2e : CL_NEG_BIG;
+            v = fmaxf(v, st[h][r]);
+          }
+        mxl = v;
+        if (step == 0 && m_run < 0.5f * CL_NEG_BIG) {
+          // first step (nothing accumulated yet): its own maximum is the reference
+          float mx = mxl;
+          mx = fmaxf(mx, lane_xor(mx, lane, 16));
+          mx = fmaxf(mx, lane_xor(mx, lane, 32));
+          m_run = mx;
+        } else if (__builtin_amdgcn_ballot_w64(mxl > m_run + MP_RESCALE_STEP)) {   // wave-uniform
+          raise_any = true;
+          break;
+        }
+
+        elem8 pf;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) pf[4 * h + r] = to_elem(fast_exp2(st[h][r] - m_run));
+
+        // out^T block fb: rows = features 16 fb + (0..15), slots = tokens 4 g + (0..3), 16 + 4 g + (0..3)
+        l_acc = mfma16(ones, pf, l_acc);
+#pragma unroll
+        for (int fb = 0; fb < MP_FB; ++fb) {
+          const elem_t* p = tile + (fb >> 2) * MP_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
+          const mp_s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((mp_lds_s16x4*)(p));
+          const mp_s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((mp_lds_s16x4*)(p + 16 * 64));
+          const elem8 a = __builtin_bit_cast(elem8, (mp_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+          acc[fb] = mfma16(a, pf, acc[fb]);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, CL_LDS_AHEAD, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+        for (int n = 0; n < MP_FB - CL_LDS_AHEAD / 2; ++n) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, CL_LDS_AHEAD / 2, 0);
+
+        ++step;
+        front_done = false;
+      }
+      if (!raise_any) break;
+      // cold: raise the reference and rescale what has been accumulated
+      float mx = mxl;
+      mx = fmaxf(mx, lane_xor(mx, lane, 16));
+      mx = fmaxf(mx, lane_xor(mx, lane, 32));
+      const bool up = mx > m_run + MP_RESCALE_STEP;
+      const float m_new = up ? mx : m_run;
+      const float alpha = up ? fast_exp2(m_run - m_new) : 1.0f;
+      m_run = m_new;
+      l_acc *= alpha;
+#pragma unroll
+      for (int fb = 0; fb < MP_FB; ++fb) acc[fb] *= alpha;
+    }
+    // no load may still be on its way into LDS when the workgroup ends
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+  }
+
+  // ---- write this wave's heads ------------------------------------------------------------------
+  const float l = l_acc[0];
+  const int f0 = 4 * g;
+#if CL_CHUNKED
+  const i64 prow = (i64)item * CL_HEADS + head0 + c;
+#pragma unroll
+  for (int fb = 0; fb < MP_FB; ++fb)
+    *reinterpret_cast<f32x4*>(CL_ARG_PO + prow * CL_CKV + f0 + 16 * fb) = acc[fb];
+  if (g == 0) {
+    CL_ARG_PM[prow] = m_run;
+    CL_ARG_PL[prow] = l;
+  }
+#else
+  // an empty request has l == 0: the floor turns 0/0 into 0 and its lse is -inf
+  const float inv = 1.0f / fmaxf(l, 1.0e-30f);
+  elem_t* dst_row = CL_ARG_OUT + qrow * CL_CKV;
+#if CL_EMIT_LSE
+  if (g == 0) CL_ARG_LSE[qrow] = l > 0.f ? m_run + fast_log2(l) : CL_NEG_INF;
+#endif
+#pragma unroll
+  for (int fb = 0; fb < MP_FB; ++fb) {
+    elem4 y;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[fb][r] * inv);
+    *reinterpret_cast<elem4*>(dst_row + f0 + 16 * fb) = y;
+  }
+#endif
+}
+#endif  // CL_EMIT_PARTIAL

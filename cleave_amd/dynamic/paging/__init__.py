@@ -1,7 +1,8 @@
-"""Paged access layers over the dense decode-attention template."""
+"""Paged access layers over the dense decode-attention and MLA decode templates."""
 
-from .apply import (DenseAttention, apply_paging, apply_paging_split, build_split_decode, can_page, paging_accept,
-                    read_dense_attention, read_dense_combine, read_dense_partial)
+from .apply import (DenseAttention, DenseMLA, apply_paging, apply_paging_split, build_split_decode, can_page,
+                    paging_accept, read_dense, read_dense_attention, read_dense_combine, read_dense_mla,
+                    read_dense_partial)
 from .errors import InvalidSpec, NotDenseAttention, PagingRefusal, UnsupportedTiling
 from .kinds import (BUILT_KINDS, CAUSAL_KINDS, KINDS, MLA_KINDS, MLA_PAGED_DECODE, MLA_PAGED_PREFILL_CAUSAL,
                     PAGED_DECODE, PAGED_DECODE_SLAB, PAGED_KINDS, PAGED_PREFILL_CAUSAL, PARTIAL_MAX, PARTIAL_ROWSUM,

@@ -18,7 +18,7 @@ from dataclasses import dataclass
 
 from ...schedule.plan import KernelPlan, ParamSpec
 from .errors import NotDenseAttention, UnsupportedTiling
-from .kinds import BUILT_KINDS, PAGED_DECODE, PAGED_DECODE_SLAB
+from .kinds import BUILT_KINDS, MLA_PAGED_DECODE, PAGED_DECODE, PAGED_DECODE_SLAB
 from .specs import CombineTiling, MLASpec, PagingSpec
 
 KV_STEP = 32  # tokens one wave consumes per step of the decode template
@@ -43,6 +43,49 @@ class DenseAttention:
     # `waves` is then the kv-head count) instead of `split` equal parts per request.  -1 lets the
     # launch choose the size from the page-table length so that one item lands on each compute unit.
     chunk_pages: int = 0
+
+
+@dataclass(frozen=True)
+class DenseMLA:
+    """What the access layer reads off a scheduled dense MLA decode plan: the operator's widths;
+    the paged kernel has one tiling (one wave per 16 heads and work item, 32-token steps)."""
+
+    heads: int
+    ckv: int
+    kpe: int
+    dtype: str
+    out_dtype: str
+    kv_tile: int = KV_STEP
+    n_threads: int = 64
+    split: int | None = None
+    # split form: table entries per work item; -1 lets the launch choose the size from the
+    # table length so that two items land on each compute unit
+    chunk_pages: int = -1
+
+    @property
+    def query_rows(self) -> int:
+        return self.heads
+
+    @property
+    def head_dim(self) -> int:
+        return self.ckv
+
+
+def read_dense_mla(plan: KernelPlan) -> DenseMLA:
+    if not isinstance(plan, KernelPlan) or plan.template != "mla_decode" or plan.family != "mla":
+        raise NotDenseAttention("expected a scheduled dense MLA decode plan (template mla_decode)")
+    p = plan.problem
+    if p.get("paged"):
+        raise NotDenseAttention("the plan is already paged")
+    if p["batch"] != 1:
+        raise NotDenseAttention("the dense body of a paged MLA operator is one request: q (H, D), kv (SKV, D)")
+    return DenseMLA(heads=p["heads"], ckv=p["ckv"], kpe=p["kpe"], dtype=plan.dtype, out_dtype=plan.dtype,
+                    split=plan.split_factor)
+
+
+def read_dense(plan: KernelPlan, spec):
+    """The dense tiling object of ``plan`` for the layer ``spec`` asks for."""
+    return read_dense_mla(plan) if isinstance(spec, MLASpec) else read_dense_attention(plan)
 
 
 def read_dense_attention(plan: KernelPlan) -> DenseAttention:
@@ -77,14 +120,20 @@ def read_dense_combine(plan: KernelPlan) -> CombineTiling:
     return CombineTiling(split=int(plan.split_factor))
 
 
-def _check_tiling(spec, dense: DenseAttention, split: bool = False) -> None:
-    if isinstance(spec, MLASpec):
-        raise UnsupportedTiling("the paged MLA layer is not built by this back end yet (dense MLA decode is)")
+def _check_tiling(spec, dense, split: bool = False) -> None:
+    if isinstance(spec, MLASpec) != isinstance(dense, DenseMLA):
+        raise NotDenseAttention("the spec and the dense plan are not of the same operator family (GQA vs MLA)")
     if spec.kind not in BUILT_KINDS:
         raise UnsupportedTiling(f"the {spec.kind!r} layer is not built by this back end yet "
                                 f"(built: {', '.join(BUILT_KINDS)})")
-    if split and spec.kind not in (PAGED_DECODE, PAGED_DECODE_SLAB):
+    if split and spec.kind not in (PAGED_DECODE, PAGED_DECODE_SLAB, MLA_PAGED_DECODE):
         raise UnsupportedTiling(f"split-KV is a decode transformation; got the {spec.kind!r} layer")
+    if isinstance(spec, MLASpec):
+        if dense.heads != spec.num_qo_heads:
+            raise UnsupportedTiling(f"the dense body has {dense.heads} heads, the spec {spec.num_qo_heads}")
+        if dense.ckv % 64 or dense.kpe % 64:
+            raise UnsupportedTiling(f"latent / rope widths {dense.ckv} / {dense.kpe} are not multiples of 64")
+        return
     if dense.query_rows < spec.group:
         raise UnsupportedTiling(f"a block's query tile holds {dense.query_rows} rows but the head group needs "
                                 f"{spec.group}; re-tile with at least {spec.group} query rows")
@@ -156,9 +205,88 @@ def chunk_pages_expr(spec, chunk_pages: int) -> str:
             f"max(1, {cus} - {spec.batch_dim}))))")
 
 
+# ----------------------------------------------------------------------------- paged MLA decode
+# Parameter order of the reference's operator (``python/cleave/dynamic/reference.py:282-295``):
+# q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, sm_scale, [partials], out, lse.
+def _mla_params(spec: MLASpec, dense: DenseMLA):
+    dt, b, pages = dense.dtype, spec.batch_dim, spec.pages_dim
+    ph = lambda n: f"PlaceHolder_{n}"  # noqa: E731
+    params = [
+        ParamSpec(ph(spec.query_inputs[0]), dt, (b, spec.num_qo_heads, dense.ckv), "input"),
+        ParamSpec(ph(spec.query_inputs[1]), dt, (b, spec.num_qo_heads, dense.kpe), "input"),
+        ParamSpec(ph(spec.cache_inputs[0]), dt, (pages, spec.page_size, dense.ckv), "input"),
+        ParamSpec(ph(spec.cache_inputs[1]), dt, (pages, spec.page_size, dense.kpe), "input"),
+        ParamSpec(ph(spec.indptr_input), "int32", (spec.indptr_dim,), "input"),
+        ParamSpec(ph(spec.index_input), "int32", (spec.index_dim,), "input"),
+        ParamSpec(spec.scale_input, "float32", (), "scalar"),
+    ]
+    operands = {"Q": params[0].name, "QPE": params[1].name, "KV": params[2].name, "KPE": params[3].name,
+                "INDPTR": params[4].name, "INDICES": params[5].name}
+    return params, operands
+
+
+def _mla_outputs(spec: MLASpec, dense: DenseMLA):
+    outs = [ParamSpec("OutputNode_0", dense.out_dtype, (spec.batch_dim, spec.num_qo_heads, dense.ckv), "output")]
+    operands = {"OUT": "OutputNode_0"}
+    if spec.emit_lse:
+        outs.append(ParamSpec("OutputNode_1", "float32", (spec.batch_dim, spec.num_qo_heads), "output"))
+        operands["OUT1"] = "OutputNode_1"
+    return outs, operands
+
+
+def mla_chunk_pages_expr(spec: MLASpec, chunk_pages: int) -> str:
+    """Launch-time item size of the split form: the fixed value, or for -1 the size that puts about
+    two items on every compute unit (two one-wave workgroups fit one), at least one 32-token step."""
+    if chunk_pages > 0:
+        return str(chunk_pages)
+    from ...core.target import current_target
+
+    cus = current_target().arch.compute_units
+    return f"max(32, min(512, ceildiv({spec.index_dim}, max(1, {2 * cus} - {spec.batch_dim}))))"
+
+
+def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None) -> KernelPlan:
+    dyn = (spec.batch_dim, spec.pages_dim, spec.index_dim)
+    problem = {"paged": True, "page_size": spec.page_size, "heads": spec.num_qo_heads, "ckv": dense.ckv,
+               "kpe": dense.kpe, "emit_lse": bool(spec.emit_lse), "batch": None, "skv": 0, "scale": 1.0,
+               "dim_names": {"batch": spec.batch_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim}}
+    tiling, extra = {}, {}
+    if split:
+        tiling["CHUNK_PAGES"] = dense.chunk_pages
+        extra["derived_dims"] = [("chunk_pages", mla_chunk_pages_expr(spec, dense.chunk_pages))]
+    return KernelPlan(template="mla_decode", role=role, family="mla", dtype=dense.dtype, extra=extra, problem=problem,
+                      tiling=tiling, params=params, operands=operands, split_factor=split, dyn_dims=dyn,
+                      n_threads=dense.n_threads, label=f"kv={dense.kv_tile} q={dense.heads} thr={dense.n_threads}")
+
+
+def _mla_split_decode(spec: MLASpec, dense: DenseMLA, split: int) -> list:
+    if dense.chunk_pages == 0 or dense.chunk_pages < -1:
+        raise UnsupportedTiling("the split form of paged MLA decode cuts the token table into items: chunk_pages "
+                                "must be positive or -1 (chosen at launch)")
+    params, operands = _mla_params(spec, dense)
+    b, h, d = spec.batch_dim, spec.num_qo_heads, dense.ckv
+    items = f"ceildiv({spec.index_dim}, chunk_pages) + {b}"
+    bufs = [("PM", (items, h)), ("PL", (items, h)), ("PO", (items, h, d))]
+    part_outs = [ParamSpec(f"OutputNode_{i}", "float32", shape, "output") for i, (_, shape) in enumerate(bufs)]
+    part_ops = {**operands, **{name: p.name for (name, _), p in zip(bufs, part_outs)}}
+    partial = _mla_plan(spec, dense, "partial", params + part_outs, part_ops, split)
+    comb_ins = [ParamSpec(f"PlaceHolder_{name}", "float32", shape, "input") for name, shape in bufs]
+    outs, out_ops = _mla_outputs(spec, dense)
+    indptr = next(q for q in params if q.name == operands["INDPTR"])
+    comb_ops = {**{name: p.name for (name, _), p in zip(bufs, comb_ins)}, **out_ops, "INDPTR": indptr.name}
+    combine = _mla_plan(spec, dense, "combine", comb_ins + [indptr] + outs, comb_ops, split)
+    return [partial, combine]
+
+
 def apply_paging(plan: KernelPlan, spec) -> KernelPlan:
     """A single paged decode kernel at ``plan``'s tiling."""
     spec.validate()
+    if isinstance(spec, MLASpec):
+        dense = read_dense_mla(plan)
+        _check_tiling(spec, dense)
+        params, operands = _mla_params(spec, dense)
+        outs, out_ops = _mla_outputs(spec, dense)
+        return _mla_plan(spec, dense, "main", params + outs, {**operands, **out_ops})
     dense = read_dense_attention(plan)
     _check_tiling(spec, dense)
     params, operands = _paged_params(spec, dense)
@@ -174,6 +302,8 @@ def build_split_decode(spec, dense: DenseAttention, split: int, comb: CombineTil
         raise UnsupportedTiling(f"the combine tiling is for {comb.split} splits but the partial makes {split}")
     comb.validate(dense.head_dim)
     _check_tiling(spec, dense, split=True)
+    if isinstance(spec, MLASpec):
+        return _mla_split_decode(spec, dense, split)
     params, operands = _paged_params(spec, dense)
     b, h, d = spec.batch_dim, spec.num_qo_heads, dense.head_dim
     # split-major partials: one request's splits sit one stride apart
@@ -207,6 +337,12 @@ def apply_paging_split(plans, spec) -> list:
         raise NotDenseAttention(f"expected a [partial, combine] pair, got {len(plans)} plans")
     partial, combine = plans
     spec.validate()
+    if isinstance(spec, MLASpec):
+        dense = read_dense_mla(partial)
+        if partial.role != "partial" or not partial.split_factor:
+            raise NotDenseAttention("expected the partial plan of a split pair")
+        comb = read_dense_combine(combine)
+        return build_split_decode(spec, dense, int(partial.split_factor), comb)
     dense, split = read_dense_partial(partial)
     comb = read_dense_combine(combine)
     if comb.split != split:
@@ -219,7 +355,7 @@ def can_page(plan, spec) -> bool:
 
     try:
         spec.validate()
-        _check_tiling(spec, read_dense_attention(plan))
+        _check_tiling(spec, read_dense(plan, spec))
     except PagingRefusal:
         return False
     return True

@@ -145,3 +145,66 @@ def gqa_paged_decode_reference(dims, kv_lens, page_size=1, dtype=None):
         return [out, lse]
 
     return reference
+
+
+# ----------------------------------------------------------------------------- MLA paged decode
+def _mla_attend_rows(qn, qp, kc, kp, scale, keep=None):
+    """MLA over a block of query rows (``python/cleave/dynamic/reference.py:108-126``): ``qn``
+    (n_q, heads, ckv), ``qp`` (n_q, heads, kpe), ``kc`` (n_kv, ckv) both keys and values, ``kp``
+    (n_kv, kpe) -> out fp32 (n_q, heads, ckv), base-2 lse (n_q, heads)."""
+    torch = _torch()
+    n_q, heads, _ = qn.shape
+    kcf, kpf = kc.float(), kp.float()
+    step = max(1, min(n_q, CHUNK_ELEMS // max(1, heads * kc.shape[0])))
+    outs, lses = [], []
+    for lo in range(0, n_q, step):
+        hi = min(lo + step, n_q)
+        logits = (torch.einsum("qhd,kd->qhk", qn[lo:hi].float(), kcf)
+                  + torch.einsum("qhd,kd->qhk", qp[lo:hi].float(), kpf)) * scale
+        if keep is not None:
+            logits = logits.masked_fill(~keep[lo:hi, None, :], NEG_INF)
+        w, lse = _finish(logits)
+        outs.append(torch.einsum("qhk,kd->qhd", w, kcf))
+        lses.append(lse)
+    return torch.cat(outs), torch.cat(lses)
+
+
+def mla_paged_decode_inputs(dims, kv_lens, scale=None, dtype=None, device="cuda", seed=SEED):
+    """The operator's arguments in declaration order (``python/cleave/dynamic/reference.py:282-295``):
+    q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, sm_scale.
+    ``dims`` = (batch, qo_heads, ckv, kpe, num_pages, n_idx)."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    batch, heads, ckv, kpe, num_pages, n_idx = dims[:6]
+    gen = _generator(device, seed)
+    kv_indices = _pad_indices(_page_table(num_pages, sum(int(n) for n in kv_lens), device, seed), n_idx)
+
+    def randn(*shape):
+        return torch.randn(*shape, device=device, dtype=dtype, generator=gen)
+
+    return [randn(batch, heads, ckv), randn(batch, heads, kpe), randn(num_pages, 1, ckv), randn(num_pages, 1, kpe),
+            _i32(_indptr(kv_lens), device), kv_indices, float(ckv + kpe) ** -0.5 if scale is None else float(scale)]
+
+
+def mla_paged_decode_reference(dims, kv_lens, dtype=None):
+    """``python/cleave/dynamic/reference.py:297-321``: per request, the rows its table slice names
+    (page size 1) attended by its one query row per head; empty requests stay 0 / -inf."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    batch, heads, ckv = dims[:3]
+
+    def reference(q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, sm_scale):
+        out = torch.zeros(batch, heads, ckv, device=q_nope.device, dtype=dtype)
+        lse = torch.full((batch, heads), NEG_INF, device=q_nope.device, dtype=torch.float32)
+        starts = kv_indptr.tolist()
+        for b, kv_len in enumerate(kv_lens):
+            if kv_len <= 0:
+                continue
+            base = int(starts[b])
+            pages = kv_indices[base:base + int(kv_len)].long()
+            o, l = _mla_attend_rows(q_nope[b:b + 1], q_pe[b:b + 1], ckv_cache[pages, 0], kpe_cache[pages, 0], sm_scale)
+            out[b] = o[0].to(dtype)
+            lse[b] = l[0]
+        return [out, lse]
+
+    return reference

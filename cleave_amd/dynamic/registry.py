@@ -1,8 +1,8 @@
 """Shipped dynamic operators: the spec that names each one's inputs and the tiling it is
 built at (``python/cleave/dynamic/registry.py:37-231``).  Of the reference's nine operators
-the three paged GQA decode ones are built here (page size 1 with 8 and 4 kv heads, page size 64);
-the prefill and MLA ones are recognised by the frontend and refused by the access layer until
-their templates exist."""
+the four decode ones are built here (paged GQA: page size 1 with 8 and 4 kv heads, page size 64;
+paged MLA); the causal prefill ones are recognised by the frontend and refused by the access
+layer until their templates exist."""
 
 from __future__ import annotations
 
@@ -10,7 +10,7 @@ from dataclasses import dataclass, field
 
 from ..runtime.validate import Tolerance
 from . import workloads as _wl
-from .paging import PAGED_DECODE_SLAB, PagingSpec
+from .paging import PAGED_DECODE_SLAB, MLASpec, PagingSpec
 
 # Paged kernels reproduce their references far more tightly than the loose default bound;
 # equal_nan stays off: an empty request is defined as 0 / -inf, so a NaN is a defect.
@@ -30,10 +30,13 @@ class DynamicOperator:
 
     @property
     def is_mla(self) -> bool:
-        return False
+        return isinstance(self.spec, MLASpec)
 
     def matches(self, attention) -> bool:
         a = attention
+        if self.is_mla:
+            return (a.is_mla and a.kind == self.spec.kind and a.page_size == self.page_size
+                    and (a.num_qo_heads, a.head_dim, a.pe_dim) == tuple(self.dims[:3]))
         return (not a.is_mla and (a.num_qo_heads, a.num_kv_heads, a.head_dim) == tuple(self.dims[:3])
                 and a.page_size == self.page_size and a.kind == self.spec.kind)
 
@@ -52,10 +55,15 @@ class DynamicOperator:
     def kernel_source(self) -> str:
         """HIP source of this operator at its tuned tiling (single kernel)."""
         from ..codegen import HipCodeGen
-        from .paging import DenseAttention
-        from .paging.apply import _paged_outputs, _paged_params, _plan
+        from .paging import DenseAttention, DenseMLA
+        from .paging.apply import _mla_outputs, _mla_params, _mla_plan, _paged_outputs, _paged_params, _plan
 
         t = self.tuned_tiling
+        if self.is_mla:
+            dense = DenseMLA(self.dims[0], self.dims[1], self.dims[2], "bfloat16", "bfloat16")
+            params, ops = _mla_params(self.spec, dense)
+            outs, out_ops = _mla_outputs(self.spec, dense)
+            return HipCodeGen().gen(_mla_plan(self.spec, dense, "main", params + outs, {**ops, **out_ops}))
         dense = DenseAttention(t["query_rows"], t["kv_tile"], t["head_dim"], t["waves"] * 64, "bfloat16", "bfloat16",
                                waves=t["waves"])
         params, ops = _paged_params(self.spec, dense)
@@ -80,4 +88,9 @@ OPERATORS = {op.name: op for op in (
                    pass_configs={}),
         dict(query_rows=16, kv_tile=32, head_dim=128, waves=4), (32, 8, 128),
         _wl.WORKLOADS["gqa_paged_decode_h32_kv8_d128_ps64"], page_size=64),
+    # latent attention: one compressed cache (keys and values) + a rope cache, 16 heads, token table
+    DynamicOperator(
+        "mla_paged_decode_h16_ckv512_kpe64_ps1", MLASpec(num_qo_heads=16),
+        dict(query_rows=16, kv_tile=32, n_threads=64, ckv=512, kpe=64), (16, 512, 64),
+        _wl.WORKLOADS["mla_paged_decode_h16_ckv512_kpe64_ps1"], page_size=1, scale=_wl.MLA_SM_SCALE),
 )}

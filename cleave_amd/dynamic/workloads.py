@@ -17,7 +17,12 @@ WORKLOADS = {
     "gqa_paged_decode_h32_kv8_d128_ps1": ((1, 11, 10), (16, 1069, 1034), (16, 81390, 12942), (64, 68237, 58966)),
     "gqa_paged_decode_h32_kv4_d128_ps1": ((1, 8, 7), (16, 1070, 1020), (16, 32348, 23079), (64, 61535, 61519)),
     "gqa_paged_decode_h32_kv8_d128_ps64": ((4, 349, 212), (16, 1686, 1033), (32, 15178, 14103), (128, 52033, 47438)),
+    "mla_paged_decode_h16_ckv512_kpe64_ps1": ((1, 989669, 8), (16, 989669, 457), (64, 989669, 9945),
+                                              (64, 989669, 75145)),
 }
+
+# The softmax scale the reference's MLA operators are run at (``python/cleave/dynamic/workloads.py:12-13``).
+MLA_SM_SCALE = 0.1352337747812271
 
 # Geomean latency over exactly those axes on the reference's own back end, as recorded in its
 # checked-in baseline (``tests/perf/baselines/h100-80gb-hbm3.json``, NVIDIA H100 80GB HBM3, bf16):
@@ -26,6 +31,7 @@ REFERENCE_H100_US = {
     "gqa_paged_decode_h32_kv8_d128_ps1": (2.4898, 5.2114, 59.4166, 137.0866),
     "gqa_paged_decode_h32_kv4_d128_ps1": (2.4530, 5.0890, 80.3984, 131.4043),
     "gqa_paged_decode_h32_kv8_d128_ps64": (74.0303, 149.6087, 1667.6903, 4817.6807),
+    "mla_paged_decode_h16_ckv512_kpe64_ps1": (5.8886, 8.6802, 35.6304, 258.9872),
 }
 
 
@@ -58,6 +64,11 @@ def case(operator, axes, dims, page_size=1, scale=None, dtype=None, device="cuda
     from . import reference
 
     batch, pool, n_idx, kv_lens = decode_lengths(operator, axes, page_size)
+    if operator.startswith("mla_paged_decode"):
+        wl = (batch, *dims[:3], pool, n_idx)
+        inputs = reference.mla_paged_decode_inputs(wl, kv_lens, scale=scale, dtype=dtype, device=device)
+        expected = reference.mla_paged_decode_reference(wl, kv_lens, dtype=dtype)
+        return inputs, expected(*inputs)
     wl = (batch, *dims[:3], pool, n_idx)
     inputs = reference.gqa_paged_decode_inputs(wl, kv_lens, page_size=page_size, scale=scale, dtype=dtype, device=device)
     expected = reference.gqa_paged_decode_reference(wl, kv_lens, page_size=page_size, dtype=dtype)

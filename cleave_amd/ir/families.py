@@ -324,8 +324,13 @@ def _try_attention(view, out):
             (qpe, kpe), (q, kv) = terms
         if kv is not v:
             return None
+        if len(q.shape) == 2 and len(kv.shape) == 2:
+            # one request: q (H, D), kv (SKV, D) -- the dense body of a paged MLA operator
+            prob = {"batch": 1, "heads": q.shape[0], "ckv": q.shape[1], "kpe": qpe.shape[1],
+                    "skv": kv.shape[0], "scale": sc["scale"], "exact": sc["exact"], "shift": sc["shift"]}
+            return "mla", prob, {"Q": q, "QPE": qpe, "KV": kv, "KPE": kpe}
         if not (len(q.shape) == 3 and len(kv.shape) == 3 and q.shape[0] == kv.shape[0]):
-            raise LoweringRejected("MLA is built for q (B, H, D), kv (B, SKV, D)")
+            raise LoweringRejected("MLA is built for q ([B,] H, D), kv ([B,] SKV, D)")
         prob = {"batch": q.shape[0], "heads": q.shape[1], "ckv": q.shape[2], "kpe": qpe.shape[2],
                 "skv": kv.shape[1], "scale": sc["scale"], "exact": sc["exact"], "shift": sc["shift"]}
         return "mla", prob, {"Q": q, "QPE": qpe, "KV": kv, "KPE": kpe}

@@ -13,7 +13,15 @@ access layer.  TEST INFRASTRUCTURE: see the package docstring.
   * ``valid_len``        the slab layer's length formula (``paging/builders/slab.py:138-142``):
                          ``min(max(n_pages-1, 0)*P + max(last, 0), n_pages*P)``;
   * ``split_ranges``     ``tile0`` / ``my_trip`` (``paging/stages.py:331-347``): tiles dealt
-                         ``ceil(n_tiles / split)`` per split, a trailing split may get none.
+                         ``ceil(n_tiles / split)`` per split, a trailing split may get none;
+  * ``mla_attend`` / ``mla_decode``   ``_mla_attend_rows`` (``reference.py:108-126``) and
+                         ``mla_paged_decode_reference`` (``:297-321``): logits
+                         ``(q_nope c^T + q_pe r^T) * scale`` over the rows a request's table slice
+                         names (page size 1), softmax, values = the same latent rows ``c``.
+                         Pins (tests/test_oracle.py): equals ``attend`` on the concatenated
+                         operands (the sum of two products is one product over joined features),
+                         float64 brute force, page-permutation invariance, 0 / -inf for an empty
+                         request.
 """
 
 from __future__ import annotations
@@ -81,6 +89,37 @@ def decode(q, k_cache, v_cache, kv_indptr, kv_indices, kv_lens, page_size, sm_sc
         kk = np.repeat(gather(kc, indices, int(indptr[b]), n, page_size), group, axis=1)
         vv = np.repeat(gather(vc, indices, int(indptr[b]), n, page_size), group, axis=1)
         o, l = attend(qf[b], kk, vv, sm_scale)
+        out[b] = round_to_dtype(o, out_dtype)
+        lse[b] = l
+    return out, lse
+
+
+def mla_attend(qn: np.ndarray, qp: np.ndarray, kc: np.ndarray, kp: np.ndarray, scale: float):
+    """``qn`` (heads, ckv), ``qp`` (heads, kpe), ``kc`` (n_kv, ckv), ``kp`` (n_kv, kpe), all float32
+    -> (out (heads, ckv), lse2 (heads,))."""
+    logits = (np.einsum("hd,kd->hk", qn, kc, dtype=np.float32)
+              + np.einsum("hd,kd->hk", qp, kp, dtype=np.float32)) * np.float32(scale)
+    m = logits.max(axis=-1, keepdims=True)
+    e = np.exp(logits - m, dtype=np.float32)
+    s = e.sum(axis=-1, keepdims=True, dtype=np.float32)
+    lse2 = (m[:, 0] + np.log(s[:, 0], dtype=np.float32)) / np.float32(math.log(2.0))
+    return np.einsum("hk,kd->hd", e / s, kc, dtype=np.float32), lse2
+
+
+def mla_decode(q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, kv_lens, sm_scale, out_dtype="bfloat16"):
+    """-> ``(out (batch, heads, ckv) float32 on out_dtype's grid, lse (batch, heads) float32)``."""
+    qn, qp, cc, pc = to_f32(q_nope), to_f32(q_pe), to_f32(ckv_cache), to_f32(kpe_cache)
+    indptr = np.asarray(kv_indptr.cpu() if hasattr(kv_indptr, "cpu") else kv_indptr, dtype=np.int64)
+    indices = np.asarray(kv_indices.cpu() if hasattr(kv_indices, "cpu") else kv_indices, dtype=np.int64)
+    batch, heads, ckv = qn.shape
+    out = np.zeros((batch, heads, ckv), dtype=np.float32)
+    lse = np.full((batch, heads), -np.inf, dtype=np.float32)
+    for b, n in enumerate(kv_lens):
+        n = int(n)
+        if n <= 0:
+            continue
+        rows = indices[int(indptr[b]):int(indptr[b]) + n]
+        o, l = mla_attend(qn[b], qp[b], cc[rows, 0], pc[rows, 0], sm_scale)
         out[b] = round_to_dtype(o, out_dtype)
         lse[b] = l
     return out, lse

@@ -162,3 +162,22 @@ def paged_decode_op(hq=32, hkv=8, d=128, page=64, dtype=cl.f16, name=None):
         ann["kv_last_page_len"] = cl.Tensor[_batch, cl.i32] | None
     op.__annotations__ = ann
     return cleave_amd.jit(name=name, dtype=dtype)(op)
+
+
+def mla_paged_decode_op(heads=16, ckv=512, kpe=64, dtype=cl.bf16, name=None):
+    """The paged MLA decode operator as a ``@jit`` program (the reference's registry form,
+    ``demo/dynamic/mla_paged_decode.py``): one compressed cache that is both keys and values, a
+    rope cache adding a second score term, a token table (page size 1)."""
+    name = name or f"mla_paged_decode_h{heads}_ckv{ckv}_kpe{kpe}_ps1"
+
+    def op(qn, qp, ckv_cache, kpe_cache, kv_indptr, kvi, sm_scale):
+        pages = cl.PageTable(kv_indptr, kvi, length=_kv_len)
+        c, r = cl.paged_gather(ckv_cache, pages), cl.paged_gather(kpe_cache, pages)
+        p, lse = cl.softmax((qn @ c.mT + qp @ r.mT) * sm_scale, dim=-1, return_lse=True)
+        return p @ c, lse
+
+    op.__annotations__ = {"qn": cl.Tensor[_batch, heads, ckv], "qp": cl.Tensor[_batch, heads, kpe],
+                          "ckv_cache": cl.Tensor[_num_pages, 1, ckv], "kpe_cache": cl.Tensor[_num_pages, 1, kpe],
+                          "kv_indptr": cl.Tensor[_batch + 1, cl.i32], "kvi": cl.Tensor[_n_idx, cl.i32],
+                          "sm_scale": cl.Scalar[cl.f32]}
+    return cleave_amd.jit(name=name, dtype=dtype)(op)

@@ -125,6 +125,40 @@ def test_only_the_registered_paged_layers_are_built():
         build_split_decode(spec, DenseAttention(16, 32, 128, 256, "float16", "float16", waves=4), 8, CombineTiling(8))
 
 
+def test_paged_mla_layer_plans_and_signature():
+    """The paged MLA decode layer: the single kernel and the chunked split pair carry the
+    reference operator's argument order, the item count and item size are launch-time
+    expressions over the table length, and what is not built is refused by name."""
+    from cleave_amd.codegen import HipCodeGen, parse_manifest
+    from cleave_amd.dynamic import registry
+    from cleave_amd.dynamic.paging import (MLA_PAGED_PREFILL_CAUSAL, CombineTiling, DenseAttention, DenseMLA, MLASpec,
+                                           NotDenseAttention, UnsupportedTiling, build_split_decode)
+
+    op = registry.OPERATORS["mla_paged_decode_h16_ckv512_kpe64_ps1"]
+    assert op.is_mla and op.scale == pytest.approx(0.1352337747812271) and len(op.workloads) == 4
+    m = parse_manifest(op.kernel_source())
+    assert [p["name"] for p in m["params"]] == ["PlaceHolder_QN", "PlaceHolder_QP", "PlaceHolder_CKV", "PlaceHolder_KPE",
+                                               "PlaceHolder_KV_INDPTR", "PlaceHolder_KVI", "sm_scale", "OutputNode_0",
+                                               "OutputNode_1"]
+    by = {p["name"]: p for p in m["params"]}
+    assert by["PlaceHolder_CKV"]["shape"] == ["num_pages", 1, 512] and by["OutputNode_1"]["dtype"] == "float32"
+    assert m["launches"][0]["grid"] == ["batch", "1", "1"] and m["launches"][0]["block"][0] == 64
+    spec, dense = MLASpec(num_qo_heads=32), DenseMLA(32, 512, 64, "bfloat16", "bfloat16")
+    pair = parse_manifest(HipCodeGen().gen(build_split_decode(spec, dense, 8, CombineTiling(split=8))))
+    assert [l["entry"] for l in pair["launches"]] == ["main_kernel", "main_kernel_combine"]
+    assert pair["launches"][0]["grid"][:2] == ["ceildiv(n_idx, chunk_pages) + batch", "2"]
+    assert dict(pair["derived_dims"])["chunk_pages"].startswith("max(32, min(512, ceildiv(n_idx")
+    scratch = {p["name"]: p for p in pair["params"] if p["role"] == "scratch"}
+    assert scratch["Partial_PO_split"]["shape"] == ["ceildiv(n_idx, chunk_pages) + batch", 32, 512]
+    with pytest.raises(UnsupportedTiling, match="not built"):
+        build_split_decode(MLASpec(16, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True), DenseMLA(16, 512, 64, "bfloat16", "bfloat16"),
+                           8, CombineTiling(split=8))
+    with pytest.raises(NotDenseAttention, match="same operator family"):
+        build_split_decode(MLASpec(16), DenseAttention(16, 32, 128, 256, "bfloat16", "bfloat16"), 8, CombineTiling(split=8))
+    with pytest.raises(UnsupportedTiling, match="heads"):
+        build_split_decode(MLASpec(32), DenseMLA(16, 512, 64, "bfloat16", "bfloat16"), 8, CombineTiling(split=8))
+
+
 def test_presets_and_configs():
     from cleave_amd.pipeline.config import (EvalConfig, ScheduleConfig, SuperoptConfig, auto_max_ops, get_preset,
                                             list_presets)

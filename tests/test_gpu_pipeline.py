@@ -150,3 +150,27 @@ def test_registry_row_gather_operators(cache_root, name):
     _close(out, want_o)
     live = np.isfinite(want_l)
     np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
+
+
+def test_registry_mla_decode_operator(cache_root):
+    """The shipped paged MLA decode operator through ``compile``: the dense one-request body is
+    tiled, paged (single kernel and chunked split pair), validated over the captured workload
+    axes against the torch reference and timed; then one call against the numpy oracle."""
+    from cleave_amd.dynamic import OPERATORS
+    from cleave_amd.dynamic import reference as dref
+
+    name = "mla_paged_decode_h16_ckv512_kpe64_ps1"
+    op = OPERATORS[name]
+    kernel = cleave_amd.compile(C.mla_paged_decode_op(name=name), schedule=P.ScheduleConfig(topk=1),
+                                split=cl.Split("kv_len", (4,)), max_workloads=2)
+    rep = kernel.report
+    assert rep.best() is not None and len(rep.correct) >= 2 and rep.n_workloads == len(op.workloads)
+    assert rep.dispatch is not None and {"split", "single"} <= set(rep.dispatch["geomean_us"])
+    lens = [37, 0, 700, 1]
+    args = dref.mla_paged_decode_inputs((len(lens), 16, 512, 64, 1000, sum(lens)), lens, scale=op.scale, device="cuda")
+    out, lse = kernel(*args)
+    want_o, want_l = paged_oracle.mla_decode(*[a.cpu() for a in args[:6]], lens, args[6])
+    _close(out, want_o)
+    live = np.isfinite(want_l)
+    np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
+    assert np.all(np.isneginf(lse.cpu().numpy()[~live]))

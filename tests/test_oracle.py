@@ -164,3 +164,62 @@ def test_program_reference_and_oracle_agree_on_the_graded_programs():
         ins = mk(C.SMALL[name])
         want = prog.reference(*ins)[0].float().numpy()
         np.testing.assert_allclose(po.evaluate(prog, ins)[0], want, rtol=4e-3, atol=4e-3)
+
+
+# ----------------------------------------------------------------------------- paged MLA decode
+def _mla_case(lens, num_pages=300, heads=16, ckv=64, kpe=16, seed=5):
+    rng = np.random.default_rng(seed)
+    total = sum(lens)
+    qn = rng.standard_normal((len(lens), heads, ckv)).astype(np.float32)
+    qp = rng.standard_normal((len(lens), heads, kpe)).astype(np.float32)
+    cc = rng.standard_normal((num_pages, 1, ckv)).astype(np.float32)
+    pc = rng.standard_normal((num_pages, 1, kpe)).astype(np.float32)
+    idx = rng.permutation(num_pages)[:total].astype(np.int32)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    return qn, qp, cc, pc, ptr, idx
+
+
+def test_mla_attend_is_attend_over_joined_features():
+    """(q_nope c^T + q_pe r^T) is one product over the concatenated features, and the values are
+    the latent part of the keys: MLA must equal the GQA oracle on the joined operands (a dropped
+    term, a swapped operand or values taken from the rope part all break this)."""
+    qn, qp, cc, pc, _, idx = _mla_case([23])
+    rows = idx[:23]
+    out, lse = paged_oracle.mla_attend(qn[0], qp[0], cc[rows, 0], pc[rows, 0], 0.17)
+    q_joined = np.concatenate([qn[0], qp[0]], axis=-1)
+    k_joined = np.concatenate([cc[rows, 0], pc[rows, 0]], axis=-1)[:, None, :].repeat(16, axis=1)
+    v_latent = cc[rows, 0][:, None, :].repeat(16, axis=1)
+    want_o, want_l = paged_oracle.attend(q_joined, k_joined, v_latent, 0.17)
+    np.testing.assert_allclose(out, want_o, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(lse, want_l, rtol=1e-5, atol=1e-6)
+
+
+def test_mla_decode_against_float64_brute_force_and_empty_requests():
+    lens = [7, 0, 40, 1]
+    qn, qp, cc, pc, ptr, idx = _mla_case(lens)
+    out, lse = paged_oracle.mla_decode(qn, qp, cc, pc, ptr, idx, lens, 0.3, out_dtype="float32")
+    for b, n in enumerate(lens):
+        if n == 0:
+            assert np.all(out[b] == 0) and np.all(np.isneginf(lse[b]))
+            continue
+        rows = idx[ptr[b]:ptr[b] + n]
+        for h in range(16):
+            logits = np.array([(np.dot(qn[b, h].astype(np.float64), cc[r, 0]) + np.dot(qp[b, h].astype(np.float64), pc[r, 0]))
+                               * 0.3 for r in rows])
+            w = np.exp(logits - logits.max())
+            w /= w.sum()
+            want = sum(wi * cc[r, 0].astype(np.float64) for wi, r in zip(w, rows))
+            np.testing.assert_allclose(out[b, h], want, rtol=2e-5, atol=2e-6)
+            assert lse[b, h] == pytest.approx(np.log2(np.exp(logits - logits.max()).sum()) + logits.max() / np.log(2), rel=1e-5)
+
+
+def test_mla_decode_depends_on_the_table_only_through_the_rows_it_names():
+    """Moving the named rows elsewhere in the pool and renaming them in the table changes nothing."""
+    lens = [9, 30]
+    qn, qp, cc, pc, ptr, idx = _mla_case(lens)
+    out, lse = paged_oracle.mla_decode(qn, qp, cc, pc, ptr, idx, lens, 0.2)
+    perm = np.random.default_rng(1).permutation(cc.shape[0])
+    cc2, pc2 = np.empty_like(cc), np.empty_like(pc)
+    cc2[perm], pc2[perm] = cc, pc
+    out2, lse2 = paged_oracle.mla_decode(qn, qp, cc2, pc2, ptr, perm[idx].astype(np.int32), lens, 0.2)
+    assert np.array_equal(out, out2) and np.array_equal(lse, lse2)
