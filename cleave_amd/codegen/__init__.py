@@ -389,6 +389,28 @@ class HipCodeGen:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv({grid_rows} * {p['vdim'] // 4}, 256)", 1, 1), 256, 0, args)
 
+    def _emit_attn_prefill(self, unit, plan, params, partial, combine, fused):
+        """Causal prefill over ragged queries (token-table or packed keys): one item per 16-row tile
+        (tokens x head group of one kv head), one wave per kv head."""
+        p, op = plan.problem, plan.operands
+        if combine or (plan.split_factor or 1) > 1:
+            raise CodegenError("prefill has no split-KV form")
+        emit_lse = bool(p.get("emit_lse"))
+        self._attn_common(unit, plan, params, partial, combine, fused, p["vdim"], f"(total_q * {p['q_heads']})", emit_lse)
+        d, group = p["head_dim"], p["group"]
+        if d % 32 or not (d % 128 == 0 or d == 64) or 16 % group or p["kv_heads"] > 16:
+            raise CodegenError("prefill needs head_dim 64 or k*128, a head group dividing 16 and at most 16 kv heads")
+        for k, v in (("CL_HEAD_DIM", d), ("CL_KV_HEADS", p["kv_heads"]), ("CL_Q_HEADS", p["q_heads"]),
+                     ("CL_RAGGED", bool(p["ragged"]))):
+            unit.define(k, v)
+        for role, macro in (("Q", "CL_ARG_Q"), ("K", "CL_ARG_K"), ("V", "CL_ARG_V"), ("QINDPTR", "CL_ARG_QINDPTR"),
+                            ("INDPTR", "CL_ARG_INDPTR"), ("INDICES", "CL_ARG_INDICES")):
+            if role in op:
+                unit.define(macro, op[role])
+        unit.templates.append("attn_prefill.hip")
+        items = f"ceildiv({p['dim_names']['total_q']}, {16 // group}) + batch"
+        unit.launch(ENTRY, (items, 1, 1), p["kv_heads"] * 64, p["kv_heads"] * 16 * d * 4, self._partial_args)
+
     def _emit_mla_decode(self, unit, plan, params, partial, combine, fused):
         p, t, op = plan.problem, plan.tiling, plan.operands
         if p.get("paged"):

@@ -18,7 +18,8 @@ from dataclasses import dataclass
 
 from ...schedule.plan import KernelPlan, ParamSpec
 from .errors import NotDenseAttention, UnsupportedTiling
-from .kinds import BUILT_KINDS, MLA_PAGED_DECODE, PAGED_DECODE, PAGED_DECODE_SLAB
+from .kinds import (BUILT_KINDS, CAUSAL_KINDS, MLA_PAGED_DECODE, PAGED_DECODE, PAGED_DECODE_SLAB,
+                    RAGGED_PREFILL_CAUSAL)
 from .specs import CombineTiling, MLASpec, PagingSpec
 
 KV_STEP = 32  # tokens one wave consumes per step of the decode template
@@ -128,6 +129,10 @@ def _check_tiling(spec, dense, split: bool = False) -> None:
                                 f"(built: {', '.join(BUILT_KINDS)})")
     if split and spec.kind not in (PAGED_DECODE, PAGED_DECODE_SLAB, MLA_PAGED_DECODE):
         raise UnsupportedTiling(f"split-KV is a decode transformation; got the {spec.kind!r} layer")
+    if spec.kind in CAUSAL_KINDS:
+        if 16 % spec.group or spec.num_kv_heads > 16:
+            raise UnsupportedTiling(f"the prefill tile is 16 rows = tokens x head group: the group ({spec.group}) must "
+                                    "divide 16, with at most 16 kv heads (one wave each)")
     if isinstance(spec, MLASpec):
         if dense.heads != spec.num_qo_heads:
             raise UnsupportedTiling(f"the dense body has {dense.heads} heads, the spec {spec.num_qo_heads}")
@@ -203,6 +208,47 @@ def chunk_pages_expr(spec, chunk_pages: int) -> str:
     cus = current_target().arch.compute_units
     return (f"max(1, min({MAX_CHUNK_PAGES}, ceildiv({spec.index_dim}, "
             f"max(1, {cus} - {spec.batch_dim}))))")
+
+
+# ----------------------------------------------------------------------------- causal prefill
+# Parameter order of the reference's operators (``python/cleave/dynamic/reference.py:204-278``):
+# q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, sm_scale (token table) or
+# q, k, v, qo_indptr, kv_indptr, sm_scale (packed keys); then out (total_q, heads, d), lse.
+def _prefill_plan(spec: PagingSpec, dense: DenseAttention) -> KernelPlan:
+    d, dt = dense.head_dim, dense.dtype
+    ragged = spec.kind == RAGGED_PREFILL_CAUSAL
+    tq = spec.tokens_dim
+    ph = lambda n: f"PlaceHolder_{n}"  # noqa: E731
+    kv_shape = (spec.kv_tokens_dim, spec.num_kv_heads, d) if ragged else (spec.pages_dim, 1, spec.num_kv_heads, d)
+    params = [
+        ParamSpec(ph(spec.query_input), dt, (tq, spec.num_qo_heads, d), "input"),
+        ParamSpec(ph(spec.cache_inputs[0]), dt, kv_shape, "input"),
+        ParamSpec(ph(spec.cache_inputs[1]), dt, kv_shape, "input"),
+        ParamSpec(ph(spec.query_indptr_input), "int32", (spec.indptr_dim,), "input"),
+        ParamSpec(ph(spec.indptr_input), "int32", (spec.indptr_dim,), "input"),
+    ]
+    operands = {"Q": params[0].name, "K": params[1].name, "V": params[2].name, "QINDPTR": params[3].name,
+                "INDPTR": params[4].name}
+    if not ragged:
+        params.append(ParamSpec(ph(spec.index_input), "int32", (spec.index_dim,), "input"))
+        operands["INDICES"] = params[-1].name
+    params.append(ParamSpec(spec.scale_input, "float32", (), "scalar"))
+    outs = [ParamSpec("OutputNode_0", dense.out_dtype, (tq, spec.num_qo_heads, d), "output")]
+    operands["OUT"] = "OutputNode_0"
+    if spec.emit_lse:
+        outs.append(ParamSpec("OutputNode_1", "float32", (tq, spec.num_qo_heads), "output"))
+        operands["OUT1"] = "OutputNode_1"
+    # kernel-side names of the run-time extents: the key count is the table length or the packed
+    # key rows; the request count follows from the row pointers
+    dim_names = {"total_q": tq, "n_idx": spec.kv_tokens_dim} if ragged else \
+        {"total_q": tq, "num_pages": spec.pages_dim, "n_idx": spec.index_dim}
+    problem = {"paged": True, "prefill": True, "ragged": ragged, "kv_heads": spec.num_kv_heads,
+               "q_heads": spec.num_qo_heads, "group": spec.group, "head_dim": d, "vdim": d,
+               "emit_lse": bool(spec.emit_lse), "units": None, "skv": 0, "sq": 0, "scale": 1.0, "dim_names": dim_names}
+    return KernelPlan(template="attn_prefill", role="main", family="attention", dtype=dense.dtype,
+                      extra={"derived_dims": [("batch", f"{spec.indptr_dim} - 1")]}, problem=problem, tiling={},
+                      params=params + outs, operands=operands, split_factor=None, dyn_dims=tuple(dim_names.values()),
+                      n_threads=spec.num_kv_heads * 64, label=f"kv={KV_STEP} q=16 thr={spec.num_kv_heads * 64}")
 
 
 # ----------------------------------------------------------------------------- paged MLA decode
@@ -289,6 +335,8 @@ def apply_paging(plan: KernelPlan, spec) -> KernelPlan:
         return _mla_plan(spec, dense, "main", params + outs, {**operands, **out_ops})
     dense = read_dense_attention(plan)
     _check_tiling(spec, dense)
+    if spec.kind in CAUSAL_KINDS:
+        return _prefill_plan(spec, dense)
     params, operands = _paged_params(spec, dense)
     outs, out_ops = _paged_outputs(spec, dense)
     return _plan(spec, dense, "main", params + outs, {**operands, **out_ops})

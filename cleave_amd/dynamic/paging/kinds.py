@@ -16,7 +16,7 @@ MLA_KINDS = (MLA_PAGED_DECODE, MLA_PAGED_PREFILL_CAUSAL)
 SPLIT_KINDS = (PAGED_DECODE, PAGED_DECODE_SLAB, MLA_PAGED_DECODE)
 
 # Layers this back end has a HIP template for; the others are recognised and refused.
-BUILT_KINDS = (PAGED_DECODE, PAGED_DECODE_SLAB, MLA_PAGED_DECODE)
+BUILT_KINDS = (PAGED_DECODE, PAGED_DECODE_SLAB, PAGED_PREFILL_CAUSAL, RAGGED_PREFILL_CAUSAL, MLA_PAGED_DECODE)
 
 OPTIONAL_FIELDS = ("batch_dim", "tokens_dim", "kv_tokens_dim", "pages_dim", "index_dim", "index_input",
                    "last_page_len_input", "query_indptr_input", "grid_order")

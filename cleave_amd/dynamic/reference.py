@@ -208,3 +208,98 @@ def mla_paged_decode_reference(dims, kv_lens, dtype=None):
         return [out, lse]
 
     return reference
+
+
+# ----------------------------------------------------------------------------- causal prefill
+def causal_keep(q_len, kv_len, device):
+    """End-aligned causal mask (``python/cleave/dynamic/reference.py:129-133``): keep
+    ``kv_pos <= kv_len - q_len + q_pos``; (q_len, kv_len) bool."""
+    torch = _torch()
+    q_pos = torch.arange(q_len, device=device)[:, None]
+    kv_pos = torch.arange(kv_len, device=device)[None, :]
+    return kv_pos <= (kv_len - q_len) + q_pos
+
+
+def gqa_paged_prefill_inputs(dims, q_lens, kv_lens, scale=None, dtype=None, device="cuda", seed=SEED):
+    """q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, sm_scale
+    (``python/cleave/dynamic/reference.py:204-219``); ``dims`` = (qo_heads, kv_heads, head_dim,
+    num_pages, n_idx, total_q)."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    hq, hkv, d, num_pages, n_idx, total_q = dims[:6]
+    gen = _generator(device, seed)
+    kv_indptr = _indptr(kv_lens)
+    kv_indices = _pad_indices(_page_table(num_pages, kv_indptr[-1], device, seed), n_idx)
+
+    def randn(*shape):
+        return torch.randn(*shape, device=device, dtype=dtype, generator=gen)
+
+    return [randn(total_q, hq, d), randn(num_pages, 1, hkv, d), randn(num_pages, 1, hkv, d),
+            _i32(_indptr(q_lens), device), _i32(kv_indptr, device), kv_indices,
+            float(d) ** -0.5 if scale is None else float(scale)]
+
+
+def gqa_ragged_prefill_inputs(dims, q_lens, kv_lens, scale=None, dtype=None, device="cuda", seed=SEED):
+    """q, k, v, qo_indptr, kv_indptr, sm_scale (``python/cleave/dynamic/reference.py:245-255``);
+    ``dims`` = (qo_heads, kv_heads, head_dim, total_q, total_kv)."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    hq, hkv, d, total_q, total_kv = dims[:5]
+    gen = _generator(device, seed)
+
+    def randn(*shape):
+        return torch.randn(*shape, device=device, dtype=dtype, generator=gen)
+
+    return [randn(total_q, hq, d), randn(total_kv, hkv, d), randn(total_kv, hkv, d), _i32(_indptr(q_lens), device),
+            _i32(_indptr(kv_lens), device), float(d) ** -0.5 if scale is None else float(scale)]
+
+
+def _prefill_reference(hq, hkv, d, total_q, q_lens, kv_lens, dtype, rows_of):
+    """Shared body of the two prefill references (``reference.py:221-242,258-278``): per request
+    with both lengths positive, its query rows attend its keys under the end-aligned causal mask;
+    everything else stays 0 / -inf.  ``rows_of(r, kv_len, tensors)`` -> (K rows, V rows)."""
+    torch = _torch()
+    group = hq // hkv
+
+    def reference(q, *rest):
+        sm_scale = rest[-1]
+        qo_indptr = rest[2].tolist()
+        out = torch.zeros(total_q, hq, d, device=q.device, dtype=dtype)
+        lse = torch.full((total_q, hq), NEG_INF, device=q.device, dtype=torch.float32)
+        for r, (q_len, kv_len) in enumerate(zip(q_lens, kv_lens)):
+            if q_len <= 0 or kv_len <= 0:
+                continue
+            qs, qe = int(qo_indptr[r]), int(qo_indptr[r + 1])
+            kk, vv = rows_of(r, int(kv_len), rest)
+            o, l = _attend(q[qs:qe], kk.repeat_interleave(group, dim=1), vv.repeat_interleave(group, dim=1), sm_scale,
+                           causal_keep(int(q_len), int(kv_len), q.device))
+            out[qs:qe] = o.to(dtype)
+            lse[qs:qe] = l
+        return [out, lse]
+
+    return reference
+
+
+def gqa_paged_prefill_reference(dims, q_lens, kv_lens, dtype=None):
+    torch = _torch()
+    hq, hkv, d, _pages, _n_idx, total_q = dims[:6]
+
+    def rows_of(r, kv_len, rest):
+        k_cache, v_cache, _qo, kv_indptr, kv_indices = rest[:5]
+        base = int(kv_indptr[r])
+        pages = kv_indices[base:base + kv_len].long()
+        return k_cache[pages, 0], v_cache[pages, 0]
+
+    return _prefill_reference(hq, hkv, d, total_q, q_lens, kv_lens, dtype or torch.bfloat16, rows_of)
+
+
+def gqa_ragged_prefill_reference(dims, q_lens, kv_lens, dtype=None):
+    torch = _torch()
+    hq, hkv, d, total_q, _total_kv = dims[:5]
+
+    def rows_of(r, kv_len, rest):
+        k, v, _qo, kv_indptr = rest[:4]
+        ks = int(kv_indptr[r])
+        return k[ks:ks + kv_len], v[ks:ks + kv_len]
+
+    return _prefill_reference(hq, hkv, d, total_q, q_lens, kv_lens, dtype or torch.bfloat16, rows_of)

@@ -21,7 +21,16 @@ access layer.  TEST INFRASTRUCTURE: see the package docstring.
                          Pins (tests/test_oracle.py): equals ``attend`` on the concatenated
                          operands (the sum of two products is one product over joined features),
                          float64 brute force, page-permutation invariance, 0 / -inf for an empty
-                         request.
+                         request;
+  * ``causal_keep`` / ``prefill``   ``_causal_keep`` (``reference.py:129-133``: keep
+                         ``kv_pos <= kv_len - q_len + q_pos``) and the two causal prefill
+                         references (``:221-242`` token table, ``:258-278`` packed keys): ragged
+                         query rows per request, fully masked rows 0 / -inf.  Pins
+                         (tests/test_oracle.py): a request with one query row equals ``decode``
+                         of the same keys; row i equals ``attend`` over the first
+                         ``kv_len - q_len + i + 1`` keys (the mask as a prefix length); rows with
+                         ``kv_len - q_len + i < 0`` are 0 / -inf; token-table and packed forms
+                         agree on the same rows.
 """
 
 from __future__ import annotations
@@ -122,4 +131,54 @@ def mla_decode(q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, kv_len
         o, l = mla_attend(qn[b], qp[b], cc[rows, 0], pc[rows, 0], sm_scale)
         out[b] = round_to_dtype(o, out_dtype)
         lse[b] = l
+    return out, lse
+
+
+def causal_keep(q_len: int, kv_len: int) -> np.ndarray:
+    q_pos = np.arange(q_len)[:, None]
+    kv_pos = np.arange(kv_len)[None, :]
+    return kv_pos <= (kv_len - q_len) + q_pos
+
+
+def _attend_masked(q, k, v, scale, keep):
+    """``q`` (n_q, heads, d), ``k``/``v`` (n_kv, heads, d) float32, ``keep`` (n_q, n_kv) bool ->
+    out (n_q, heads, d), lse2 (n_q, heads); a row with nothing kept gives 0 and -inf."""
+    logits = np.einsum("qhd,khd->qhk", q, k, dtype=np.float32) * np.float32(scale)
+    logits = np.where(keep[:, None, :], logits, -np.inf).astype(np.float32)
+    m = logits.max(axis=-1, keepdims=True)
+    dead = np.isneginf(m)
+    e = np.exp(logits - np.where(dead, 0.0, m), dtype=np.float32)
+    s = e.sum(axis=-1, keepdims=True, dtype=np.float32)
+    w = np.where(dead, 0.0, e / np.where(dead, 1.0, s)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        lse2 = np.where(dead[..., 0], -np.inf, (m[..., 0] + np.log(s[..., 0], dtype=np.float32)) / np.float32(math.log(2.0)))
+    return np.einsum("qhk,khd->qhd", w, v, dtype=np.float32), lse2.astype(np.float32)
+
+
+def prefill(q, k, v, qo_indptr, kv_indptr, kv_indices, q_lens, kv_lens, sm_scale, out_dtype="bfloat16"):
+    """Causal prefill of ragged queries.  ``kv_indices`` is the token table (then ``k``/``v`` are
+    caches (num_pages, 1, kv_heads, d)) or None (packed keys (total_kv, kv_heads, d))."""
+    qf, kf, vf = to_f32(q), to_f32(k), to_f32(v)
+    as_i64 = lambda a: np.asarray(a.cpu() if hasattr(a, "cpu") else a, dtype=np.int64)  # noqa: E731
+    qo, kvp = as_i64(qo_indptr), as_i64(kv_indptr)
+    idx = None if kv_indices is None else as_i64(kv_indices)
+    total_q, hq, d = qf.shape
+    hkv = kf.shape[-2]
+    group = hq // hkv
+    out = np.zeros((total_q, hq, d), dtype=np.float32)
+    lse = np.full((total_q, hq), -np.inf, dtype=np.float32)
+    for r, (ql, kl) in enumerate(zip(q_lens, kv_lens)):
+        ql, kl = int(ql), int(kl)
+        if ql <= 0 or kl <= 0:
+            continue
+        qs = int(qo[r])
+        if idx is None:
+            kk, vv = kf[int(kvp[r]):int(kvp[r]) + kl], vf[int(kvp[r]):int(kvp[r]) + kl]
+        else:
+            rows = idx[int(kvp[r]):int(kvp[r]) + kl]
+            kk, vv = kf[rows, 0], vf[rows, 0]
+        o, l = _attend_masked(qf[qs:qs + ql], np.repeat(kk, group, axis=1), np.repeat(vv, group, axis=1), sm_scale,
+                              causal_keep(ql, kl))
+        out[qs:qs + ql] = round_to_dtype(o, out_dtype)
+        lse[qs:qs + ql] = l
     return out, lse
