@@ -281,7 +281,7 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
 
 # ----------------------------------------------------------------------------- shipped paged operators
 def run_dynamic(names=None):
-    """The registry's paged decode operators (GQA and MLA, bf16) over their captured workload axes:
+    """The registry's operators (paged GQA / MLA decode, causal prefill; bf16) over their captured workload axes:
     ``compile`` searches tilings and split-KV pairs, validates every candidate on every workload
     against the torch reference and times the valid ones; with a split pair and a single kernel
     it calibrates which to run per workload.  Reported: the best geomean, per-workload times of
@@ -302,7 +302,10 @@ def run_dynamic(names=None):
         if names and name not in names:
             continue
         if op.is_mla:
-            fn = C.mla_paged_decode_op(*op.dims[:3], dtype=cl.bf16, name=name)
+            make = C.mla_paged_prefill_op if "prefill" in name else C.mla_paged_decode_op
+            fn = make(*op.dims[:3], dtype=cl.bf16, name=name)
+        elif "prefill" in name:
+            fn = C.prefill_op(*op.dims[:3], ragged="ragged" in name, dtype=cl.bf16, name=name)
         else:
             hq, hkv, d = op.dims[:3]
             fn = C.paged_decode_op(hq, hkv, d, op.page_size, dtype=cl.bf16, name=name)
@@ -313,7 +316,8 @@ def run_dynamic(names=None):
         rep = kernel.report
         best = rep.best()
         keys = sorted(best.latency_us, key=lambda k: [int(x) for x in k.split("_")[1:]])
-        ref = dict(zip((f"wl_{a}_{b}_{c}" for a, b, c in op.workloads), wl.REFERENCE_H100_US.get(name, ())))
+        ref = dict(zip(("wl_" + "_".join(str(a) for a in axes) for axes in op.workloads),
+                       wl.REFERENCE_H100_US.get(name, ())))
         row = {"op": name, "dtype": "bf16", "workloads": len(keys), "candidates": len(rep.candidates),
                "validated": len(rep.correct), "best": best.label, "geomean_us": round(best.geomean_us, 2),
                "per_workload_us": {k: round(best.latency_us[k], 2) for k in keys},
@@ -397,7 +401,7 @@ def main():
             results[name] = run_copy(max(10, args.steps // 4), max(2, args.warmup // 4))
             continue
         if name == "dyn":
-            results[name] = {"op": "dyn", "workload": "registry paged decode operators (GQA, MLA) over their captured axes",
+            results[name] = {"op": "dyn", "workload": "registry operators (paged GQA / MLA decode, causal prefill) over their captured axes",
                              "operators": run_dynamic([n for n in args.dyn_ops.split(",") if n] or None)}
             continue
         if name == "c5":

@@ -462,17 +462,23 @@ class HipCodeGen:
         items are requests (single kernel) or table slices of at most ``chunk_pages`` entries
         (split form, folded by the chunked combine)."""
         p, t, op = plan.problem, plan.tiling, plan.operands
-        batch_name = p["dim_names"]["batch"]
+        prefill = bool(p.get("prefill"))
+        batch_name = "batch" if prefill else p["dim_names"]["batch"]
         emit_lse = bool(p.get("emit_lse"))
-        self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], f"(batch * {p['heads']})", emit_lse)
+        rows = f"(total_q * {p['heads']})" if prefill else f"(batch * {p['heads']})"
+        self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], rows, emit_lse)
+        if prefill and (plan.split_factor or 1) > 1:
+            raise CodegenError("prefill has no split-KV form")
         if p["heads"] % 16 or p["ckv"] % 64 or p["kpe"] % 64:
             raise CodegenError("paged MLA decode needs heads % 16 == 0 and latent / rope widths that are multiples of 64")
         chunked = (plan.split_factor or 1) > 1
         if chunked and not t.get("CHUNK_PAGES"):
             raise CodegenError("the split form of paged MLA decode is the chunked one (CHUNK_PAGES)")
         for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_CHUNKED", chunked),
-                     ("CL_CHUNK_PAGES", chunked), ("CL_Q_HEADS", p["heads"])):
+                     ("CL_CHUNK_PAGES", chunked), ("CL_Q_HEADS", p["heads"]), ("CL_PREFILL", prefill)):
             unit.define(k, v)
+        if prefill:
+            unit.define("CL_ARG_QINDPTR", op["QINDPTR"])
         if "LDS_AHEAD" in t:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
         for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE"),
@@ -481,6 +487,8 @@ class HipCodeGen:
         unit.templates += ["mla_paged_decode.hip", "attn_combine.hip"]
         if partial:
             items = f"ceildiv({p['dim_names']['n_idx']}, chunk_pages) + {batch_name}" if chunked else batch_name
+            if prefill:
+                items = p["dim_names"]["total_q"]
             unit.launch(ENTRY, (items, p["heads"] // 16, 1), 64, 0, self._partial_args)
         if combine:
             entry, args = self._combine_args

@@ -70,6 +70,22 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   int ext = off + (hi - 1 - q0) + 1;                    // keys the item's last row may see
   ext = ext < kv_len ? ext : kv_len;
   ext = ext > 0 ? ext : 0;
+  if (ext == 0) {
+    // no row of the item sees a key (a key window shorter than the query run leaves whole tiles
+    // like this): zeros and -inf, nothing to read
+    for (int idx = lane; idx < n_rows * (CL_HEAD_DIM / 4); idx += 64) {
+      const int row = idx / (CL_HEAD_DIM / 4), d = (idx % (CL_HEAD_DIM / 4)) * 4;
+      const i64 orow = (i64)(lo + row / PF_GROUP) * CL_Q_HEADS + head * PF_GROUP + row % PF_GROUP;
+      elem4 y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = to_elem(0.f);
+      *reinterpret_cast<elem4*>(CL_ARG_OUT + orow * CL_HEAD_DIM + d) = y;
+    }
+#if CL_EMIT_LSE
+    if (g == 0 && live) CL_ARG_LSE[(i64)tok * CL_Q_HEADS + qhead] = CL_NEG_INF;
+#endif
+    return;
+  }
   const float scale2 = sm_scale * 1.4426950408889634f;
   const i64 row_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
   const elem_t* kbase = CL_ARG_K + (i64)head * CL_HEAD_DIM;

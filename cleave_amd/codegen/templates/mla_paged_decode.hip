@@ -14,10 +14,16 @@
 // read.  Scores, softmax and value product are the dense kernel's (16 heads per wave, Q fragments
 // resident, fixed softmax reference raised outside the hot loop).
 //
-//   CL_HEADS (multiple of 16)  CL_CKV  CL_KPE (multiples of 64)  CL_CHUNKED
+// CL_PREFILL: causal prefill over ragged query rows -- an item is one query token (rows = its 16
+// heads) and the keys its causal limit admits; out and lse are per query token.
+//
+//   CL_HEADS (multiple of 16)  CL_CKV  CL_KPE (multiples of 64)  CL_CHUNKED  CL_PREFILL
 //   run-time: batch, num_pages, n_idx [, chunk_pages]; scalar sm_scale (> 0 or not: the
 //   maximum is taken over scaled scores)
 
+#ifndef CL_PREFILL
+#define CL_PREFILL 0
+#endif
 #define MP_STEP 32
 #define MP_D (CL_CKV + CL_KPE)
 #define MP_PANEL (MP_STEP * 64)
@@ -85,6 +91,29 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lo = p0 > chunk * chunk_pages ? p0 : chunk * chunk_pages;
   const int hi = p1 < (chunk + 1) * chunk_pages ? p1 : (chunk + 1) * chunk_pages;
   if (hi <= lo) return;                               // an index no (chunk, request) pair maps to
+#elif CL_PREFILL
+  // causal prefill: an item is one query token (its 16 heads are the tile); it sees the keys
+  // kv_pos <= kv_len - q_len + q_pos of its request
+  const int qtok = blockIdx.x;
+  int req = 0;
+  {
+    int hi_b = batch - 1;                               // the last b with qo_indptr[b] <= qtok
+    while (req < hi_b) {
+      const int mid = (req + hi_b + 1) >> 1;
+      if (mp_clamp(CL_ARG_QINDPTR[mid], 0, total_q) <= qtok) req = mid;
+      else hi_b = mid - 1;
+    }
+  }
+  const int q0 = mp_clamp(CL_ARG_QINDPTR[req], 0, total_q), q1 = mp_clamp(CL_ARG_QINDPTR[req + 1], 0, total_q);
+  const int lo = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx);
+  int hi;
+  {
+    int kv_len = mp_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx) - lo;
+    kv_len = kv_len > 0 ? kv_len : 0;
+    int ext = kv_len - (q1 - q0) + (qtok - q0) + 1;
+    ext = qtok < q1 ? ext : 0;                          // (a token past its request's rows: nothing)
+    hi = lo + mp_clamp(ext, 0, kv_len);
+  }
 #else
   const int req = blockIdx.x;
   const int lo = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx);
@@ -94,11 +123,17 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int n_tok = hi - lo;
   const int n_steps = (n_tok + MP_STEP - 1) / MP_STEP;
   const float scale_log2e = sm_scale * 1.4426950408889634f;
+#if CL_PREFILL
+  const i64 qrow = (i64)qtok * CL_HEADS + head0 + c;
+#else
   const i64 qrow = (i64)req * CL_HEADS + head0 + c;
+#endif
   const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)mp_tiles;
 
   float m_run = CL_NEG_BIG;            // softmax reference point of head c (log2 domain), uniform over g
-  f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};  // every component: sum of the weights of head c
+  f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};  // every component: sum of the (element-typed) weights of head c: normalises out
+  float l_exact = 0.f;                 // this lane's share of the sum of the unrounded weights: the lse (a row
+                                       // with a handful of keys would show the rounding in its lse otherwise)
   f32x4 acc[MP_FB];                    // acc[fb][r] = O[head c][16 fb + 4 g + r]
 #pragma unroll
   for (int fb = 0; fb < MP_FB; ++fb) acc[fb] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -234,7 +269,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) pf[4 * h + r] = to_elem(fast_exp2(st[h][r] - m_run));
+          for (int r = 0; r < 4; ++r) {
+            const float p = fast_exp2(st[h][r] - m_run);
+            l_exact += p;
+            pf[4 * h + r] = to_elem(p);
+          }
 
         // out^T block fb: rows = features 16 fb + (0..15), slots = tokens 4 g + (0..3), 16 + 4 g + (0..3)
         l_acc = mfma16(ones, pf, l_acc);
@@ -268,6 +307,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       const float alpha = up ? fast_exp2(m_run - m_new) : 1.0f;
       m_run = m_new;
       l_acc *= alpha;
+      l_exact *= alpha;
 #pragma unroll
       for (int fb = 0; fb < MP_FB; ++fb) acc[fb] *= alpha;
     }
@@ -292,7 +332,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const float inv = 1.0f / fmaxf(l, 1.0e-30f);
   elem_t* dst_row = CL_ARG_OUT + qrow * CL_CKV;
 #if CL_EMIT_LSE
-  if (g == 0) CL_ARG_LSE[qrow] = l > 0.f ? m_run + fast_log2(l) : CL_NEG_INF;
+  l_exact += lane_xor(l_exact, lane, 16);
+  l_exact += lane_xor(l_exact, lane, 32);
+  if (g == 0) CL_ARG_LSE[qrow] = l_exact > 0.f ? m_run + fast_log2(l_exact) : CL_NEG_INF;
 #endif
 #pragma unroll
   for (int fb = 0; fb < MP_FB; ++fb) {

@@ -18,8 +18,8 @@ from dataclasses import dataclass
 
 from ...schedule.plan import KernelPlan, ParamSpec
 from .errors import NotDenseAttention, UnsupportedTiling
-from .kinds import (BUILT_KINDS, CAUSAL_KINDS, MLA_PAGED_DECODE, PAGED_DECODE, PAGED_DECODE_SLAB,
-                    RAGGED_PREFILL_CAUSAL)
+from .kinds import (BUILT_KINDS, CAUSAL_KINDS, MLA_PAGED_DECODE, MLA_PAGED_PREFILL_CAUSAL, PAGED_DECODE,
+                    PAGED_DECODE_SLAB, RAGGED_PREFILL_CAUSAL)
 from .specs import CombineTiling, MLASpec, PagingSpec
 
 KV_STEP = 32  # tokens one wave consumes per step of the decode template
@@ -254,28 +254,39 @@ def _prefill_plan(spec: PagingSpec, dense: DenseAttention) -> KernelPlan:
 # ----------------------------------------------------------------------------- paged MLA decode
 # Parameter order of the reference's operator (``python/cleave/dynamic/reference.py:282-295``):
 # q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, sm_scale, [partials], out, lse.
+def _mla_rows_dim(spec: MLASpec) -> str:
+    """Extent of the query / output row axis: requests (decode) or packed query tokens (prefill)."""
+    return spec.tokens_dim if spec.kind == MLA_PAGED_PREFILL_CAUSAL else spec.batch_dim
+
+
 def _mla_params(spec: MLASpec, dense: DenseMLA):
-    dt, b, pages = dense.dtype, spec.batch_dim, spec.pages_dim
+    """Decode: q_nope, q_pe, ckv_cache, kpe_cache, kv_indptr, kv_indices, sm_scale; the causal
+    prefill operator has qo_indptr before kv_indptr (``python/cleave/dynamic/reference.py:324-339``)."""
+    dt, b, pages = dense.dtype, _mla_rows_dim(spec), spec.pages_dim
     ph = lambda n: f"PlaceHolder_{n}"  # noqa: E731
     params = [
         ParamSpec(ph(spec.query_inputs[0]), dt, (b, spec.num_qo_heads, dense.ckv), "input"),
         ParamSpec(ph(spec.query_inputs[1]), dt, (b, spec.num_qo_heads, dense.kpe), "input"),
         ParamSpec(ph(spec.cache_inputs[0]), dt, (pages, spec.page_size, dense.ckv), "input"),
         ParamSpec(ph(spec.cache_inputs[1]), dt, (pages, spec.page_size, dense.kpe), "input"),
-        ParamSpec(ph(spec.indptr_input), "int32", (spec.indptr_dim,), "input"),
-        ParamSpec(ph(spec.index_input), "int32", (spec.index_dim,), "input"),
-        ParamSpec(spec.scale_input, "float32", (), "scalar"),
     ]
-    operands = {"Q": params[0].name, "QPE": params[1].name, "KV": params[2].name, "KPE": params[3].name,
-                "INDPTR": params[4].name, "INDICES": params[5].name}
+    operands = {"Q": params[0].name, "QPE": params[1].name, "KV": params[2].name, "KPE": params[3].name}
+    if spec.kind == MLA_PAGED_PREFILL_CAUSAL:
+        params.append(ParamSpec(ph(spec.query_indptr_input), "int32", (spec.indptr_dim,), "input"))
+        operands["QINDPTR"] = params[-1].name
+    params += [ParamSpec(ph(spec.indptr_input), "int32", (spec.indptr_dim,), "input"),
+               ParamSpec(ph(spec.index_input), "int32", (spec.index_dim,), "input"),
+               ParamSpec(spec.scale_input, "float32", (), "scalar")]
+    operands.update(INDPTR=params[-3].name, INDICES=params[-2].name)
     return params, operands
 
 
 def _mla_outputs(spec: MLASpec, dense: DenseMLA):
-    outs = [ParamSpec("OutputNode_0", dense.out_dtype, (spec.batch_dim, spec.num_qo_heads, dense.ckv), "output")]
+    rows = _mla_rows_dim(spec)
+    outs = [ParamSpec("OutputNode_0", dense.out_dtype, (rows, spec.num_qo_heads, dense.ckv), "output")]
     operands = {"OUT": "OutputNode_0"}
     if spec.emit_lse:
-        outs.append(ParamSpec("OutputNode_1", "float32", (spec.batch_dim, spec.num_qo_heads), "output"))
+        outs.append(ParamSpec("OutputNode_1", "float32", (rows, spec.num_qo_heads), "output"))
         operands["OUT1"] = "OutputNode_1"
     return outs, operands
 
@@ -292,11 +303,16 @@ def mla_chunk_pages_expr(spec: MLASpec, chunk_pages: int) -> str:
 
 
 def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None) -> KernelPlan:
-    dyn = (spec.batch_dim, spec.pages_dim, spec.index_dim)
-    problem = {"paged": True, "page_size": spec.page_size, "heads": spec.num_qo_heads, "ckv": dense.ckv,
-               "kpe": dense.kpe, "emit_lse": bool(spec.emit_lse), "batch": None, "skv": 0, "scale": 1.0,
-               "dim_names": {"batch": spec.batch_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim}}
+    prefill = spec.kind == MLA_PAGED_PREFILL_CAUSAL
+    dim_names = {"total_q": spec.tokens_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim} if prefill else \
+        {"batch": spec.batch_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim}
+    dyn = tuple(dim_names.values())
+    problem = {"paged": True, "prefill": prefill, "page_size": spec.page_size, "heads": spec.num_qo_heads,
+               "ckv": dense.ckv, "kpe": dense.kpe, "emit_lse": bool(spec.emit_lse), "batch": None, "skv": 0, "scale": 1.0,
+               "dim_names": dim_names}
     tiling, extra = {}, {}
+    if prefill:     # the request count follows from the row pointers
+        extra["derived_dims"] = [("batch", f"{spec.indptr_dim} - 1")]
     if split:
         tiling["CHUNK_PAGES"] = dense.chunk_pages
         extra["derived_dims"] = [("chunk_pages", mla_chunk_pages_expr(spec, dense.chunk_pages))]

@@ -15,8 +15,8 @@ MLA_PAGED_PREFILL_CAUSAL = "mla_paged_prefill_causal"
 MLA_KINDS = (MLA_PAGED_DECODE, MLA_PAGED_PREFILL_CAUSAL)
 SPLIT_KINDS = (PAGED_DECODE, PAGED_DECODE_SLAB, MLA_PAGED_DECODE)
 
-# Layers this back end has a HIP template for; the others are recognised and refused.
-BUILT_KINDS = (PAGED_DECODE, PAGED_DECODE_SLAB, PAGED_PREFILL_CAUSAL, RAGGED_PREFILL_CAUSAL, MLA_PAGED_DECODE)
+# Layers this back end has a HIP template for (all of them).
+BUILT_KINDS = KINDS + MLA_KINDS
 
 OPTIONAL_FIELDS = ("batch_dim", "tokens_dim", "kv_tokens_dim", "pages_dim", "index_dim", "index_input",
                    "last_page_len_input", "query_indptr_input", "grid_order")

@@ -303,3 +303,48 @@ def gqa_ragged_prefill_reference(dims, q_lens, kv_lens, dtype=None):
         return k[ks:ks + kv_len], v[ks:ks + kv_len]
 
     return _prefill_reference(hq, hkv, d, total_q, q_lens, kv_lens, dtype or torch.bfloat16, rows_of)
+
+
+# ----------------------------------------------------------------------------- MLA paged prefill
+def mla_paged_prefill_inputs(dims, q_lens, kv_lens, scale=None, dtype=None, device="cuda", seed=SEED):
+    """q_nope, q_pe, ckv_cache, kpe_cache, qo_indptr, kv_indptr, kv_indices, sm_scale
+    (``python/cleave/dynamic/reference.py:324-339``); ``dims`` = (qo_heads, ckv, kpe, num_pages,
+    n_idx, total_q)."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    heads, ckv, kpe, num_pages, n_idx, total_q = dims[:6]
+    gen = _generator(device, seed)
+    kv_indptr = _indptr(kv_lens)
+    kv_indices = _pad_indices(_page_table(num_pages, kv_indptr[-1], device, seed), n_idx)
+
+    def randn(*shape):
+        return torch.randn(*shape, device=device, dtype=dtype, generator=gen)
+
+    return [randn(total_q, heads, ckv), randn(total_q, heads, kpe), randn(num_pages, 1, ckv), randn(num_pages, 1, kpe),
+            _i32(_indptr(q_lens), device), _i32(kv_indptr, device), kv_indices,
+            float(ckv + kpe) ** -0.5 if scale is None else float(scale)]
+
+
+def mla_paged_prefill_reference(dims, q_lens, kv_lens, dtype=None):
+    """``python/cleave/dynamic/reference.py:341-370``: per request with both lengths positive, its
+    query rows attend the rows its table slice names under the end-aligned causal mask."""
+    torch = _torch()
+    dtype = dtype or torch.bfloat16
+    heads, ckv, _kpe, _pages, _n_idx, total_q = dims[:6]
+
+    def reference(q_nope, q_pe, ckv_cache, kpe_cache, qo_indptr, kv_indptr, kv_indices, sm_scale):
+        out = torch.zeros(total_q, heads, ckv, device=q_nope.device, dtype=dtype)
+        lse = torch.full((total_q, heads), NEG_INF, device=q_nope.device, dtype=torch.float32)
+        qo, kvp = qo_indptr.tolist(), kv_indptr.tolist()
+        for r, (q_len, kv_len) in enumerate(zip(q_lens, kv_lens)):
+            if q_len <= 0 or kv_len <= 0:
+                continue
+            qs, qe = int(qo[r]), int(qo[r + 1])
+            pages = kv_indices[int(kvp[r]):int(kvp[r]) + int(kv_len)].long()
+            o, l = _mla_attend_rows(q_nope[qs:qe], q_pe[qs:qe], ckv_cache[pages, 0], kpe_cache[pages, 0], sm_scale,
+                                    causal_keep(int(q_len), int(kv_len), q_nope.device))
+            out[qs:qe] = o.to(dtype)
+            lse[qs:qe] = l
+        return [out, lse]
+
+    return reference

@@ -1,8 +1,8 @@
 """Shipped dynamic operators: the spec that names each one's inputs and the tiling it is
 built at (``python/cleave/dynamic/registry.py:37-231``).  Of the reference's nine operators
-the four decode ones are built here (paged GQA: page size 1 with 8 and 4 kv heads, page size 64;
-paged MLA); the causal prefill ones are recognised by the frontend and refused by the access
-layer until their templates exist."""
+All nine of the reference's operators are built: the four decode ones (paged GQA: page size 1
+with 8 and 4 kv heads, page size 64; paged MLA) and the five causal prefill ones (GQA with a
+token table or packed keys, 8 and 4 kv heads; paged MLA)."""
 
 from __future__ import annotations
 
@@ -10,7 +10,8 @@ from dataclasses import dataclass, field
 
 from ..runtime.validate import Tolerance
 from . import workloads as _wl
-from .paging import PAGED_DECODE_SLAB, MLASpec, PagingSpec
+from .paging import (MLA_PAGED_PREFILL_CAUSAL, PAGED_DECODE_SLAB, PAGED_PREFILL_CAUSAL, RAGGED_PREFILL_CAUSAL, MLASpec,
+                     PagingSpec)
 
 # Paged kernels reproduce their references far more tightly than the loose default bound;
 # equal_nan stays off: an empty request is defined as 0 / -inf, so a NaN is a defect.
@@ -59,6 +60,12 @@ class DynamicOperator:
         from .paging.apply import _mla_outputs, _mla_params, _mla_plan, _paged_outputs, _paged_params, _plan
 
         t = self.tuned_tiling
+        if self.spec.kind in (PAGED_PREFILL_CAUSAL, RAGGED_PREFILL_CAUSAL):
+            from .paging.apply import _prefill_plan
+
+            dense = DenseAttention(16, 32, t["head_dim"], self.spec.num_kv_heads * 64, "bfloat16", "bfloat16",
+                                   waves=self.spec.num_kv_heads)
+            return HipCodeGen().gen(_prefill_plan(self.spec, dense))
         if self.is_mla:
             dense = DenseMLA(self.dims[0], self.dims[1], self.dims[2], "bfloat16", "bfloat16")
             params, ops = _mla_params(self.spec, dense)
@@ -88,9 +95,29 @@ OPERATORS = {op.name: op for op in (
                    pass_configs={}),
         dict(query_rows=16, kv_tile=32, head_dim=128, waves=4), (32, 8, 128),
         _wl.WORKLOADS["gqa_paged_decode_h32_kv8_d128_ps64"], page_size=64),
+    # causal prefill over ragged queries: keys through a token table ...
+    *(DynamicOperator(
+        f"gqa_paged_prefill_causal_h32_kv{kv}_d128_ps1",
+        PagingSpec(num_qo_heads=32, num_kv_heads=kv, kind=PAGED_PREFILL_CAUSAL, causal=True),
+        dict(query_rows=16, kv_tile=32, head_dim=128), (32, kv, 128),
+        _wl.WORKLOADS[f"gqa_paged_prefill_causal_h32_kv{kv}_d128_ps1"], page_size=1) for kv in (8, 4)),
+    # ... or packed per request
+    *(DynamicOperator(
+        f"gqa_ragged_prefill_causal_h32_kv{kv}_d128",
+        PagingSpec(num_qo_heads=32, num_kv_heads=kv, kind=RAGGED_PREFILL_CAUSAL, causal=True, rasterization=None,
+                   cache_inputs=("K", "V")),
+        dict(query_rows=16, kv_tile=32, head_dim=128), (32, kv, 128),
+        _wl.WORKLOADS[f"gqa_ragged_prefill_causal_h32_kv{kv}_d128"], page_size=1) for kv in (8, 4)),
     # latent attention: one compressed cache (keys and values) + a rope cache, 16 heads, token table
     DynamicOperator(
         "mla_paged_decode_h16_ckv512_kpe64_ps1", MLASpec(num_qo_heads=16),
         dict(query_rows=16, kv_tile=32, n_threads=64, ckv=512, kpe=64), (16, 512, 64),
         _wl.WORKLOADS["mla_paged_decode_h16_ckv512_kpe64_ps1"], page_size=1, scale=_wl.MLA_SM_SCALE),
+    DynamicOperator(
+        "mla_paged_prefill_causal_h16_ckv512_kpe64_ps1",
+        MLASpec(num_qo_heads=16, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True, index_window_tiles=4, prefetch=False,
+                rasterization=1, query_inputs=("Q_NOPE", "Q_PE"), cache_inputs=("CKV_CACHE", "KPE_CACHE"),
+                index_input="KV_INDICES"),
+        dict(query_rows=16, kv_tile=32, n_threads=64, ckv=512, kpe=64), (16, 512, 64),
+        _wl.WORKLOADS["mla_paged_prefill_causal_h16_ckv512_kpe64_ps1"], page_size=1, scale=_wl.MLA_SM_SCALE),
 )}

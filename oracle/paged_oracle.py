@@ -30,7 +30,10 @@ access layer.  TEST INFRASTRUCTURE: see the package docstring.
                          of the same keys; row i equals ``attend`` over the first
                          ``kv_len - q_len + i + 1`` keys (the mask as a prefix length); rows with
                          ``kv_len - q_len + i < 0`` are 0 / -inf; token-table and packed forms
-                         agree on the same rows.
+                         agree on the same rows;
+  * ``mla_prefill``      ``mla_paged_prefill_reference`` (``reference.py:341-370``): the MLA scores
+                         and latent values of ``mla_attend`` under ``causal_keep``.  Pin: equals
+                         ``prefill`` on the joined features with the latent part as values.
 """
 
 from __future__ import annotations
@@ -179,6 +182,31 @@ def prefill(q, k, v, qo_indptr, kv_indptr, kv_indices, q_lens, kv_lens, sm_scale
             kk, vv = kf[rows, 0], vf[rows, 0]
         o, l = _attend_masked(qf[qs:qs + ql], np.repeat(kk, group, axis=1), np.repeat(vv, group, axis=1), sm_scale,
                               causal_keep(ql, kl))
+        out[qs:qs + ql] = round_to_dtype(o, out_dtype)
+        lse[qs:qs + ql] = l
+    return out, lse
+
+
+def mla_prefill(q_nope, q_pe, ckv_cache, kpe_cache, qo_indptr, kv_indptr, kv_indices, q_lens, kv_lens, sm_scale,
+                out_dtype="bfloat16"):
+    """-> ``(out (total_q, heads, ckv) float32 on out_dtype's grid, lse (total_q, heads) float32)``."""
+    qn, qp, cc, pc = to_f32(q_nope), to_f32(q_pe), to_f32(ckv_cache), to_f32(kpe_cache)
+    as_i64 = lambda a: np.asarray(a.cpu() if hasattr(a, "cpu") else a, dtype=np.int64)  # noqa: E731
+    qo, kvp, idx = as_i64(qo_indptr), as_i64(kv_indptr), as_i64(kv_indices)
+    total_q, heads, ckv = qn.shape
+    out = np.zeros((total_q, heads, ckv), dtype=np.float32)
+    lse = np.full((total_q, heads), -np.inf, dtype=np.float32)
+    for r, (ql, kl) in enumerate(zip(q_lens, kv_lens)):
+        ql, kl = int(ql), int(kl)
+        if ql <= 0 or kl <= 0:
+            continue
+        qs = int(qo[r])
+        rows = idx[int(kvp[r]):int(kvp[r]) + kl]
+        # scores of both terms as one product over joined features; values = the latent rows
+        q_joined = np.concatenate([qn[qs:qs + ql], qp[qs:qs + ql]], axis=-1)
+        k_joined = np.concatenate([cc[rows, 0], pc[rows, 0]], axis=-1)[:, None, :].repeat(heads, axis=1)
+        v_latent = cc[rows, 0][:, None, :].repeat(heads, axis=1)
+        o, l = _attend_masked(q_joined, k_joined, v_latent, sm_scale, causal_keep(ql, kl))
         out[qs:qs + ql] = round_to_dtype(o, out_dtype)
         lse[qs:qs + ql] = l
     return out, lse

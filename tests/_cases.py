@@ -181,3 +181,67 @@ def mla_paged_decode_op(heads=16, ckv=512, kpe=64, dtype=cl.bf16, name=None):
                           "kv_indptr": cl.Tensor[_batch + 1, cl.i32], "kvi": cl.Tensor[_n_idx, cl.i32],
                           "sm_scale": cl.Scalar[cl.f32]}
     return cleave_amd.jit(name=name, dtype=dtype)(op)
+
+
+_total_q, _total_kv = cl.dims("total_q total_kv", dynamic=True)
+_q_len = cl.Dim("q_len", dynamic=True)
+
+
+def prefill_op(hq=32, hkv=8, d=128, ragged=False, dtype=cl.bf16, name=None):
+    """The causal prefill operators as ``@jit`` programs (the reference's registry forms,
+    ``demo/dynamic/gqa_paged_prefill.py`` / ``gqa_ragged_prefill.py``): ragged query rows per
+    request; keys through a token table, or packed per request."""
+    g = hq // hkv
+    if ragged:
+        name = name or f"gqa_ragged_prefill_causal_h{hq}_kv{hkv}_d{d}"
+
+        def op(q, k, v, qo_indptr, kv_indptr, sm_scale):
+            rows = cl.PageTable(qo_indptr, length=_q_len)
+            keys = cl.PageTable(kv_indptr, length=_kv_len)
+            qr = cl.paged_gather(q, rows).view(_batch, hkv, g, _q_len, d)
+            kr = cl.paged_gather(k, keys).view(_batch, hkv, 1, _kv_len, d)
+            vr = cl.paged_gather(v, keys).view(_batch, hkv, 1, _kv_len, d)
+            p, lse = cl.softmax((qr @ kr.mT) * sm_scale, dim=-1, causal=True, return_lse=True)
+            return (p @ vr).view(_total_q, hq, d), lse.view(_total_q, hq)
+
+        op.__annotations__ = {"q": cl.Tensor[_total_q, hq, d], "k": cl.Tensor[_total_kv, hkv, d],
+                              "v": cl.Tensor[_total_kv, hkv, d], "qo_indptr": cl.Tensor[_batch + 1, cl.i32],
+                              "kv_indptr": cl.Tensor[_batch + 1, cl.i32], "sm_scale": cl.Scalar[cl.f32]}
+    else:
+        name = name or f"gqa_paged_prefill_causal_h{hq}_kv{hkv}_d{d}_ps1"
+
+        def op(q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, sm_scale):
+            rows = cl.PageTable(qo_indptr, length=_q_len)
+            pages = cl.PageTable(kv_indptr, kv_indices, length=_kv_len)
+            qr = cl.paged_gather(q, rows).view(_batch, hkv, g, _q_len, d)
+            k = cl.paged_gather(k_cache, pages).view(_batch, hkv, 1, _kv_len, d)
+            v = cl.paged_gather(v_cache, pages).view(_batch, hkv, 1, _kv_len, d)
+            p, lse = cl.softmax((qr @ k.mT) * sm_scale, dim=-1, causal=True, return_lse=True)
+            return (p @ v).view(_total_q, hq, d), lse.view(_total_q, hq)
+
+        op.__annotations__ = {"q": cl.Tensor[_total_q, hq, d], "k_cache": cl.Tensor[_num_pages, 1, hkv, d],
+                              "v_cache": cl.Tensor[_num_pages, 1, hkv, d], "qo_indptr": cl.Tensor[_batch + 1, cl.i32],
+                              "kv_indptr": cl.Tensor[_batch + 1, cl.i32], "kv_indices": cl.Tensor[_n_idx, cl.i32],
+                              "sm_scale": cl.Scalar[cl.f32]}
+    return cleave_amd.jit(name=name, dtype=dtype)(op)
+
+
+def mla_paged_prefill_op(heads=16, ckv=512, kpe=64, dtype=cl.bf16, name=None):
+    """The paged MLA causal prefill operator as a ``@jit`` program (the reference's registry form,
+    ``demo/dynamic/mla_paged_prefill.py``)."""
+    name = name or f"mla_paged_prefill_causal_h{heads}_ckv{ckv}_kpe{kpe}_ps1"
+
+    def op(q_nope, q_pe, ckv_cache, kpe_cache, qo_indptr, kv_indptr, kv_indices, sm_scale):
+        rows = cl.PageTable(qo_indptr, length=_q_len)
+        pages = cl.PageTable(kv_indptr, kv_indices, length=_kv_len)
+        qn, qp = cl.paged_gather(q_nope, rows), cl.paged_gather(q_pe, rows)     # (batch, heads, q_len, width)
+        c = cl.paged_gather(ckv_cache, pages).view(_batch, 1, _kv_len, ckv)
+        r = cl.paged_gather(kpe_cache, pages).view(_batch, 1, _kv_len, kpe)
+        p, lse = cl.softmax((qn @ c.mT + qp @ r.mT) * sm_scale, dim=-1, causal=True, return_lse=True)
+        return (p @ c).view(_total_q, heads, ckv), lse.view(_total_q, heads)
+
+    op.__annotations__ = {"q_nope": cl.Tensor[_total_q, heads, ckv], "q_pe": cl.Tensor[_total_q, heads, kpe],
+                          "ckv_cache": cl.Tensor[_num_pages, 1, ckv], "kpe_cache": cl.Tensor[_num_pages, 1, kpe],
+                          "qo_indptr": cl.Tensor[_batch + 1, cl.i32], "kv_indptr": cl.Tensor[_batch + 1, cl.i32],
+                          "kv_indices": cl.Tensor[_n_idx, cl.i32], "sm_scale": cl.Scalar[cl.f32]}
+    return cleave_amd.jit(name=name, dtype=dtype)(op)

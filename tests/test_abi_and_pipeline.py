@@ -150,9 +150,20 @@ def test_paged_mla_layer_plans_and_signature():
     assert dict(pair["derived_dims"])["chunk_pages"].startswith("max(32, min(512, ceildiv(n_idx")
     scratch = {p["name"]: p for p in pair["params"] if p["role"] == "scratch"}
     assert scratch["Partial_PO_split"]["shape"] == ["ceildiv(n_idx, chunk_pages) + batch", 32, 512]
-    with pytest.raises(UnsupportedTiling, match="not built"):
+    with pytest.raises(UnsupportedTiling, match="decode transformation"):
         build_split_decode(MLASpec(16, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True), DenseMLA(16, 512, 64, "bfloat16", "bfloat16"),
                            8, CombineTiling(split=8))
+    pre = parse_manifest(registry.OPERATORS["mla_paged_prefill_causal_h16_ckv512_kpe64_ps1"].kernel_source())
+    assert [p["name"] for p in pre["params"]] == ["PlaceHolder_Q_NOPE", "PlaceHolder_Q_PE", "PlaceHolder_CKV_CACHE",
+                                                 "PlaceHolder_KPE_CACHE", "PlaceHolder_QO_INDPTR", "PlaceHolder_KV_INDPTR",
+                                                 "PlaceHolder_KV_INDICES", "sm_scale", "OutputNode_0", "OutputNode_1"]
+    assert pre["launches"][0]["grid"][0] == "total_q" and dict(pre["derived_dims"]) == {"batch": "len_indptr - 1"}
+    gqa = parse_manifest(registry.OPERATORS["gqa_ragged_prefill_causal_h32_kv8_d128"].kernel_source())
+    assert [p["name"] for p in gqa["params"]] == ["PlaceHolder_Q", "PlaceHolder_K", "PlaceHolder_V", "PlaceHolder_QO_INDPTR",
+                                                 "PlaceHolder_KV_INDPTR", "sm_scale", "OutputNode_0", "OutputNode_1"]
+    assert gqa["launches"][0]["grid"][0] == "ceildiv(total_q, 4) + batch" and gqa["launches"][0]["block"][0] == 512
+    assert set(registry.OPERATORS) >= {"gqa_paged_prefill_causal_h32_kv8_d128_ps1", "gqa_paged_prefill_causal_h32_kv4_d128_ps1",
+                                       "gqa_ragged_prefill_causal_h32_kv4_d128"} and len(registry.OPERATORS) == 9
     with pytest.raises(NotDenseAttention, match="same operator family"):
         build_split_decode(MLASpec(16), DenseAttention(16, 32, 128, 256, "bfloat16", "bfloat16"), 8, CombineTiling(split=8))
     with pytest.raises(UnsupportedTiling, match="heads"):

@@ -9,7 +9,7 @@ import torch
 
 from cleave_amd.codegen import HipCodeGen
 from cleave_amd.dynamic import reference as dref
-from cleave_amd.dynamic.paging import CombineTiling, DenseMLA, MLASpec, build_split_decode
+from cleave_amd.dynamic.paging import MLA_PAGED_PREFILL_CAUSAL, CombineTiling, DenseMLA, MLASpec, build_split_decode
 from cleave_amd.dynamic.paging.apply import _mla_outputs, _mla_params, _mla_plan
 from cleave_amd.runtime.compile import _compile, _load_main_kernel_from_code
 from oracle import paged_oracle
@@ -104,3 +104,32 @@ def test_registry_mla_operator_workloads(axes):
     args = dref.mla_paged_decode_inputs((batch, 16, 512, 64, pool, n_idx), lens, scale=op.scale, device="cpu")
     for split in (None, 8):
         check(mla_kernel(split=split), args, lens, f"registry axes {axes} split={split}")
+
+
+def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16"):
+    spec = MLASpec(num_qo_heads=heads, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True)
+    spec.validate()
+    dense = DenseMLA(heads, ckv, kpe, dtype, dtype)
+    params, ops = _mla_params(spec, dense)
+    outs, out_ops = _mla_outputs(spec, dense)
+    loaded = _load_main_kernel_from_code(HipCodeGen().gen(_mla_plan(spec, dense, "main", params + outs, {**ops, **out_ops})))
+    return _compile(loaded, loaded.manifest["out_idx"])
+
+
+@pytest.mark.parametrize("q_lens,kv_lens", [([1, 4, 5, 33, 0, 40, 7], [1, 4, 40, 33, 9, 300, 3]), ([6, 0, 3], [0, 5, 3]),
+                                            ([90], [700])])
+def test_paged_mla_causal_prefill(q_lens, kv_lens):
+    """Ragged query rows, one item per query token: equal lengths, a cached prefix, windows shorter
+    than the query run (fully masked rows), requests without queries or without keys, a long
+    prefix (table windows reloaded)."""
+    tq, tk = sum(q_lens), sum(kv_lens)
+    args = dref.mla_paged_prefill_inputs((16, 512, 64, 4 * tk + 64, tk + 3, tq), q_lens, kv_lens, device="cpu")
+    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens}", flush=True)
+    out, lse = mla_prefill_kernel()(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+    torch.cuda.synchronize()
+    got_o, got_l = out.float().cpu().numpy(), lse.cpu().numpy()
+    want_o, want_l = paged_oracle.mla_prefill(*args[:7], q_lens, kv_lens, args[7])
+    np.testing.assert_allclose(got_o, want_o, rtol=1e-2, atol=1e-2)
+    live = np.isfinite(want_l)
+    np.testing.assert_allclose(got_l[live], want_l[live], rtol=1e-3, atol=1e-3)
+    assert np.all(np.isneginf(got_l[~live])) and np.all(got_o[~live.any(axis=1)] == 0)

@@ -174,3 +174,55 @@ def test_registry_mla_decode_operator(cache_root):
     live = np.isfinite(want_l)
     np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
     assert np.all(np.isneginf(lse.cpu().numpy()[~live]))
+
+
+@pytest.mark.parametrize("name", ["gqa_paged_prefill_causal_h32_kv4_d128_ps1", "gqa_ragged_prefill_causal_h32_kv8_d128"])
+def test_registry_prefill_operators(cache_root, name):
+    """A shipped causal prefill operator of each key layout through ``compile``: validated over the
+    captured workload axes against the torch reference, timed; then one call against the oracle."""
+    from cleave_amd.dynamic import OPERATORS
+    from cleave_amd.dynamic import reference as dref
+
+    op = OPERATORS[name]
+    hq, hkv, d = op.dims
+    ragged = "ragged" in name
+    kernel = cleave_amd.compile(C.prefill_op(hq, hkv, d, ragged=ragged, name=name), schedule=P.ScheduleConfig(topk=1),
+                                max_workloads=2)
+    rep = kernel.report
+    assert rep.best() is not None and len(rep.correct) >= 1 and rep.n_workloads == len(op.workloads)
+    q_lens, kv_lens = [3, 0, 40, 9], [10, 5, 40, 2]
+    tq, tk = sum(q_lens), sum(kv_lens)
+    if ragged:
+        args = dref.gqa_ragged_prefill_inputs((hq, hkv, d, tq, tk), q_lens, kv_lens, device="cuda")
+        table = None
+    else:
+        args = dref.gqa_paged_prefill_inputs((hq, hkv, d, 500, tk, tq), q_lens, kv_lens, device="cuda")
+        table = args[5].cpu()
+    out, lse = kernel(*args)
+    want_o, want_l = paged_oracle.prefill(*[a.cpu() for a in args[:5]], table, q_lens, kv_lens, args[-1])
+    _close(out, want_o)
+    live = np.isfinite(want_l)
+    np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
+    assert np.all(np.isneginf(lse.cpu().numpy()[~live]))
+
+
+def test_registry_mla_prefill_operator(cache_root):
+    """The shipped paged MLA causal prefill operator through ``compile`` over its captured workload
+    axes, then one call against the numpy oracle."""
+    from cleave_amd.dynamic import OPERATORS
+    from cleave_amd.dynamic import reference as dref
+
+    name = "mla_paged_prefill_causal_h16_ckv512_kpe64_ps1"
+    op = OPERATORS[name]
+    kernel = cleave_amd.compile(C.mla_paged_prefill_op(name=name), schedule=P.ScheduleConfig(topk=1), max_workloads=2)
+    rep = kernel.report
+    assert rep.best() is not None and len(rep.correct) >= 1 and rep.n_workloads == len(op.workloads)
+    q_lens, kv_lens = [3, 0, 20, 6], [10, 5, 20, 2]
+    args = dref.mla_paged_prefill_inputs((16, 512, 64, 400, sum(kv_lens), sum(q_lens)), q_lens, kv_lens, scale=op.scale,
+                                         device="cuda")
+    out, lse = kernel(*args)
+    want_o, want_l = paged_oracle.mla_prefill(*[a.cpu() for a in args[:7]], q_lens, kv_lens, args[7])
+    _close(out, want_o)
+    live = np.isfinite(want_l)
+    np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
+    assert np.all(np.isneginf(lse.cpu().numpy()[~live]))

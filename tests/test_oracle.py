@@ -223,3 +223,62 @@ def test_mla_decode_depends_on_the_table_only_through_the_rows_it_names():
     cc2[perm], pc2[perm] = cc, pc
     out2, lse2 = paged_oracle.mla_decode(qn, qp, cc2, pc2, ptr, perm[idx].astype(np.int32), lens, 0.2)
     assert np.array_equal(out, out2) and np.array_equal(lse, lse2)
+
+
+# ----------------------------------------------------------------------------- causal prefill
+def _prefill_case(q_lens, kv_lens, hq=8, hkv=2, d=16, seed=9):
+    rng = np.random.default_rng(seed)
+    tq, tk = sum(q_lens), sum(kv_lens)
+    q = rng.standard_normal((tq, hq, d)).astype(np.float32)
+    k = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((tk, hkv, d)).astype(np.float32)
+    qo = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    kvp = np.concatenate([[0], np.cumsum(kv_lens)]).astype(np.int32)
+    return q, k, v, qo, kvp
+
+
+def test_causal_mask_is_a_prefix_length_per_query_row():
+    """Row i of a request sees exactly the first kv_len - q_len + i + 1 keys: each row must equal
+    plain attention over that prefix (an off-by-one or a start-aligned mask breaks this), rows
+    whose prefix is empty are 0 / -inf, and a request with one query row is a decode."""
+    q_lens, kv_lens = [5, 3, 1, 4], [9, 3, 6, 2]          # cached prefix, equal, decode-like, window shorter than the run
+    q, k, v, qo, kvp = _prefill_case(q_lens, kv_lens)
+    out, lse = paged_oracle.prefill(q, k, v, qo, kvp, None, q_lens, kv_lens, 0.25, out_dtype="float32")
+    assert np.array_equal(paged_oracle.causal_keep(3, 5), np.array([[1, 1, 1, 0, 0], [1, 1, 1, 1, 0], [1, 1, 1, 1, 1]], bool))
+    for r, (ql, kl) in enumerate(zip(q_lens, kv_lens)):
+        for i in range(ql):
+            n = kl - ql + i + 1
+            row = qo[r] + i
+            if n <= 0:
+                assert np.all(out[row] == 0) and np.all(np.isneginf(lse[row]))
+                continue
+            kk = np.repeat(k[kvp[r]:kvp[r] + n], 4, axis=1)
+            vv = np.repeat(v[kvp[r]:kvp[r] + n], 4, axis=1)
+            want_o, want_l = paged_oracle.attend(q[row], kk, vv, 0.25)
+            np.testing.assert_allclose(out[row], want_o, rtol=1e-5, atol=1e-6)
+            np.testing.assert_allclose(lse[row], want_l, rtol=1e-5, atol=1e-6)
+
+
+def test_token_table_and_packed_prefill_agree_and_mla_prefill_is_prefill_over_joined_features():
+    q_lens, kv_lens = [4, 2], [7, 5]
+    q, k, v, qo, kvp = _prefill_case(q_lens, kv_lens)
+    out, lse = paged_oracle.prefill(q, k, v, qo, kvp, None, q_lens, kv_lens, 0.3)
+    # the same rows scattered over a pool and named by a table
+    perm = np.random.default_rng(2).permutation(40)[:k.shape[0]]
+    kc, vc = np.zeros((40, 1, 2, 16), np.float32), np.zeros((40, 1, 2, 16), np.float32)
+    kc[perm, 0], vc[perm, 0] = k, v
+    out2, lse2 = paged_oracle.prefill(q, kc, vc, qo, kvp, perm.astype(np.int32), q_lens, kv_lens, 0.3)
+    assert np.array_equal(out, out2) and np.array_equal(lse, lse2)
+    # MLA: one "kv head" whose keys are [latent | rope] and whose values are the latent part
+    rng = np.random.default_rng(4)
+    qn, qp = rng.standard_normal((6, 4, 16)).astype(np.float32), rng.standard_normal((6, 4, 8)).astype(np.float32)
+    cc, pc = rng.standard_normal((40, 1, 16)).astype(np.float32), rng.standard_normal((40, 1, 8)).astype(np.float32)
+    idx = perm[:12].astype(np.int32)
+    mo, ml = paged_oracle.mla_prefill(qn, qp, cc, pc, qo, kvp, idx, q_lens, kv_lens, 0.3, out_dtype="float32")
+    for r, (ql, kl) in enumerate(zip(q_lens, kv_lens)):
+        rows = idx[kvp[r]:kvp[r] + kl]
+        for i in range(ql):
+            n = kl - ql + i + 1
+            o, l = paged_oracle.mla_attend(qn[qo[r] + i], qp[qo[r] + i], cc[rows[:n], 0], pc[rows[:n], 0], 0.3)
+            np.testing.assert_allclose(mo[qo[r] + i], o, rtol=1e-5, atol=1e-6)
+            np.testing.assert_allclose(ml[qo[r] + i], l, rtol=1e-5, atol=1e-6)
