@@ -407,6 +407,14 @@ class HipCodeGen:
                             ("INDPTR", "CL_ARG_INDPTR"), ("INDICES", "CL_ARG_INDICES")):
             if role in op:
                 unit.define(macro, op[role])
+        if int(plan.tiling.get("SHARED", 0)):
+            # four waves share every key tile through LDS: 128 query rows per workgroup and kv head
+            if d % 64 or d > 256:
+                raise CodegenError("the LDS-shared prefill kernel needs a head dim of whole 64-feature panels (<= 256)")
+            unit.templates.append("attn_prefill_lds.hip")
+            items = f"ceildiv({p['dim_names']['total_q']}, {128 // group}) + batch"
+            unit.launch(ENTRY, (items, p["kv_heads"], 1), 256, 0, self._partial_args)
+            return
         unit.templates.append("attn_prefill.hip")
         items = f"ceildiv({p['dim_names']['total_q']}, {16 // group}) + batch"
         unit.launch(ENTRY, (items, 1, 1), p["kv_heads"] * 64, p["kv_heads"] * 16 * d * 4, self._partial_args)

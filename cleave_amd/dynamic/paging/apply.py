@@ -214,8 +214,13 @@ def chunk_pages_expr(spec, chunk_pages: int) -> str:
 # Parameter order of the reference's operators (``python/cleave/dynamic/reference.py:204-278``):
 # q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, sm_scale (token table) or
 # q, k, v, qo_indptr, kv_indptr, sm_scale (packed keys); then out (total_q, heads, d), lse.
-def _prefill_plan(spec: PagingSpec, dense: DenseAttention) -> KernelPlan:
+def _prefill_plan(spec: PagingSpec, dense: DenseAttention, shared: bool | None = None) -> KernelPlan:
+    """``shared``: the kernel whose four waves share every key tile through LDS (128 query rows per
+    workgroup, for long requests) instead of the one-wave-per-kv-head kernel with 16-row items;
+    None: follow the dense tiling (four or more waves ask for the shared form)."""
     d, dt = dense.head_dim, dense.dtype
+    if shared is None:
+        shared = dense.waves >= 4 and d % 64 == 0
     ragged = spec.kind == RAGGED_PREFILL_CAUSAL
     tq = spec.tokens_dim
     ph = lambda n: f"PlaceHolder_{n}"  # noqa: E731
@@ -245,10 +250,18 @@ def _prefill_plan(spec: PagingSpec, dense: DenseAttention) -> KernelPlan:
     problem = {"paged": True, "prefill": True, "ragged": ragged, "kv_heads": spec.num_kv_heads,
                "q_heads": spec.num_qo_heads, "group": spec.group, "head_dim": d, "vdim": d,
                "emit_lse": bool(spec.emit_lse), "units": None, "skv": 0, "sq": 0, "scale": 1.0, "dim_names": dim_names}
+    threads, rows = (256, 128) if shared else (spec.num_kv_heads * 64, 16)
     return KernelPlan(template="attn_prefill", role="main", family="attention", dtype=dense.dtype,
-                      extra={"derived_dims": [("batch", f"{spec.indptr_dim} - 1")]}, problem=problem, tiling={},
-                      params=params + outs, operands=operands, split_factor=None, dyn_dims=tuple(dim_names.values()),
-                      n_threads=spec.num_kv_heads * 64, label=f"kv={KV_STEP} q=16 thr={spec.num_kv_heads * 64}")
+                      extra={"derived_dims": [("batch", f"{spec.indptr_dim} - 1")]}, problem=problem,
+                      tiling={"SHARED": int(bool(shared))}, params=params + outs, operands=operands, split_factor=None,
+                      dyn_dims=tuple(dim_names.values()), n_threads=threads, label=f"kv={KV_STEP} q={rows} thr={threads}")
+
+
+def prefill_variants(plan: KernelPlan, spec) -> list:
+    """Both kernels of a causal prefill layer at ``plan``'s dense tiling (the search times each)."""
+    dense = read_dense_attention(plan)
+    _check_tiling(spec, dense)
+    return [_prefill_plan(spec, dense, shared=s) for s in ((False, True) if dense.head_dim % 64 == 0 else (False,))]
 
 
 # ----------------------------------------------------------------------------- paged MLA decode

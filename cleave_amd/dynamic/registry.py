@@ -65,7 +65,7 @@ class DynamicOperator:
 
             dense = DenseAttention(16, 32, t["head_dim"], self.spec.num_kv_heads * 64, "bfloat16", "bfloat16",
                                    waves=self.spec.num_kv_heads)
-            return HipCodeGen().gen(_prefill_plan(self.spec, dense))
+            return HipCodeGen().gen(_prefill_plan(self.spec, dense, shared=True))   # the measured winner
         if self.is_mla:
             dense = DenseMLA(self.dims[0], self.dims[1], self.dims[2], "bfloat16", "bfloat16")
             params, ops = _mla_params(self.spec, dense)

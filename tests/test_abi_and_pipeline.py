@@ -161,7 +161,15 @@ def test_paged_mla_layer_plans_and_signature():
     gqa = parse_manifest(registry.OPERATORS["gqa_ragged_prefill_causal_h32_kv8_d128"].kernel_source())
     assert [p["name"] for p in gqa["params"]] == ["PlaceHolder_Q", "PlaceHolder_K", "PlaceHolder_V", "PlaceHolder_QO_INDPTR",
                                                  "PlaceHolder_KV_INDPTR", "sm_scale", "OutputNode_0", "OutputNode_1"]
-    assert gqa["launches"][0]["grid"][0] == "ceildiv(total_q, 4) + batch" and gqa["launches"][0]["block"][0] == 512
+    # the operator's own kernel is the one whose four waves share key tiles through LDS (128 rows = 32 tokens x 4)
+    assert gqa["launches"][0]["grid"][:2] == ["ceildiv(total_q, 32) + batch", "8"] and gqa["launches"][0]["block"][0] == 256
+    from cleave_amd.dynamic.paging import RAGGED_PREFILL_CAUSAL, PagingSpec
+    from cleave_amd.dynamic.paging.apply import _prefill_plan
+
+    spec = PagingSpec(32, 8, kind=RAGGED_PREFILL_CAUSAL, causal=True, cache_inputs=("K", "V"))
+    rows16 = parse_manifest(HipCodeGen().gen(_prefill_plan(spec, DenseAttention(16, 32, 128, 512, "bfloat16", "bfloat16",
+                                                                                waves=8), shared=False)))
+    assert rows16["launches"][0]["grid"][0] == "ceildiv(total_q, 4) + batch" and rows16["launches"][0]["block"][0] == 512
     assert set(registry.OPERATORS) >= {"gqa_paged_prefill_causal_h32_kv8_d128_ps1", "gqa_paged_prefill_causal_h32_kv4_d128_ps1",
                                        "gqa_ragged_prefill_causal_h32_kv4_d128"} and len(registry.OPERATORS) == 9
     with pytest.raises(NotDenseAttention, match="same operator family"):

@@ -17,16 +17,16 @@ from oracle import paged_oracle
 pytestmark = pytest.mark.gpu
 
 
-def prefill_kernel(ragged, hq=32, hkv=8, d=128, dtype="bfloat16"):
+def prefill_kernel(ragged, hq=32, hkv=8, d=128, dtype="bfloat16", shared=False):
     kw = dict(cache_inputs=("K", "V")) if ragged else {}
     spec = PagingSpec(hq, hkv, kind=RAGGED_PREFILL_CAUSAL if ragged else PAGED_PREFILL_CAUSAL, causal=True, **kw)
     spec.validate()
     dense = DenseAttention(16, 32, d, hkv * 64, dtype, dtype, waves=hkv)
-    loaded = _load_main_kernel_from_code(HipCodeGen().gen(_prefill_plan(spec, dense)))
+    loaded = _load_main_kernel_from_code(HipCodeGen().gen(_prefill_plan(spec, dense, shared=shared)))
     return _compile(loaded, loaded.manifest["out_idx"])
 
 
-def check(ragged, q_lens, kv_lens, hq=32, hkv=8, d=128, pad=0, what=""):
+def check(ragged, q_lens, kv_lens, hq=32, hkv=8, d=128, pad=0, what="", shared=False):
     total_q, total_kv = sum(q_lens), sum(kv_lens)
     if ragged:
         args = dref.gqa_ragged_prefill_inputs((hq, hkv, d, total_q, total_kv), q_lens, kv_lens, device="cpu")
@@ -35,8 +35,8 @@ def check(ragged, q_lens, kv_lens, hq=32, hkv=8, d=128, pad=0, what=""):
         args = dref.gqa_paged_prefill_inputs((hq, hkv, d, 4 * total_kv + 50, total_kv + pad, total_q), q_lens, kv_lens,
                                              device="cpu")
         table = args[5]
-    print(f"prefill case ragged={ragged} h{hq}/kv{hkv} q_lens={q_lens} kv_lens={kv_lens} {what}", flush=True)
-    out, lse = prefill_kernel(ragged, hq, hkv, d)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+    print(f"prefill case ragged={ragged} shared={shared} h{hq}/kv{hkv} q_lens={q_lens} kv_lens={kv_lens} {what}", flush=True)
+    out, lse = prefill_kernel(ragged, hq, hkv, d, shared=shared)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
     torch.cuda.synchronize()
     got_o, got_l = out.float().cpu().numpy(), lse.cpu().numpy()
     want_o, want_l = paged_oracle.prefill(args[0], args[1], args[2], args[3], args[4], table, q_lens, kv_lens, args[-1])
@@ -51,23 +51,32 @@ Q_LENS = [1, 4, 5, 33, 0, 64, 7, 130]
 KV_LENS = [1, 4, 40, 33, 9, 200, 3, 130]       # equal, cached prefix, no queries, window shorter than the run
 
 
+SHARED = pytest.mark.parametrize("shared", [False, True], ids=["rows16", "lds128"])
+
+
+@SHARED
 @pytest.mark.parametrize("ragged", [False, True])
-def test_causal_prefill(ragged):
-    check(ragged, Q_LENS, KV_LENS, pad=5)
+def test_causal_prefill(ragged, shared):
+    check(ragged, Q_LENS, KV_LENS, pad=5, shared=shared)
 
 
+@SHARED
 @pytest.mark.parametrize("ragged", [False, True])
-def test_causal_prefill_four_kv_heads(ragged):
-    """Eight query heads per kv head: two tokens per 16-row tile, four waves per workgroup."""
-    check(ragged, [3, 70, 1, 0, 18], [3, 70, 50, 4, 6], hq=32, hkv=4)
+def test_causal_prefill_four_kv_heads(ragged, shared):
+    """Eight query heads per kv head: two tokens per 16-row tile (16 per 128-row workgroup)."""
+    check(ragged, [3, 70, 1, 0, 18], [3, 70, 50, 4, 6], hq=32, hkv=4, shared=shared)
 
 
-def test_causal_prefill_requests_without_keys_or_queries():
-    check(False, [5, 0, 9], [0, 7, 9], what="kv_len 0 / q_len 0")
-    check(True, [5, 0, 9], [0, 7, 9], what="kv_len 0 / q_len 0")
+@SHARED
+def test_causal_prefill_requests_without_keys_or_queries(shared):
+    check(False, [5, 0, 9], [0, 7, 9], what="kv_len 0 / q_len 0", shared=shared)
+    check(True, [5, 0, 9], [0, 7, 9], what="kv_len 0 / q_len 0", shared=shared)
 
 
-def test_causal_prefill_long_request():
-    """One request long enough for many key steps per tile and hundreds of tiles."""
-    check(True, [700], [700])
-    check(False, [300, 2], [1000, 900], what="long cached prefix")
+@SHARED
+def test_causal_prefill_long_request(shared):
+    """Requests long enough for many key steps per tile, hundreds of tiles and several 256-entry
+    table windows."""
+    check(True, [700], [700], shared=shared)
+    check(False, [300, 2], [1000, 900], what="long cached prefix", shared=shared)
+    check(False, [40, 33], [600, 290], what="table windows", shared=shared)
