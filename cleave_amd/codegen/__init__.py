@@ -412,7 +412,12 @@ class HipCodeGen:
             if d % 64 or d > 256:
                 raise CodegenError("the LDS-shared prefill kernel needs a head dim of whole 64-feature panels (<= 256)")
             unit.templates.append("attn_prefill_lds.hip")
-            items = f"ceildiv({p['dim_names']['total_q']}, {128 // group}) + batch"
+            for k, v in plan.tiling.items():
+                if k != "SHARED":
+                    unit.define(f"CL_PF_{k}", int(v))
+            # the item axis is padded to a multiple of 8 so that the kernel can hand every XCD one
+            # contiguous eighth of the (kv head, item) space
+            items = f"ceildiv(ceildiv({p['dim_names']['total_q']}, {128 // group}) + batch, 8) * 8"
             unit.launch(ENTRY, (items, p["kv_heads"], 1), 256, 0, self._partial_args)
             return
         unit.templates.append("attn_prefill.hip")

@@ -9,8 +9,13 @@
 //   image [D/64][32][64]   64-feature panels, 128-byte key rows, 16-byte chunk ^ (key & 6)
 // K is read as the A operand of scores^T = K Q^T with 16-byte reads, V with transposing reads as
 // the A operand of out^T += V^T P^T; each operand read feeds both row tiles of the wave.  Three
-// stages rotate (two steps of loads in flight), one barrier per step; the softmax is the exact
-// online one of the decode kernel, lane-local per query row.
+// stages rotate (two steps of loads in flight), one barrier per step.  The softmax is the exact
+// online one (running max per query row, accumulators rescaled only when a max moved), slimmed
+// for the vector unit, which is the busiest unit of this kernel: the loop is unrolled over the
+// three stages so that LDS addresses are immediates, steps below every row's causal limit run a
+// body without mask arithmetic, scale and max subtraction are one multiply-add per score, the
+// row maximum crosses the four key groups with two row-swap instructions, and one sum of the
+// unrounded weights serves both the normalisation and the lse.
 //
 // Work items: a new item at every multiple of PL_QT packed query tokens and at every request
 // boundary (item t = chunk w + request b for the one pair that overlaps); an item stops at the
@@ -19,6 +24,12 @@
 //   CL_HEAD_DIM (multiple of 64)  CL_KV_HEADS  CL_Q_HEADS (group divides 16)  CL_RAGGED
 //   run-time: batch, total_q, n_idx (table length / total_kv), num_pages (table form), sm_scale
 
+#ifndef CL_PF_XCD
+#define CL_PF_XCD 1
+#endif
+#ifndef CL_PF_REVERSE
+#define CL_PF_REVERSE 1
+#endif
 #define PL_STEP 32
 #define PL_GROUP (CL_Q_HEADS / CL_KV_HEADS)
 #define PL_ROWS 128
@@ -27,16 +38,18 @@
 #define PL_PANEL (PL_STEP * 64)               // elements of one 64-feature panel
 #define PL_IMG (PL_PANELS * PL_PANEL)         // elements of one operand image
 #define PL_STAGE (2 * PL_IMG)                 // K image, then V image
-#define PL_STAGES 3
+#define PL_STAGES 4
 #define PL_KJ (CL_HEAD_DIM / 32)
 #define PL_FB (CL_HEAD_DIM / 16)
 #define PL_UNITS_PER (2 * PL_PANELS)          // 1 KiB loads per wave and step: its 8-key group of every panel of K and V
-#define PL_WINDOW 256                         // table entries held in registers at a time
 static_assert(CL_Q_HEADS % CL_KV_HEADS == 0 && 16 % PL_GROUP == 0, "the head group divides the 16-row query tile");
 static_assert(CL_HEAD_DIM % 64 == 0 && CL_HEAD_DIM <= 256, "head dim in whole 64-feature panels");
 static_assert(PL_UNITS_PER < 16, "load counter range");
 
 __shared__ __attribute__((aligned(1024))) elem_t pl_tiles[PL_STAGES * PL_STAGE];
+#if !CL_RAGGED
+__shared__ __attribute__((aligned(256))) int pl_ids[2][4][64];   // table entries on their way in: [step parity][wave][lane]
+#endif
 
 typedef short pl_s16x4 __attribute__((ext_vector_type(4)));
 typedef short pl_s16x8 __attribute__((ext_vector_type(8)));
@@ -52,6 +65,11 @@ CL_DEVICE void pl_dma16(const void* gptr, unsigned lds_byte) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
                :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory");
 }
+// 4 bytes per lane, the same way
+CL_DEVICE void pl_dma4(const void* gptr, unsigned lds_byte) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)) : "memory");
+}
 template <int P>
 CL_DEVICE void pl_issue_panels(const char* src, unsigned group_byte) {
   if constexpr (P < PL_PANELS) {
@@ -60,12 +78,43 @@ CL_DEVICE void pl_issue_panels(const char* src, unsigned group_byte) {
   }
 }
 
+template <int I> struct PlC { static constexpr int value = I; };
+
+// max of x over the four lanes that share lane % 16 (the key groups of one query row): the two
+// row-swap instructions exchange 16-lane rows 1<->0', 3<->2' and then 2,3<->0',1' of a register pair
+CL_DEVICE float pl_max_over_groups(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0\n\tv_max_f32 %0, %0, %1\n\tv_mov_b32 %1, %0\n\t"
+               "s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0\n\tv_max_f32 %0, %0, %1"
+               : "+v"(a), "+v"(b));
+  return a;
+}
+
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(256, 2)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
-  const int item = blockIdx.x, head = blockIdx.y;
+  // Workgroups go to the 8 XCDs round-robin in launch order; every XCD has its own L2.  XCD x
+  // takes the x-th eighth of the (kv head, item) space (the item axis is padded to a multiple of
+  // 8), so the workgroups resident on an XCD are neighbouring items of one kv head and re-read
+  // the same keys out of that L2.  Heaviest first: within a request later items see more keys, so
+  // every eighth is walked backwards.
+  int item, head;
+  {
+    const int gx = (int)gridDim.x, launch = (int)blockIdx.x + gx * (int)blockIdx.y;
+#if CL_PF_XCD
+    const int eighth = gx * (int)gridDim.y / 8;
+    int lin = (launch % 8) * eighth + launch / 8;
+#else
+    int lin = launch;
+#endif
+#if CL_PF_REVERSE
+    lin = gx * (int)gridDim.y - 1 - lin;
+#endif
+    item = lin % gx;
+    head = lin / gx;
+  }
   // the request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item
   int req = 0;
   {
@@ -120,53 +169,62 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     return;
   }
 
-  const float scale2 = sm_scale * 1.4426950408889634f;
+  // the softmax scale as a positive factor of the raw scores (its sign goes into the Q rows, exactly)
+  const float scale2 = fmaxf(fabsf(sm_scale) * 1.4426950408889634f, 1.0e-30f);
+  const unsigned q_sign = sm_scale < 0.f ? 0x80008000u : 0u;
   const i64 row_bytes = (i64)CL_KV_HEADS * CL_HEAD_DIM * 2;
   const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_HEAD_DIM * 2;
   const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_HEAD_DIM * 2;
   const int n_steps = (ext + PL_STEP - 1) / PL_STEP;
   const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)pl_tiles;
 
-  // Table entries of a 256-key window: register k holds the entry of key 256 w + 64 k + lane
-  // (positions past the item's last key repeat it; ids outside the pool are clamped into it).
-#if !CL_RAGGED
-  auto load_window = [&](int w, int (&ids)[4]) __attribute__((always_inline)) {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      int t = w * PL_WINDOW + 64 * k + lane;
-      t = t < ext - 1 ? t : ext - 1;
-      ids[k] = pl_clamp(CL_ARG_INDICES[kv0 + t], 0, num_pages - 1);
-    }
-  };
-  int ids_cur[4], ids_next[4];     // the window the loads are in, and the one after it
-  load_window(0, ids_cur);
-  load_window(1, ids_next);        // (clamped onto the last key when there is no second window)
-#endif
   // This wave's share of step s (clamped onto the last step: a step past the end reloads the last
   // one into an image nobody reads, so the load counter holds the same number of steps at every
   // wait): key rows 8 wave + lane / 8 of every panel of K and V, the chunk for slot lane % 8.
-  auto issue_step = [&](int s, int slot) __attribute__((always_inline)) {
+  // The lane's key row is kv0 + position (packed keys) or its table entry, which `row_of` reads
+  // (positions past the item's last key repeat it; ids outside the pool are clamped into it).
+  const int my_r = 8 * wave + (lane >> 3);
+  auto key_pos = [&](int s) __attribute__((always_inline)) {
     s = s < n_steps - 1 ? s : n_steps - 1;
-    const int r = 8 * wave + (lane >> 3);
-    int t = s * PL_STEP + r;
-    t = t < ext - 1 ? t : ext - 1;
+    const int t = s * PL_STEP + my_r;
+    return t < ext - 1 ? t : ext - 1;
+  };
+  auto row_of = [&](int s) __attribute__((always_inline)) {
 #if CL_RAGGED
-    const i64 row = (i64)(kv0 + t);
+    return kv0 + key_pos(s);
 #else
-    const int in_window = s % (PL_WINDOW / PL_STEP);
-    const int k = in_window >> 1;
-    const int held = k == 0 ? ids_cur[0] : k == 1 ? ids_cur[1] : k == 2 ? ids_cur[2] : ids_cur[3];
-    const i64 row = __builtin_amdgcn_ds_bpermute((t - (s - in_window) * PL_STEP - 64 * k) << 2, held);
+    return pl_clamp(CL_ARG_INDICES[kv0 + key_pos(s)], 0, num_pages - 1);
 #endif
-    const int chunk = (lane & 7) ^ pl_swz(r);
+  };
+#if !CL_RAGGED
+  // In the loop the lane's table entry travels like the tiles do, global -> LDS on the kernel's
+  // own load counter, a step ahead of the loads that need it (a load the compiler tracks would
+  // make it wait for every load in flight): entry of step s into pl_ids[s & 1][wave][lane].
+  const unsigned ids_byte = (unsigned)(size_t)(__attribute__((address_space(3))) int*)&pl_ids[0][0][0];
+  auto fetch_id = [&](int s) __attribute__((always_inline)) {
+    pl_dma4(CL_ARG_INDICES + kv0 + key_pos(s), ids_byte + (unsigned)(((s & 1) * 4 + wave) * 256));
+  };
+  auto fetched_row = [&](int s) __attribute__((always_inline)) {
+    return pl_clamp(pl_ids[s & 1][wave][lane], 0, num_pages - 1);
+  };
+#endif
+  auto issue_step = [&](int row, int slot) __attribute__((always_inline)) {
+    const int chunk = (lane & 7) ^ pl_swz(my_r);
     const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024);
-    pl_issue_panels<0>(kbase + row * row_bytes + 16 * chunk, group_byte);
-    pl_issue_panels<0>(vbase + row * row_bytes + 16 * chunk, group_byte + PL_IMG * 2);
+    pl_issue_panels<0>(kbase + (i64)row * row_bytes + 16 * chunk, group_byte);
+    pl_issue_panels<0>(vbase + (i64)row * row_bytes + 16 * chunk, group_byte + PL_IMG * 2);
   };
 #define PL_WAITCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 
-  issue_step(0, 0);
-  issue_step(1, 1);
+  {
+    const int row0 = row_of(0), row1 = row_of(1), row2 = row_of(2);
+    issue_step(row0, 0);
+    issue_step(row1, 1);
+#if !CL_RAGGED
+    fetch_id(3);
+#endif
+    issue_step(row2, 2);
+  }
 
   // Query rows as the B operand: lane (c, g) holds Q[row][32 j + 8 g .. +8]; padded rows are 0.
   elem8 qf[2][PL_KJ];
@@ -177,13 +235,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     for (int j = 0; j < PL_KJ; ++j) {
       u32x4 raw = ld16(row + 32 * j);
       if (!live[rt]) raw = (u32x4){0u, 0u, 0u, 0u};
-      qf[rt][j] = as_elem8(raw);
+      qf[rt][j] = as_elem8(raw ^ q_sign);
     }
   }
 
   float m_run[2] = {CL_NEG_BIG, CL_NEG_BIG};   // running max of the scaled scores (log2 domain), uniform over g
-  float l_run[2] = {0.f, 0.f};                 // this lane's share of the sum of the rounded weights (normalises out)
-  float l_exact[2] = {0.f, 0.f};               // ... of the unrounded ones (the lse)
+  float l_run[2] = {0.f, 0.f};                 // this lane's share of the sum of the weights
   f32x4 acc[2][PL_FB];                         // acc[rt][fb][r] = O[row][16 fb + 4 g + r]
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt)
@@ -194,106 +251,218 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int a_lo = c * 64 + ((g ^ pl_swz(c)) << 3);
   const int vtok = 4 * g + (c >> 2);
   const int v_lo = vtok * 64 + (((((c & 3) >> 1)) ^ pl_swz(vtok)) << 3) + 4 * (c & 1);
+  // causal limit of the lane's rows relative to its first key slot (slot q of half h is key t0 + 16 h + 4 g + q)
+  const int lim_rel[2] = {limit[0] - 4 * g, limit[1] - 4 * g};
+  // Steps every key of which every live row of this wave sees need no mask: the wave's first
+  // row has the smallest limit (a wave without live rows masks nothing: its rows are not written).
+  int n_full = n_steps;
+  if (32 * wave < n_rows) {
+    const int first_limit = off + (lo + (32 * wave) / PL_GROUP - q0);
+    n_full = first_limit < 0 ? 0 : (first_limit + 1) / PL_STEP;
+    n_full = n_full < n_steps ? n_full : n_steps;
+  }
+  n_full = __builtin_amdgcn_readfirstlane(n_full);
 
-  for (int step = 0; step < n_steps; ++step) {
-    // step's images: this wave's share has landed when at most the next step's loads are
-    // outstanding; the barrier makes that everybody's share and frees the images of step - 1
-    PL_WAITCNT(PL_UNITS_PER);
-    __syncthreads();
-#if !CL_RAGGED
-    // the loads enter a new window: its entries were read a window ago; read the one after it now
-    const bool new_window = (step + 2) % (PL_WINDOW / PL_STEP) == 0 && step + 2 < n_steps;
-    if (new_window) {
-#pragma unroll
-      for (int k = 0; k < 4; ++k) ids_cur[k] = ids_next[k];
-    }
-#endif
-    issue_step(step + 2, (step + 2) % PL_STAGES);
-#if !CL_RAGGED
-    if (new_window) load_window((step + 2) / (PL_WINDOW / PL_STEP) + 1, ids_next);
-#endif
-    const elem_t* kimg = pl_tiles + (step % PL_STAGES) * PL_STAGE;
-    const elem_t* vimg = kimg + PL_IMG;
-    const int t0 = step * PL_STEP;
+  // scores^T of one step out of the K image in stage SLOT: a 16-byte read per 16-key half and
+  // 32-feature block, each feeding the wave's two row tiles
+  auto k_frag = [&](auto slot_c, int j, int h) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    return *reinterpret_cast<const elem8*>(pl_tiles + SLOT * PL_STAGE + (j >> 1) * PL_PANEL + 16 * h * 64 +
+                                           (a_lo ^ ((4 * (j & 1)) << 3)));
+  };
+  // value operand for feature block fb out of the V image in stage SLOT: rows = features
+  // 16 fb + (0..15), slots = keys 4 g + (0..3), 16 + 4 g + (0..3)
+  auto v_frag = [&](auto slot_c, int fb) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    const elem_t* p = pl_tiles + SLOT * PL_STAGE + PL_IMG + (fb >> 2) * PL_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
+    const pl_s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p));
+    const pl_s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p + 16 * 64));
+    return __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
 
-    // scores^T for the two 16-key halves and the wave's two row tiles
-    f32x4 st[2][2];
+  // The loop is skewed by one step: body s turns the scores of step s (made in body s - 1) into
+  // weights and adds their value product, and between those vector instructions it issues the
+  // score products of step s + 1, so that the matrix unit works in the shadow of the softmax.
+  f32x4 st[2][2];                              // raw scores^T of the step the next body weighs
+#if CL_RAGGED
+  PL_WAITCNT(2 * PL_UNITS_PER);
+#else
+  PL_WAITCNT(2 * PL_UNITS_PER + 1);
+#endif
+  __syncthreads();
+  {
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) st[rt][0] = st[rt][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < PL_KJ; ++j)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const elem8 a = *reinterpret_cast<const elem8*>(kimg + (j >> 1) * PL_PANEL + 16 * h * 64 +
-                                                        (a_lo ^ ((4 * (j & 1)) << 3)));
+        const elem8 a = k_frag(PlC<0>{}, j, h);
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) st[rt][h] = mfma16(a, qf[rt][j], st[rt][h]);
       }
+  }
 
-    elem8 pf[2];
+  // Body of step `step`, whose images are in stage SLOT (compile-time: every LDS address is a
+  // register plus an immediate).
+  auto do_step = [&](auto slot_c, const int step) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    // the images of step + 1 have landed when at most the loads of step + 2 are outstanding; the
+    // barrier makes that everybody's share and frees the stage step - 1 has left, which the
+    // loads of step + 3 fill
+    PL_WAITCNT(PL_UNITS_PER);
+    __syncthreads();
+#if !CL_PF_DBG_NOLOADS
+#if CL_RAGGED
+    issue_step(row_of(step + 3), (SLOT + 3) % PL_STAGES);
+#else
+    // (the entry of step + 3 was asked for a body ago, before the loads the wait above left out)
+    const int row_ahead = fetched_row(step + 3);
+    fetch_id(step + 4);
+    issue_step(row_ahead, (SLOT + 3) % PL_STAGES);
+#endif
+#endif
+
+    // operands of this body's matrix work: K of step + 1, V of step (8 + 16 LDS reads)
+    elem8 kf[PL_KJ][2];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-      float s[8];
+    for (int j = 0; j < PL_KJ; ++j)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) kf[j][h] = k_frag(PlC<(SLOT + 1) % PL_STAGES>{}, j, h);
+    elem8 vf[PL_FB];
+#pragma unroll
+    for (int fb = 0; fb < PL_FB; ++fb) vf[fb] = v_frag(slot_c, fb);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- maxima of the step's scores; raise a row's reference when they pass it by 2^8 -------
+    float s[2][8];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[rt][i] = st[rt][i >> 2][i & 3];
+    if (step >= n_full) {
+      // slot i of the lane is key 32 step + 16 (i / 4) + 4 g + i % 4; a masked slot scores -inf,
+      // which a finite reference turns into a weight of exactly 0
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+        const int room = lim_rel[rt] - step * PL_STEP;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[rt][i] = 16 * (i >> 2) + (i & 3) <= room ? s[rt][i] : CL_NEG_INF;
+      }
+    }
+    // (first half of the score products of step + 1 in the shadow of the maxima)
+    f32x4 sn[2][2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) sn[rt][0] = sn[rt][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < PL_KJ / 2; ++j)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int t = t0 + 16 * h + 4 * g + q;
-          s[4 * h + q] = (t < ext && t <= limit[rt]) ? st[rt][h][q] * scale2 : CL_NEG_BIG;
-        }
-      float mx = s[0];
+        for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[j][h], qf[rt][j], sn[rt][h]);
+    float mx[2];
 #pragma unroll
-      for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-      mx = fmaxf(mx, lane_xor(mx, lane, 16));
-      mx = fmaxf(mx, lane_xor(mx, lane, 32));
-      const float m_new = fmaxf(m_run[rt], mx);
-      const float alpha = fast_exp2(m_run[rt] - m_new);
-      m_run[rt] = m_new;
-      float psum = 0.f, esum = 0.f;
+    for (int rt = 0; rt < 2; ++rt) {
+      float v = fmaxf(fmaxf(s[rt][0], s[rt][1]), s[rt][2]);
+      v = fmaxf(fmaxf(v, s[rt][3]), s[rt][4]);
+      v = fmaxf(fmaxf(v, s[rt][5]), s[rt][6]);
+      mx[rt] = pl_max_over_groups(fmaxf(v, s[rt][7])) * scale2;
+    }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        // masked slots hold CL_NEG_BIG; when the whole row is still masked m_new equals it too,
-        // so test the mask itself rather than trusting exp2 of a zero difference
-        const float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;
-        const elem_t pe = to_elem(p);
-        psum += to_f32(pe);
-        esum += p;
-        pf[rt][i] = pe;
-      }
-      l_run[rt] = l_run[rt] * alpha + psum;
-      l_exact[rt] = l_exact[rt] * alpha + esum;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // wave-uniform: skip when no max moved
+    for (int i = 0; i < 2 * PL_KJ; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    if (__builtin_amdgcn_ballot_w64(mx[0] > m_run[0] + 8.0f || mx[1] > m_run[1] + 8.0f)) {
+      // cold after the first steps of an item: weights stay below 2^8 against a reference that
+      // lags the running maximum by less than 8 (log2 domain)
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+        const float m_new = mx[rt] > m_run[rt] + 8.0f ? mx[rt] : m_run[rt];
+        const float alpha = fast_exp2(m_run[rt] - m_new);
+        m_run[rt] = m_new;
+        l_run[rt] *= alpha;
 #pragma unroll
         for (int fb = 0; fb < PL_FB; ++fb) acc[rt][fb] *= alpha;
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
 
-    // out^T block fb: rows = features 16 fb + (0..15), slots = keys 4 g + (0..3), 16 + 4 g + (0..3)
+    // ---- weights of the first row tile beside the rest of the score products -----------------
+    elem8 pf[2];
+    auto weigh = [&](int rt) __attribute__((always_inline)) {
+      float psum = 0.f;
 #pragma unroll
-    for (int fb = 0; fb < PL_FB; ++fb) {
-      const elem_t* p = vimg + (fb >> 2) * PL_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
-      const pl_s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p));
-      const pl_s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p + 16 * 64));
-      const elem8 a = __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+      for (int i = 0; i < 8; ++i) {
+        const float p = fast_exp2(__builtin_fmaf(s[rt][i], scale2, -m_run[rt]));
+        psum += p;
+        pf[rt][i] = to_elem(p);
+      }
+      l_run[rt] += psum;
+    };
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt) acc[rt][fb] = mfma16(a, pf[rt], acc[rt][fb]);
+    for (int j = PL_KJ / 2; j < PL_KJ; ++j)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[j][h], qf[rt][j], sn[rt][h]);
+    weigh(0);
+#pragma unroll
+    for (int i = 0; i < 2 * PL_KJ; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
     }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- weights of the second row tile beside the value product of the first ----------------
+#pragma unroll
+    for (int fb = 0; fb < PL_FB; ++fb) acc[0][fb] = mfma16(vf[fb], pf[0], acc[0][fb]);
+    weigh(1);
+#pragma unroll
+    for (int i = 0; i < PL_FB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- value product of the second row tile ------------------------------------------------
+#pragma unroll
+    for (int fb = 0; fb < PL_FB; ++fb) acc[1][fb] = mfma16(vf[fb], pf[1], acc[1][fb]);
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) st[rt][h] = sn[rt][h];
+  };
+
+  for (int step = 0;;) {
+    do_step(PlC<0>{}, step);
+    if (++step >= n_steps) break;
+    do_step(PlC<1>{}, step);
+    if (++step >= n_steps) break;
+    do_step(PlC<2>{}, step);
+    if (++step >= n_steps) break;
+    do_step(PlC<3>{}, step);
+    if (++step >= n_steps) break;
   }
   // no load may still be on its way into LDS when the workgroup ends
   PL_WAITCNT(0);
 
   // ---- each lane writes its rows' features (a row that saw no key: 0 and lse -inf) --------------
+  // (row coordinates are worked out again from the lane number, behind a barrier for the
+  // optimiser: kept across the loop they would cost registers the loop needs)
+  int lane_e = lane;
+  asm volatile("" : "+v"(lane_e));
+  const int c_e = lane_e & 15, g_e = lane_e >> 4;
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
-    float l = l_run[rt], le = l_exact[rt];
-    l += lane_xor(l, lane, 16);
-    l += lane_xor(l, lane, 32);
-    le += lane_xor(le, lane, 16);
-    le += lane_xor(le, lane, 32);
-    if (!live[rt]) continue;
+    float l = l_run[rt];
+    l += lane_xor(l, lane_e, 16);
+    l += lane_xor(l, lane_e, 32);
+    const int m = 32 * wave + 16 * rt + c_e;
+    if (m >= n_rows) continue;
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
-    const i64 orow = (i64)tok[rt] * CL_Q_HEADS + qhead[rt];
-    elem_t* dst = CL_ARG_OUT + orow * CL_HEAD_DIM + 4 * g;
+    const i64 orow = (i64)(lo + m / PL_GROUP) * CL_Q_HEADS + head * PL_GROUP + m % PL_GROUP;
+    elem_t* dst = CL_ARG_OUT + orow * CL_HEAD_DIM + 4 * g_e;
 #pragma unroll
     for (int fb = 0; fb < PL_FB; ++fb) {
       elem4 y;
@@ -302,7 +471,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       *reinterpret_cast<elem4*>(dst + 16 * fb) = y;
     }
 #if CL_EMIT_LSE
-    if (g == 0) CL_ARG_LSE[orow] = le > 0.f ? m_run[rt] + fast_log2(le) : CL_NEG_INF;
+    if (g_e == 0) CL_ARG_LSE[orow] = l > 0.f ? m_run[rt] + fast_log2(l) : CL_NEG_INF;
 #endif
   }
 }

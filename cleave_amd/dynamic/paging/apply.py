@@ -214,10 +214,11 @@ def chunk_pages_expr(spec, chunk_pages: int) -> str:
 # Parameter order of the reference's operators (``python/cleave/dynamic/reference.py:204-278``):
 # q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, sm_scale (token table) or
 # q, k, v, qo_indptr, kv_indptr, sm_scale (packed keys); then out (total_q, heads, d), lse.
-def _prefill_plan(spec: PagingSpec, dense: DenseAttention, shared: bool | None = None) -> KernelPlan:
+def _prefill_plan(spec: PagingSpec, dense: DenseAttention, shared: bool | None = None, knobs=None) -> KernelPlan:
     """``shared``: the kernel whose four waves share every key tile through LDS (128 query rows per
     workgroup, for long requests) instead of the one-wave-per-kv-head kernel with 16-row items;
-    None: follow the dense tiling (four or more waves ask for the shared form)."""
+    None: follow the dense tiling (four or more waves ask for the shared form).  ``knobs``: further
+    tiling entries of the shared kernel (each becomes a ``CL_PF_<name>`` definition)."""
     d, dt = dense.head_dim, dense.dtype
     if shared is None:
         shared = dense.waves >= 4 and d % 64 == 0
@@ -253,7 +254,7 @@ def _prefill_plan(spec: PagingSpec, dense: DenseAttention, shared: bool | None =
     threads, rows = (256, 128) if shared else (spec.num_kv_heads * 64, 16)
     return KernelPlan(template="attn_prefill", role="main", family="attention", dtype=dense.dtype,
                       extra={"derived_dims": [("batch", f"{spec.indptr_dim} - 1")]}, problem=problem,
-                      tiling={"SHARED": int(bool(shared))}, params=params + outs, operands=operands, split_factor=None,
+                      tiling={"SHARED": int(bool(shared)), **(dict(knobs or {}) if shared else {})}, params=params + outs, operands=operands, split_factor=None,
                       dyn_dims=tuple(dim_names.values()), n_threads=threads, label=f"kv={KV_STEP} q={rows} thr={threads}")
 
 
