@@ -82,6 +82,10 @@ template <int I> struct PlC { static constexpr int value = I; };
 
 // max of x over the four lanes that share lane % 16 (the key groups of one query row): the two
 // row-swap instructions exchange 16-lane rows 1<->0', 3<->2' and then 2,3<->0',1' of a register pair
+// rows (16 lanes) 1 and 3 of `a` trade places with rows 0 and 2 of `b`
+CL_DEVICE void pl_swap_rows16(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+}
 CL_DEVICE float pl_max_over_groups(float x) {
   float a = x, b = x;
   asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0\n\tv_max_f32 %0, %0, %1\n\tv_mov_b32 %1, %0\n\t"
@@ -115,23 +119,38 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     item = lin % gx;
     head = lin / gx;
   }
-  // the request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item
-  int req = 0;
+  // The request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item.
+  // The condition holds for every request up to that one, so the lanes test 64 requests at a time
+  // and count (one round trip to memory per 64 requests instead of one per halving); with up to
+  // 63 requests the row pointers the item needs are already in the lanes.
+  int req, q0, q1, kv0, kv1;
   {
-    int hi_b = batch - 1;
-    while (req < hi_b) {
-      const int mid = (req + hi_b + 1) >> 1;
-      if (mid + pl_clamp(CL_ARG_QINDPTR[mid], 0, total_q) / PL_QT <= item) req = mid;
-      else hi_b = mid - 1;
+    const int b0 = lane < batch ? lane : batch;
+    const int qp0 = pl_clamp(CL_ARG_QINDPTR[b0], 0, total_q), kp0 = pl_clamp(CL_ARG_INDPTR[b0], 0, n_idx);
+    int count = __builtin_popcountll(__builtin_amdgcn_ballot_w64(lane < batch && lane + qp0 / PL_QT <= item));
+    for (int base = 64; base < batch; base += 64) {
+      const int b = base + lane < batch ? base + lane : batch;
+      const int qp = pl_clamp(CL_ARG_QINDPTR[b], 0, total_q);
+      count += __builtin_popcountll(__builtin_amdgcn_ballot_w64(base + lane < batch && b + qp / PL_QT <= item));
+    }
+    req = count > 0 ? count - 1 : 0;
+    if (batch < 64) {
+      q0 = __builtin_amdgcn_readlane(qp0, req);
+      q1 = __builtin_amdgcn_readlane(qp0, req + 1);
+      kv0 = __builtin_amdgcn_readlane(kp0, req);
+      kv1 = __builtin_amdgcn_readlane(kp0, req + 1);
+    } else {
+      q0 = pl_clamp(CL_ARG_QINDPTR[req], 0, total_q);
+      q1 = pl_clamp(CL_ARG_QINDPTR[req + 1], 0, total_q);
+      kv0 = pl_clamp(CL_ARG_INDPTR[req], 0, n_idx);
+      kv1 = pl_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx);
     }
   }
-  const int q0 = pl_clamp(CL_ARG_QINDPTR[req], 0, total_q), q1 = pl_clamp(CL_ARG_QINDPTR[req + 1], 0, total_q);
   const int chunk = item - req;
   const int lo = q0 > chunk * PL_QT ? q0 : chunk * PL_QT;
   const int hi = q1 < (chunk + 1) * PL_QT ? q1 : (chunk + 1) * PL_QT;
   if (hi <= lo) return;                                 // an index no (chunk, request) pair maps to
-  const int kv0 = pl_clamp(CL_ARG_INDPTR[req], 0, n_idx);
-  int kv_len = pl_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx) - kv0;
+  int kv_len = kv1 - kv0;
   kv_len = kv_len > 0 ? kv_len : 0;
   const int off = kv_len - (q1 - q0);                   // key position of the request's first query row
   const int n_rows = (hi - lo) * PL_GROUP;
@@ -156,12 +175,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
       if (!live[rt]) continue;
-      elem_t* dst = CL_ARG_OUT + ((i64)tok[rt] * CL_Q_HEADS + qhead[rt]) * CL_HEAD_DIM + 4 * g;
-      elem4 z;
+      elem_t* dst = CL_ARG_OUT + ((i64)tok[rt] * CL_Q_HEADS + qhead[rt]) * CL_HEAD_DIM + 16 * (g & 1) + 4 * (g & 2);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) z[i] = to_elem(0.f);
-#pragma unroll
-      for (int fb = 0; fb < PL_FB; ++fb) *reinterpret_cast<elem4*>(dst + 16 * fb) = z;
+      for (int fp = 0; fp < PL_FB / 2; ++fp) *reinterpret_cast<u32x4*>(dst + 32 * fp) = (u32x4){0u, 0u, 0u, 0u};
 #if CL_EMIT_LSE
       if (g == 0) CL_ARG_LSE[(i64)tok[rt] * CL_Q_HEADS + qhead[rt]] = CL_NEG_INF;
 #endif
@@ -175,7 +191,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const i64 row_bytes = (i64)CL_KV_HEADS * CL_HEAD_DIM * 2;
   const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_HEAD_DIM * 2;
   const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_HEAD_DIM * 2;
+#if CL_PF_DBG_ONESTEP
+  const int n_steps = 1;
+#else
   const int n_steps = (ext + PL_STEP - 1) / PL_STEP;
+#endif
   const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)pl_tiles;
 
   // This wave's share of step s (clamped onto the last step: a step past the end reloads the last
@@ -208,11 +228,26 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     return pl_clamp(pl_ids[s & 1][wave][lane], 0, num_pages - 1);
   };
 #endif
-  auto issue_step = [&](int row, int slot) __attribute__((always_inline)) {
+  // load `part` of a step (its K panels, then its V panels) into stage `slot`
+  auto issue_part = [&](int row, int slot, auto part_c) __attribute__((always_inline)) {
+    constexpr int PART = decltype(part_c)::value, P = PART % PL_PANELS;
     const int chunk = (lane & 7) ^ pl_swz(my_r);
-    const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024);
-    pl_issue_panels<0>(kbase + (i64)row * row_bytes + 16 * chunk, group_byte);
-    pl_issue_panels<0>(vbase + (i64)row * row_bytes + 16 * chunk, group_byte + PL_IMG * 2);
+    const char* src = (PART < PL_PANELS ? kbase : vbase) + (i64)row * row_bytes + 16 * chunk;
+    const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024) + (PART < PL_PANELS ? 0 : PL_IMG * 2);
+    pl_dma16<128 * P>(src, group_byte + (unsigned)(P * PL_PANEL * 2) - 128 * P);
+  };
+  // the quarter `place` (0..3) of a step's loads: the body spreads them between its matrix work,
+  // because a wave stands still while a load waits for the path into the CU
+  auto issue_quarter = [&](int row, int slot, auto place_c) __attribute__((always_inline)) {
+    constexpr int PLACE = decltype(place_c)::value, LO = PLACE * PL_UNITS_PER / 4, HI = (PLACE + 1) * PL_UNITS_PER / 4;
+    if constexpr (HI > LO) issue_part(row, slot, PlC<LO>{});
+    if constexpr (HI > LO + 1) issue_part(row, slot, PlC<LO + 1>{});
+  };
+  auto issue_step = [&](int row, int slot) __attribute__((always_inline)) {
+    issue_quarter(row, slot, PlC<0>{});
+    issue_quarter(row, slot, PlC<1>{});
+    issue_quarter(row, slot, PlC<2>{});
+    issue_quarter(row, slot, PlC<3>{});
   };
 #define PL_WAITCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 
@@ -233,7 +268,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     const elem_t* row = CL_ARG_Q + ((i64)tok[rt] * CL_Q_HEADS + qhead[rt]) * CL_HEAD_DIM + 8 * g;
 #pragma unroll
     for (int j = 0; j < PL_KJ; ++j) {
+#if CL_PF_DBG_NOQ
+      u32x4 raw = (u32x4){(unsigned)lane, 0x3c003c00u, (unsigned)j, 0x3c003c00u};
+#else
       u32x4 raw = ld16(row + 32 * j);
+#endif
       if (!live[rt]) raw = (u32x4){0u, 0u, 0u, 0u};
       qf[rt][j] = as_elem8(raw ^ q_sign);
     }
@@ -312,16 +351,19 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // loads of step + 3 fill
     PL_WAITCNT(PL_UNITS_PER);
     __syncthreads();
-#if !CL_PF_DBG_NOLOADS
 #if CL_RAGGED
-    issue_step(row_of(step + 3), (SLOT + 3) % PL_STAGES);
+    const int row_ahead = row_of(step + 3);
 #else
     // (the entry of step + 3 was asked for a body ago, before the loads the wait above left out)
     const int row_ahead = fetched_row(step + 3);
     fetch_id(step + 4);
-    issue_step(row_ahead, (SLOT + 3) % PL_STAGES);
 #endif
+#if CL_PF_DBG_NOLOADS
+#define PL_ISSUE(place)
+#else
+#define PL_ISSUE(place) issue_quarter(row_ahead, (SLOT + 3) % PL_STAGES, PlC<place>{})
 #endif
+    PL_ISSUE(0);
 
     // operands of this body's matrix work: K of step + 1, V of step (8 + 16 LDS reads)
     elem8 kf[PL_KJ][2];
@@ -387,6 +429,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    PL_ISSUE(1);
 
     // ---- weights of the first row tile beside the rest of the score products -----------------
     elem8 pf[2];
@@ -413,6 +456,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
+    PL_ISSUE(2);
 
     // ---- weights of the second row tile beside the value product of the first ----------------
 #pragma unroll
@@ -424,6 +468,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
+    PL_ISSUE(3);
 
     // ---- value product of the second row tile ------------------------------------------------
 #pragma unroll
@@ -460,15 +505,29 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     l += lane_xor(l, lane_e, 32);
     const int m = 32 * wave + 16 * rt + c_e;
     if (m >= n_rows) continue;
+#if CL_PF_DBG_NOSTORE
+    if (l != 12345.f) continue;
+#endif
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
     const i64 orow = (i64)(lo + m / PL_GROUP) * CL_Q_HEADS + head * PL_GROUP + m % PL_GROUP;
-    elem_t* dst = CL_ARG_OUT + orow * CL_HEAD_DIM + 4 * g_e;
+    // A lane holds features 16 fb + 4 g .. + 3 of its row for every block fb.  Lanes g and g ^ 1
+    // trade halves of a pair of blocks (one row swap per register), so that each stores 16
+    // contiguous bytes: even g the 8 features from 4 g of the even block, odd g those from
+    // 4 (g - 1) of the odd one.
+    elem_t* dst = CL_ARG_OUT + orow * CL_HEAD_DIM + 16 * (g_e & 1) + 4 * (g_e & 2);
 #pragma unroll
-    for (int fb = 0; fb < PL_FB; ++fb) {
-      elem4 y;
+    for (int fp = 0; fp < PL_FB / 2; ++fp) {
+      elem4 y0, y1;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[rt][fb][r] * inv);
-      *reinterpret_cast<elem4*>(dst + 16 * fb) = y;
+      for (int r = 0; r < 4; ++r) {
+        y0[r] = to_elem(acc[rt][2 * fp][r] * inv);
+        y1[r] = to_elem(acc[rt][2 * fp + 1][r] * inv);
+      }
+      const u32x2 a = __builtin_bit_cast(u32x2, y0), b = __builtin_bit_cast(u32x2, y1);
+      unsigned a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1];
+      pl_swap_rows16(a0, b0);
+      pl_swap_rows16(a1, b1);
+      *reinterpret_cast<u32x4*>(dst + 32 * fp) = (u32x4){a0, a1, b0, b1};
     }
 #if CL_EMIT_LSE
     if (g_e == 0) CL_ARG_LSE[orow] = l > 0.f ? m_run[rt] + fast_log2(l) : CL_NEG_INF;
