@@ -162,7 +162,9 @@ def test_paged_mla_layer_plans_and_signature():
     assert [p["name"] for p in gqa["params"]] == ["PlaceHolder_Q", "PlaceHolder_K", "PlaceHolder_V", "PlaceHolder_QO_INDPTR",
                                                  "PlaceHolder_KV_INDPTR", "sm_scale", "OutputNode_0", "OutputNode_1"]
     # the operator's own kernel is the one whose four waves share key tiles through LDS (128 rows = 32 tokens x 4)
-    assert gqa["launches"][0]["grid"][:2] == ["ceildiv(total_q, 32) + batch", "8"] and gqa["launches"][0]["block"][0] == 256
+    # (the item axis is padded to a multiple of 8: one contiguous eighth of the space per XCD)
+    assert gqa["launches"][0]["grid"][:2] == ["ceildiv(ceildiv(total_q, 32) + batch, 8) * 8", "8"]
+    assert gqa["launches"][0]["block"][0] == 256
     from cleave_amd.dynamic.paging import RAGGED_PREFILL_CAUSAL, PagingSpec
     from cleave_amd.dynamic.paging.apply import _prefill_plan
 
