@@ -129,17 +129,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   u.rows = CL_ROWS - 16 * tile_id < 16 ? CL_ROWS - 16 * tile_id : 16;
 #if CL_CHUNK_PAGES
   // the request whose items include `item`: the last b with b + indptr[b] / C <= item
-  int req = 0;
-  {
-    int hi_b = batch - 1;
-    while (req < hi_b) {
-      const int mid = (req + hi_b + 1) >> 1;
-      if (mid + att_clamp_ptr(CL_ARG_INDPTR[mid], n_idx) / chunk_pages <= item) req = mid;
-      else hi_b = mid - 1;
-    }
-  }
+  const ClRequest found = cl_find_request(CL_ARG_INDPTR, batch, n_idx, chunk_pages, 1, item, lane);
+  const int req = found.req, p0 = found.p0, p1 = found.p1;
   const int head = wave;
-  const int p0 = att_clamp_ptr(CL_ARG_INDPTR[req], n_idx), p1 = att_clamp_ptr(CL_ARG_INDPTR[req + 1], n_idx);
   const int chunk = item - req;
   const int lo = p0 > chunk * chunk_pages ? p0 : chunk * chunk_pages;
   const int hi = p1 < (chunk + 1) * chunk_pages ? p1 : (chunk + 1) * chunk_pages;

@@ -43,16 +43,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int c = lane & 15, g = lane >> 4;
   const int item = blockIdx.x;
   // the request whose items include `item`: the last b with b + qo_indptr[b] / PF_TOK <= item
-  int req = 0;
-  {
-    int hi_b = batch - 1;
-    while (req < hi_b) {
-      const int mid = (req + hi_b + 1) >> 1;
-      if (mid + pf_clamp(CL_ARG_QINDPTR[mid], 0, total_q) / PF_TOK <= item) req = mid;
-      else hi_b = mid - 1;
-    }
-  }
-  const int q0 = pf_clamp(CL_ARG_QINDPTR[req], 0, total_q), q1 = pf_clamp(CL_ARG_QINDPTR[req + 1], 0, total_q);
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, PF_TOK, 1, item, lane);
+  const int req = found.req, q0 = found.p0, q1 = found.p1;
   const int chunk = item - req;
   const int lo = q0 > chunk * PF_TOK ? q0 : chunk * PF_TOK;
   const int hi = q1 < (chunk + 1) * PF_TOK ? q1 : (chunk + 1) * PF_TOK;

@@ -44,6 +44,43 @@ CL_DEVICE float lane_read(float v, int src_lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v)));
 }
 
+// Search of a row-pointer array (batch + 1 non-decreasing entries, clamped into [0, limit]) by
+// all lanes of a wave at once: the last request b of [0, batch) with
+//   with_b * b + ptr[b] / div <= item
+// (true for every request up to that one, so the lanes test 64 requests at a time and count:
+// one round trip to memory per 256 requests where a bisection makes one per halving), and the
+// clamped ptr[b], ptr[b + 1] -- out of the lanes when there are fewer than 64 requests.
+struct ClRequest { int req, p0, p1; };
+CL_DEVICE int cl_clamp_ptr(int p, int limit) { return p < 0 ? 0 : (p > limit ? limit : p); }
+CL_DEVICE ClRequest cl_find_request(const int* __restrict__ ptr, int batch, int limit, int div, int with_b,
+                                    int item, int lane) {
+  const int v0 = cl_clamp_ptr(ptr[lane < batch ? lane : batch], limit);
+  int count = __builtin_popcountll(__builtin_amdgcn_ballot_w64(lane < batch && with_b * lane + v0 / div <= item));
+  for (int base = 64; base < batch; base += 256) {
+    int v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int b = base + 64 * k + lane;
+      v[k] = cl_clamp_ptr(ptr[b < batch ? b : batch], limit);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int b = base + 64 * k + lane;
+      count += __builtin_popcountll(__builtin_amdgcn_ballot_w64(b < batch && with_b * b + v[k] / div <= item));
+    }
+  }
+  ClRequest r;
+  r.req = count > 0 ? count - 1 : 0;
+  if (batch < 64) {
+    r.p0 = __builtin_amdgcn_readlane(v0, r.req);
+    r.p1 = __builtin_amdgcn_readlane(v0, r.req + 1);
+  } else {
+    r.p0 = cl_clamp_ptr(ptr[r.req], limit);
+    r.p1 = cl_clamp_ptr(ptr[r.req + 1], limit);
+  }
+  return r;
+}
+
 // 16-byte global load / store of eight elements.
 CL_DEVICE u32x4 ld16(const elem_t* p) { return *reinterpret_cast<const u32x4*>(p); }
 CL_DEVICE void st16(elem_t* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }

@@ -77,16 +77,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #if CL_CHUNKED
   const int item = blockIdx.x;
   // the request whose items include `item`: the last b with b + indptr[b] / C <= item
-  int req = 0;
-  {
-    int hi_b = batch - 1;
-    while (req < hi_b) {
-      const int mid = (req + hi_b + 1) >> 1;
-      if (mid + mp_clamp(CL_ARG_INDPTR[mid], 0, n_idx) / chunk_pages <= item) req = mid;
-      else hi_b = mid - 1;
-    }
-  }
-  const int p0 = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx), p1 = mp_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx);
+  const ClRequest found = cl_find_request(CL_ARG_INDPTR, batch, n_idx, chunk_pages, 1, item, lane);
+  const int req = found.req, p0 = found.p0, p1 = found.p1;
   const int chunk = item - req;
   const int lo = p0 > chunk * chunk_pages ? p0 : chunk * chunk_pages;
   const int hi = p1 < (chunk + 1) * chunk_pages ? p1 : (chunk + 1) * chunk_pages;
@@ -95,16 +87,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // causal prefill: an item is one query token (its 16 heads are the tile); it sees the keys
   // kv_pos <= kv_len - q_len + q_pos of its request
   const int qtok = blockIdx.x;
-  int req = 0;
-  {
-    int hi_b = batch - 1;                               // the last b with qo_indptr[b] <= qtok
-    while (req < hi_b) {
-      const int mid = (req + hi_b + 1) >> 1;
-      if (mp_clamp(CL_ARG_QINDPTR[mid], 0, total_q) <= qtok) req = mid;
-      else hi_b = mid - 1;
-    }
-  }
-  const int q0 = mp_clamp(CL_ARG_QINDPTR[req], 0, total_q), q1 = mp_clamp(CL_ARG_QINDPTR[req + 1], 0, total_q);
+  // its request: the last b with qo_indptr[b] <= qtok
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, 1, 0, qtok, lane);
+  const int req = found.req, q0 = found.p0, q1 = found.p1;
   const int lo = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx);
   int hi;
   {
