@@ -196,7 +196,7 @@ class HipCodeGen:
                 unit.define("CL_ARG_PACC", op["PACC"])
                 if norm:
                     unit.define("CL_ARG_PSS", op["PSS"])
-            for role, macro in (("A", "CL_ARG_A"), ("B", "CL_ARG_B"), ("GAMMA", "CL_ARG_GAMMA")):
+            for role, macro in (("A", "CL_ARG_A"), ("B", "CL_ARG_B"), ("C", "CL_ARG_C"), ("GAMMA", "CL_ARG_GAMMA")):
                 if role in op:
                     unit.define(macro, op[role])
             unit.define("CL_ARG_X", op["A"])
@@ -247,7 +247,7 @@ class HipCodeGen:
 
     def _emit_gemm_dma(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
-        if plan.family != "matmul":
+        if plan.family not in ("matmul", "swiglu"):
             raise CodegenError("the direct-to-LDS matmul template has no fused RMSNorm form")
         self._matmul_common(unit, plan, params, partial, combine, fused)
         tile = dict(BM=128, BN=128, BK=64, WM=2, WN=2)
@@ -255,6 +255,13 @@ class HipCodeGen:
         for k, v in tile.items():
             unit.define(f"CL_{k}", v)
         splits = plan.split_factor or 1
+        swiglu = plan.family == "swiglu"
+        if swiglu != bool(tile.get("SWIGLU")) or (swiglu and (splits > 1 or combine)):
+            raise CodegenError("SwiGLU is the SWIGLU tiling of the direct-to-LDS matmul, unsplit")
+        # (SwiGLU: the B tile holds BN / 2 columns of each weight, so a tile covers BN / 2 columns of the output)
+        out_bn = tile["BN"] // 2 if swiglu else tile["BN"]
+        if swiglu and (tile["BN"] // tile["WN"] // 16) % 2:
+            raise CodegenError("a SwiGLU wave owns an even number of column fragments")
         batch = max(p["batch_A"], p["batch_B"])
         unit.templates.append("gemm_dma.hip")
         if partial:
@@ -262,7 +269,7 @@ class HipCodeGen:
                 raise CodegenError(f"K={p['K']} is not a multiple of splits*64={splits * 64}")
             if (not p["trans_B"] and p["N"] % 8) or (p["trans_A"] and p["M"] % 8) or p["K"] % 8:
                 raise CodegenError("16-byte global chunks need the minor extent of each operand to be a multiple of 8")
-            grid = (-(-p["N"] // tile["BN"]), -(-p["M"] // tile["BM"]), batch * splits)
+            grid = (-(-p["N"] // out_bn), -(-p["M"] // tile["BM"]), batch * splits)
             # the tile images are static LDS arrays of the kernel: no dynamic LDS at launch
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, 0, self._partial_args)
         if combine:

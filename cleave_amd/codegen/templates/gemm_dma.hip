@@ -17,6 +17,11 @@
 //
 //   CL_M CL_N CL_K  CL_BM CL_BN  CL_WM x CL_WN waves  CL_TRANS_A / CL_TRANS_B  CL_BATCH_A/B
 //   CL_SPLITS (split-K: f32 partial tiles to CL_ARG_PACC[split])  CL_GROUP_M (tile order patch)
+//
+// CL_SWIGLU: C = (A * B) .* silu(A * G) with a second weight G (CL_ARG_C) laid out like B.  The
+// B tile is made of two halves, columns n0 .. n0 + BN/2 of B and the same columns of G, so a
+// workgroup covers BN/2 columns of C; every wave owns the same columns in both halves (half of its
+// column fragments each) and multiplies the two accumulators in its epilogue.
 
 #define GD_WAVES (CL_WM * CL_WN)
 #define GD_THREADS (GD_WAVES * 64)
@@ -34,6 +39,10 @@
 #ifndef CL_ASM_LOADS
 #define CL_ASM_LOADS 0
 #endif
+#ifndef CL_SWIGLU
+#define CL_SWIGLU 0
+#endif
+#define GD_OUT_BN (CL_SWIGLU ? CL_BN / 2 : CL_BN)   // columns of C a tile covers
 static_assert(CL_BK == 64, "K steps are 64 wide (128-byte K-minor rows)");
 static_assert((GD_TM & (GD_TM - 1)) == 0 && (GD_TN & (GD_TN - 1)) == 0, "wave tiles are powers of two");
 static_assert(CL_BM % 16 == 0 && CL_BN % 16 == 0, "tiles are multiples of 16");
@@ -68,15 +77,22 @@ CL_DEVICE int gd_swz_kmaj(int k) {
 // One operand of the product: how its tile is fetched and how fragments are read.
 //   EXT      tile extent along the operand's own axis (BM for A, BN for B)
 //   KMAJOR   stored with K as the major axis
-template <int EXT, bool KMAJOR>
+template <bool WIDE> struct GdOffset { typedef u32 type; };
+template <> struct GdOffset<true> { typedef i64 type; };
+//   DUAL     the tile's second half (rows / columns EXT/2 ..) comes from a second tensor of the
+//            same layout, `twin` bytes after the first (the same rows / columns of it)
+template <int EXT, bool KMAJOR, bool DUAL = false>
 struct GdOperand {
   static constexpr int CPR = EXT / 8;                          // K-major: chunks per k row
   static constexpr int UNITS = EXT * GD_BK * 2 / 1024;         // 1 KiB wave loads per tile
   static constexpr int PER = (UNITS + GD_WAVES - 1) / GD_WAVES;
-  u32 goff[PER];     // this lane's byte offset (from the tile's first element at k = 0) per unit
+  static constexpr int SPAN = DUAL ? EXT / 2 : EXT;            // tensor rows / columns under the tile
+  // this lane's byte offset (from the tile's first element at k = 0) per unit
+  typedef typename GdOffset<DUAL>::type off_t;
+  off_t goff[PER];
 
   // ext0: first row/column of the tile, lim: tensor extent along that axis, pitch: elements
-  CL_METHOD void init(int ext0, int lim, int pitch) {
+  CL_METHOD void init(int ext0, int lim, int pitch, i64 twin = 0) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -84,16 +100,16 @@ struct GdOperand {
       if (!KMAJOR) {
         const int r = 8 * u + (lane >> 3);
         const int chunk = (lane & 7) ^ gd_swz_kmin(r);
-        int row = ext0 + r;
+        int row = ext0 + r % SPAN;
         row = row < lim ? row : lim - 1;                        // rows past the edge repeat the last one
-        goff[i] = (u32)(((row - ext0) * pitch + 8 * chunk) * 2);
+        goff[i] = (off_t)(((row - ext0) * pitch + 8 * chunk) * 2) + (r >= SPAN ? twin : 0);
       } else {
         constexpr int RPU = 64 / CPR > 0 ? 64 / CPR : 1;        // k rows per unit
         const int k = u * RPU + lane / CPR;
         const int chunk = (lane % CPR) ^ gd_swz_kmaj<EXT>(k);
-        int col = ext0 + 8 * chunk;
+        int col = ext0 + (8 * chunk) % SPAN;
         col = col < lim - 8 ? col : lim - 8;                    // chunks past the edge repeat the last one
-        goff[i] = (u32)((k * pitch + (col - ext0)) * 2);
+        goff[i] = (off_t)((k * pitch + (col - ext0)) * 2) + (8 * chunk >= SPAN ? twin : 0);
       }
     }
   }
@@ -174,7 +190,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // Workgroups are handed to the XCDs round-robin in launch order.  Renumber them so that the
   // ones an XCD runs at the same time are neighbours in C: launch id L -> the (L / 8)-th tile of
   // XCD (L % 8)'s contiguous share, tiles ordered in patches of CL_GROUP_M row-tiles.
-  constexpr int tiles_m = (CL_M + CL_BM - 1) / CL_BM, tiles_n = (CL_N + CL_BN - 1) / CL_BN;
+  constexpr int tiles_m = (CL_M + CL_BM - 1) / CL_BM, tiles_n = (CL_N + GD_OUT_BN - 1) / GD_OUT_BN;
   constexpr int tiles = tiles_m * tiles_n;
   int tile_id = blockIdx.y * tiles_n + blockIdx.x;
   {
@@ -186,7 +202,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int band = tile_id / (group_m * tiles_n);
   const int band_rows = (tiles_m - band * group_m) < group_m ? (tiles_m - band * group_m) : group_m;
   const int in_band = tile_id - band * group_m * tiles_n;
-  const int m0 = (band * group_m + in_band % band_rows) * CL_BM, n0 = (in_band / band_rows) * CL_BN;
+  const int m0 = (band * group_m + in_band % band_rows) * CL_BM, n0 = (in_band / band_rows) * GD_OUT_BN;
   const int batch = blockIdx.z / CL_SPLITS, split = blockIdx.z % CL_SPLITS;
   constexpr int k_per_split = CL_K / CL_SPLITS;
   const int k_begin = split * k_per_split;
@@ -197,7 +213,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 
   // ---- operand movers: tile origin at K step 0 and the uniform advance per step ---------------
   GdOperand<CL_BM, CL_TRANS_A != 0> opa;
-  GdOperand<CL_BN, CL_TRANS_B == 0> opb;
+  GdOperand<CL_BN, CL_TRANS_B == 0, CL_SWIGLU != 0> opb;
+#if CL_SWIGLU
+  const i64 b_twin = reinterpret_cast<const char*>(CL_ARG_C) - reinterpret_cast<const char*>(CL_ARG_B);
+#else
+  const i64 b_twin = 0;
+#endif
 #if CL_TRANS_A
   opa.init(m0, CL_M, CL_M);                                   // A stored (K, M)
   const elem_t* a_base = A + (i64)k_begin * CL_M + m0;
@@ -208,17 +229,26 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   constexpr i64 a_step = GD_BK;
 #endif
 #if CL_TRANS_B
-  opb.init(n0, CL_N, CL_K);                                   // B stored (N, K)
+  opb.init(n0, CL_N, CL_K, b_twin);                           // B stored (N, K)
   const elem_t* b_base = B + (i64)n0 * CL_K + k_begin;
   constexpr i64 b_step = GD_BK;
 #else
-  opb.init(n0, CL_N, CL_N);                                   // B stored (K, N)
+  opb.init(n0, CL_N, CL_N, b_twin);                           // B stored (K, N)
   const elem_t* b_base = B + (i64)k_begin * CL_N + n0;
   constexpr i64 b_step = (i64)GD_BK * CL_N;
 #endif
 
   // ---- this lane's fragment offsets -------------------------------------------------------------
-  const int am = wm * (CL_BM / CL_WM), bn = wn * (CL_BN / CL_WN);   // wave origin inside the tile
+  // wave origin inside the tile (SwiGLU: inside each half of the B tile; fragments j < TN/2 come
+  // from the first half, the others from the same columns of the second)
+  const int am = wm * (CL_BM / CL_WM), bn = wn * (GD_OUT_BN / CL_WN);
+#if CL_SWIGLU
+#define GD_BSEL(j, x, y) ((j) < GD_TN / 2 ? (x) : (y))
+#define GD_BJ(j) ((j) % (GD_TN / 2))
+#else
+#define GD_BSEL(j, x, y) (x)
+#define GD_BJ(j) (j)
+#endif
 #if CL_TRANS_A
   const int a_f = gd_swz_kmaj<CL_BM>(8 * g + (c >> 2));
   const int a_off = (8 * g + (c >> 2)) * CL_BM + 8 * (((am / 8) ^ a_f) + ((c & 3) >> 1)) + 4 * (c & 1);
@@ -229,11 +259,13 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
 #if CL_TRANS_B
   const int b_off = (bn + c) * 64 + ((g ^ gd_swz_kmin(bn + c)) << 3);
-#define GD_BFRAG(tile, j, s) gd_read_kmin(tile, b_off, j, s)
+  const int b_off2 = b_off + (CL_BN / 2) * 64;                  // (BN/2 is a multiple of 8: same swizzle)
+#define GD_BFRAG(tile, j, s) gd_read_kmin(tile, GD_BSEL(j, b_off, b_off2), GD_BJ(j), s)
 #else
   const int b_f = gd_swz_kmaj<CL_BN>(8 * g + (c >> 2));
   const int b_off = (8 * g + (c >> 2)) * CL_BN + 8 * (((bn / 8) ^ b_f) + ((c & 3) >> 1)) + 4 * (c & 1);
-#define GD_BFRAG(tile, j, s) gd_read_kmaj<CL_BN>(tile, b_off, j, s)
+  const int b_off2 = (8 * g + (c >> 2)) * CL_BN + 8 * ((((CL_BN / 2 + bn) / 8) ^ b_f) + ((c & 3) >> 1)) + 4 * (c & 1);
+#define GD_BFRAG(tile, j, s) gd_read_kmaj<CL_BN>(tile, GD_BSEL(j, b_off, b_off2), GD_BJ(j), s)
 #endif
 
   f32x4 acc[GD_TM][GD_TN];
@@ -346,6 +378,20 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   for (int i = 0; i < GD_TM; ++i) {
     const int m = m0 + am + 16 * i + c;
     if (m >= CL_M) continue;
+#if CL_SWIGLU
+#pragma unroll
+    for (int j = 0; j < GD_TN / 2; ++j) {
+      const int n = n0 + bn + 16 * j + 4 * g;
+      if (n >= CL_N) continue;
+      elem4 y;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float gate = acc[i][j + GD_TN / 2][r];
+        y[r] = to_elem(acc[i][j][r] * gate / (1.0f + __expf(-gate)));
+      }
+      *reinterpret_cast<elem4*>(CL_ARG_OUT + (i64)m * CL_N + n) = y;
+    }
+#else
 #pragma unroll
     for (int j = 0; j < GD_TN; ++j) {
       const int n = n0 + bn + 16 * j + 4 * g;
@@ -359,6 +405,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       *reinterpret_cast<elem4*>(CL_ARG_OUT + ((i64)batch * CL_M + m) * CL_N + n) = y;
 #endif
     }
+#endif  // CL_SWIGLU
   }
 }
 #endif  // CL_EMIT_PARTIAL

@@ -31,7 +31,7 @@ from .graph import ComputeOpNode, Graph, Node, OutputNode, PlaceHolderNode
 class Lowered:
     """A recognised operator: family, sizes and which placeholder plays which operand."""
 
-    family: str                       # matmul | rmsnorm_matmul | attention | mla
+    family: str                       # matmul | rmsnorm_matmul | swiglu | attention | mla
     problem: dict                     # sizes and flags the template needs
     operands: dict                    # role -> PlaceHolderNode
     outputs: list                     # OutputNodes in order
@@ -198,6 +198,34 @@ def _try_matmul(view, out):
     return "matmul", prob, {"A": a, "B": b}
 
 
+def _try_swiglu(view, out):
+    """``(x @ w_up) * silu(x @ w_gate)`` with both products over the same activation: operands
+    A (activation), B (the bare product's weight), C (the weight under the silu), the roles of
+    the reference's graph (``tests/_graphs.py:403-436``)."""
+    n = view.skip(out)
+    if not (_is(n, "mul") and n.scalar is None and len(n.inputs) == 2):
+        return None
+    for up, gate in (view.ins(n), view.ins(n)[::-1]):
+        if not (_is(up, "matmul") and _is(gate, "silu")):
+            continue
+        gmm = view.ins(gate)[0]
+        if not _is(gmm, "matmul"):
+            continue
+        (a, b), (a2, c) = view.ins(up), view.ins(gmm)
+        if a is not a2 or not all(isinstance(t, PlaceHolderNode) for t in (a, b, c)):
+            continue
+        if view.is_split:
+            raise LoweringRejected("SwiGLU has no split-K form: the gate is not linear in its partial sums")
+        if (up.attrs["trans_A"], up.attrs["trans_B"]) != (gmm.attrs["trans_A"], gmm.attrs["trans_B"]) \
+                or tuple(b.shape) != tuple(c.shape):
+            raise LoweringRejected("SwiGLU needs both weights in one layout")
+        prob = _matmul_problem(a, b, up.attrs["trans_A"], up.attrs["trans_B"])
+        if prob["batch_A"] != 1 or prob["batch_B"] != 1:
+            raise LoweringRejected("SwiGLU is built for 2-D operands")
+        return "swiglu", prob, {"A": a, "B": b, "C": c}
+    return None
+
+
 def _matmul_problem(a, b, trans_a, trans_b) -> dict:
     sa, sb = tuple(a.shape), tuple(b.shape)
     if len(sa) != len(sb) or len(sa) < 2:
@@ -349,7 +377,7 @@ def _try_attention(view, out):
     return "attention", prob, {"Q": q, "K": k, "V": v}
 
 
-_MATCHERS = (_try_rmsnorm_matmul, _try_attention, _try_matmul)
+_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_attention, _try_matmul)
 
 
 def recognize(graph: Graph) -> Lowered:
@@ -371,7 +399,7 @@ def recognize(graph: Graph) -> Lowered:
                 _check_split_axes(family, operands, view.split_axes)
             return Lowered(family, problem, operands, outs, graph, dict(view.split_axes), split_dim)
     raise LoweringRejected(f"{graph.name}: ops {graph.op_kinds()} match no kernel family "
-                           "(matmul, rmsnorm_matmul, attention, mla)")
+                           "(matmul, rmsnorm_matmul, swiglu, attention, mla)")
 
 
 def _check_split_axes(family, operands, split_axes):

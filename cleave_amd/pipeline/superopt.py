@@ -121,8 +121,10 @@ def _split_dim_of(program, lowered) -> str | None:
         node, axis = lowered.operands["A"], (-2 if lowered.problem["trans_A"] else -1)
     elif lowered.family == "attention":
         node, axis = lowered.operands["K"], -2
-    else:
+    elif lowered.family == "mla":
         node, axis = lowered.operands["KV"], -2
+    else:
+        return None                     # no partial/combine form (SwiGLU: the gate is not linear)
     for spec in program.inputs:
         if f"PlaceHolder_{spec.name}" == node.name:
             d = spec.dims[axis]

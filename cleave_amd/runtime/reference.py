@@ -69,9 +69,9 @@ def make_inputs(graph, dtype=None, device: str = "cuda", seed: int | None = None
         else:
             x = torch.randn(tuple(ph.shape), generator=gen)
             low = getattr(graph, "lowered", None)
-            if low is not None and low.family in ("matmul", "rmsnorm_matmul") and getattr(graph, "role", "main") != "combine":
+            if low is not None and low.family in ("matmul", "rmsnorm_matmul", "swiglu") and getattr(graph, "role", "main") != "combine":
                 role = next((r for r, n in low.operands.items() if n is ph), None)
-                if role == "B":
+                if role in ("B", "C"):
                     x = x / math.sqrt(low.problem["K"])  # keep products O(1) so tolerances mean something
         made.append(x.to(dtype=torch_dtype(ph.dtype), device=device))
     return made
@@ -118,6 +118,17 @@ def _eval_matmul(low, feed, role, factor, out_dtype):
     if norm:
         y = y * torch.rsqrt((raw ** 2).mean(-1, keepdim=True) + p["eps"])
     return [y.to(out_dtype)]
+
+
+def _eval_swiglu(low, feed, out_dtype):
+    """``(a @ b) * silu(a @ c)``: products, gate and product of the two in fp32
+    (``tests/_graphs.py:403-436`` of the reference: every node of the graph is fp32 up to the output)."""
+    import torch
+
+    a, b = _mm_operands(low, feed)
+    c = feed[low.operands["C"].name].float()
+    c = (c.mT if low.problem["trans_B"] else c).unsqueeze(0)
+    return [((a @ b) * torch.nn.functional.silu(a @ c)).to(out_dtype)]
 
 
 def _eval_matmul_combine(low, feed, out_dtype, out_shape):
@@ -200,6 +211,8 @@ def execute(graph, inputs, device=None) -> list:
             return _eval_matmul_combine(low, feed, out_dtype, shapes[0])
         res = _eval_matmul(low, feed, role, factor, torch_dtype(graph.dtype))
         return [r.reshape(s) for r, s in zip(res, shapes)]
+    if low.family == "swiglu":
+        return [r.reshape(s) for r, s in zip(_eval_swiglu(low, feed, out_dtype), shapes)]
     if low.family in ("attention", "mla"):
         if role == "combine":
             return _eval_attention_combine(feed, out_dtype, shapes[0])

@@ -28,6 +28,8 @@ def _candidates(graph, arch):
             cands += policy.gemm_candidates(low, role, factor, arch)
         cands += policy.gemm_dma_candidates(low, role, factor, arch)
         return cands
+    if fam == "swiglu":
+        return policy.swiglu_candidates(low, role, factor, arch)
     if fam == "attention":
         if not policy.attn_ok(low):
             raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "

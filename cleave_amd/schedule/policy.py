@@ -162,6 +162,28 @@ def gemm_dma_candidates(low, role, factor, arch: Arch):
     return out
 
 
+def swiglu_candidates(low, role, factor, arch: Arch):
+    """SwiGLU runs on the direct-to-LDS matmul with a B tile made of two halves, the same
+    columns of the bare weight and of the gate weight: the tilings of a matmul twice as wide in
+    which every wave owns an even number of column fragments (half of them per weight)."""
+    import copy
+
+    if factor and factor > 1:
+        return []
+    twin = copy.copy(low)
+    twin.family, twin.problem = "matmul", dict(low.problem, N=2 * low.problem["N"])
+    out = []
+    for c in gemm_dma_candidates(twin, role, None, arch):
+        t = c.tiling
+        tn = t["BN"] // t["WN"] // 16
+        if tn % 2 or low.problem["N"] % (t["BN"] // 2):
+            continue
+        c.tiling = dict(t, SWIGLU=1)
+        c.output_tile = [t["BM"], t["BN"] // 2]
+        out.append(c)
+    return out
+
+
 # ----------------------------------------------------------------------------- few-row matmul
 def skinny_ok(low) -> bool:
     p = low.problem

@@ -30,6 +30,12 @@ def rmsnorm_matmul_plain(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
 
 
 @cleave_amd.jit
+def swiglu(x: cl.Tensor["M", "K"], w_up: cl.Tensor["K", "N"], w_gate: cl.Tensor["K", "N"]):
+    """``(x @ w_up) * silu(x @ w_gate)`` (the reference's ``demo/swiglu.py`` / ``tests/_graphs.py:403-436``)."""
+    return (x @ w_up) * cl.silu(x @ w_gate)
+
+
+@cleave_amd.jit
 def gqa_decode_exact(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
     return cl.softmax((q @ k.mT) / q.shape[-1] ** 0.5, dim=-1) @ v
 
@@ -52,6 +58,7 @@ FULL = {
     "c2": dict(M=16, K=4096, N=11008),
     "c3": dict(HQ=256, HKV=64, SQ=1, SKV=8192, D=128),
     "c4": dict(B=16, H=128, D=512, PE=64, SKV=4096),
+    "swiglu": dict(M=4096, N=14336, K=4096),
 }
 SMALL = {
     "c1": dict(M=32, N=64, K=256),
@@ -71,6 +78,14 @@ def inputs_c1(shapes, seed=1, device="cpu"):
     x = (torch.rand(M, K, generator=g) * 2 - 1) / math.sqrt(K)
     w = (torch.rand(K, N, generator=g) * 2 - 1) / math.sqrt(K)
     return [x.to(torch.float16).to(device), w.to(torch.float16).to(device)]
+
+
+def inputs_swiglu(shapes, seed=6, device="cpu"):
+    g = _gen(seed)
+    M, N, K = shapes["M"], shapes["N"], shapes["K"]
+    x = torch.randn(M, K, generator=g)
+    ws = [torch.randn(K, N, generator=g) / math.sqrt(K) for _ in range(2)]
+    return [t.to(torch.float16).to(device) for t in (x, *ws)]
 
 
 def inputs_c2(shapes, seed=2, device="cpu"):

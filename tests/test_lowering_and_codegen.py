@@ -76,6 +76,39 @@ def test_graded_programs_map_to_their_families(case, family):
         assert g.lowered.problem["scale"] == pytest.approx(192 ** -0.5)
 
 
+def test_swiglu_is_a_family_of_its_own():
+    """``(x @ w_up) * silu(x @ w_gate)`` in either operand order: A the shared activation, B the
+    bare product's weight, C the weight under the silu; tilings of the direct-to-LDS matmul whose
+    B tile holds the same columns of both weights; no split-K form."""
+    import cleave_amd
+
+    shapes = dict(M=4096, N=14336, K=4096)
+    g = stage_graph(C.swiglu.trace(cl.f16, **shapes))
+    low = g.lowered
+    assert low.family == "swiglu" and (low.problem["M"], low.problem["N"], low.problem["K"]) == (4096, 14336, 4096)
+    assert {r: n.name for r, n in low.operands.items()} == {"A": "PlaceHolder_x", "B": "PlaceHolder_w_up",
+                                                            "C": "PlaceHolder_w_gate"}
+
+    @cleave_amd.jit
+    def flipped(x: cl.Tensor["M", "K"], w_gate: cl.Tensor["K", "N"], w_up: cl.Tensor["K", "N"]):
+        return cl.silu(x @ w_gate) * (x @ w_up)
+
+    low2 = stage_graph(flipped.trace(cl.f16, **shapes)).lowered
+    assert low2.family == "swiglu" and low2.operands["C"].name == "PlaceHolder_w_gate"
+
+    cands = search_tiling(g, topk=10_000)
+    assert cands and {c.template for c in cands} == {"gemm_dma"}
+    for c in cands:
+        t = c.tiling
+        assert t["SWIGLU"] == 1 and (t["BN"] // t["WN"] // 16) % 2 == 0 and c.output_tile == [t["BM"], t["BN"] // 2]
+    m = parse_manifest(source_for(C.swiglu.trace(cl.f16, **shapes), template="gemm_dma",
+                                  tiling=dict(BM=256, BN=256, BK=64, WM=4, WN=2, SWIGLU=1)))
+    assert [p["name"] for p in m["params"]] == ["PlaceHolder_x", "PlaceHolder_w_up", "PlaceHolder_w_gate", "OutputNode_0"]
+    assert m["launches"][0]["grid"] == ["112", "16", "1"]          # 14336 / (256 / 2) column tiles
+    with pytest.raises(LoweringRejected, match="no split form"):
+        split_stages(g, 4)
+
+
 def test_unrecognised_program_is_refused():
     from cleave_amd.frontend import Program
 
