@@ -247,7 +247,7 @@ class HipCodeGen:
 
     def _emit_gemm_dma(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
-        if plan.family not in ("matmul", "swiglu"):
+        if plan.family not in ("matmul", "swiglu", "matmul_rowsum"):
             raise CodegenError("the direct-to-LDS matmul template has no fused RMSNorm form")
         self._matmul_common(unit, plan, params, partial, combine, fused)
         tile = dict(BM=128, BN=128, BK=64, WM=2, WN=2)
@@ -258,6 +258,9 @@ class HipCodeGen:
         swiglu = plan.family == "swiglu"
         if swiglu != bool(tile.get("SWIGLU")) or (swiglu and (splits > 1 or combine)):
             raise CodegenError("SwiGLU is the SWIGLU tiling of the direct-to-LDS matmul, unsplit")
+        rowsum = plan.family == "matmul_rowsum"
+        if rowsum != bool(tile.get("ROWSUM")) or (rowsum and (splits > 1 or combine or p["N"] % tile["BN"])):
+            raise CodegenError("matmul + row sum is the ROWSUM tiling of the direct-to-LDS matmul, unsplit, over whole column tiles")
         # (SwiGLU: the B tile holds BN / 2 columns of each weight, so a tile covers BN / 2 columns of the output)
         out_bn = tile["BN"] // 2 if swiglu else tile["BN"]
         if swiglu and (tile["BN"] // tile["WN"] // 16) % 2:
@@ -269,7 +272,7 @@ class HipCodeGen:
                 raise CodegenError(f"K={p['K']} is not a multiple of splits*64={splits * 64}")
             if (not p["trans_B"] and p["N"] % 8) or (p["trans_A"] and p["M"] % 8) or p["K"] % 8:
                 raise CodegenError("16-byte global chunks need the minor extent of each operand to be a multiple of 8")
-            grid = (-(-p["N"] // out_bn), -(-p["M"] // tile["BM"]), batch * splits)
+            grid = (1 if rowsum else -(-p["N"] // out_bn), -(-p["M"] // tile["BM"]), batch * splits)
             # the tile images are static LDS arrays of the kernel: no dynamic LDS at launch
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, 0, self._partial_args)
         if combine:

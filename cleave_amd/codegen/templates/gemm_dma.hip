@@ -18,6 +18,11 @@
 //   CL_M CL_N CL_K  CL_BM CL_BN  CL_WM x CL_WN waves  CL_TRANS_A / CL_TRANS_B  CL_BATCH_A/B
 //   CL_SPLITS (split-K: f32 partial tiles to CL_ARG_PACC[split])  CL_GROUP_M (tile order patch)
 //
+// CL_ROWSUM: out[m] = sum over n of (A * B)[m, n].  A workgroup owns BM rows and walks every
+// column tile of B with the same accumulators (the sum over columns needs no per-column result:
+// the K steps of all column tiles are one long step sequence), then adds up each row: over the
+// lane's accumulators, over the four lane groups, over the waves that share the rows (LDS).
+//
 // CL_SWIGLU: C = (A * B) .* silu(A * G) with a second weight G (CL_ARG_C) laid out like B.  The
 // B tile is made of two halves, columns n0 .. n0 + BN/2 of B and the same columns of G, so a
 // workgroup covers BN/2 columns of C; every wave owns the same columns in both halves (half of its
@@ -43,6 +48,9 @@
 #define CL_SWIGLU 0
 #endif
 #define GD_OUT_BN (CL_SWIGLU ? CL_BN / 2 : CL_BN)   // columns of C a tile covers
+#ifndef CL_ROWSUM
+#define CL_ROWSUM 0
+#endif
 static_assert(CL_BK == 64, "K steps are 64 wide (128-byte K-minor rows)");
 static_assert((GD_TM & (GD_TM - 1)) == 0 && (GD_TN & (GD_TN - 1)) == 0, "wave tiles are powers of two");
 static_assert(CL_BM % 16 == 0 && CL_BN % 16 == 0, "tiles are multiples of 16");
@@ -190,7 +198,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // Workgroups are handed to the XCDs round-robin in launch order.  Renumber them so that the
   // ones an XCD runs at the same time are neighbours in C: launch id L -> the (L / 8)-th tile of
   // XCD (L % 8)'s contiguous share, tiles ordered in patches of CL_GROUP_M row-tiles.
-  constexpr int tiles_m = (CL_M + CL_BM - 1) / CL_BM, tiles_n = (CL_N + GD_OUT_BN - 1) / GD_OUT_BN;
+  constexpr int tiles_m = (CL_M + CL_BM - 1) / CL_BM, tiles_n = CL_ROWSUM ? 1 : (CL_N + GD_OUT_BN - 1) / GD_OUT_BN;
   constexpr int tiles = tiles_m * tiles_n;
   int tile_id = blockIdx.y * tiles_n + blockIdx.x;
   {
@@ -206,7 +214,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int batch = blockIdx.z / CL_SPLITS, split = blockIdx.z % CL_SPLITS;
   constexpr int k_per_split = CL_K / CL_SPLITS;
   const int k_begin = split * k_per_split;
-  constexpr int KT = k_per_split / GD_BK;
+  constexpr int KT_K = k_per_split / GD_BK;                     // steps along K
+  constexpr int KT = KT_K * (CL_ROWSUM ? CL_N / CL_BN : 1);     // ... times the column tiles one workgroup walks
+#if CL_ROWSUM
+  static_assert(CL_N % CL_BN == 0 && CL_SPLITS == 1 && GD_BATCH == 1, "row sums walk whole column tiles, unsplit");
+#endif
 
   const elem_t* A = CL_ARG_A + (i64)(batch / (GD_BATCH / CL_BATCH_A)) * CL_M * CL_K;
   const elem_t* B = CL_ARG_B + (i64)(batch / (GD_BATCH / CL_BATCH_B)) * CL_K * CL_N;
@@ -327,17 +339,24 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GD_ISSUE(kt, a_lds, b_lds)
 #define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)
 #else
+#if CL_ROWSUM
+#define GD_A_AT(kt) (a_base + (i64)((kt) % KT_K) * a_step)
+#define GD_B_AT(kt) (b_base + (i64)((kt) % KT_K) * b_step + (i64)((kt) / KT_K) * (CL_TRANS_B ? (i64)CL_BN * CL_K : (i64)CL_BN))
+#else
+#define GD_A_AT(kt) (a_base + (i64)(kt) * a_step)
+#define GD_B_AT(kt) (b_base + (i64)(kt) * b_step)
+#endif
 #define GD_ISSUE(kt, a_lds, b_lds)                              \
-  opa.issue(a_base + (i64)(kt) * a_step, a_lds);                \
-  opb.issue(b_base + (i64)(kt) * b_step, b_lds);                \
+  opa.issue(GD_A_AT(kt), a_lds);                                \
+  opb.issue(GD_B_AT(kt), b_lds);                                \
   __builtin_amdgcn_sched_barrier(0);
 #define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)                                                         \
   {                                                                                                 \
     constexpr int ua_ = decltype(opa)::PER, ub_ = decltype(opb)::PER;                               \
     constexpr int per_row_ = (ua_ + ub_ + 2 * GD_TM - 1) / (2 * GD_TM);                             \
     _Pragma("unroll") for (int q_ = (r) * per_row_; q_ < ((r) + 1) * per_row_; ++q_) {             \
-      if (q_ < ua_) opa.issue_unit(q_, a_base + (i64)(kt) * a_step, a_lds);                         \
-      else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, b_base + (i64)(kt) * b_step, b_lds);        \
+      if (q_ < ua_) opa.issue_unit(q_, GD_A_AT(kt), a_lds);                                         \
+      else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, GD_B_AT(kt), b_lds);                        \
     }                                                                                               \
   }
 #endif
@@ -374,6 +393,30 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   if constexpr (KT % 2 == 1) GD_COMPUTE(gd_a0, gd_b0, GD_NO_NEXT)     // an odd number of steps ends on stage 0
 
   // ---- epilogue: acc[i][j][r] = C[m0 + am + 16 i + c][n0 + bn + 16 j + 4 g + r] ----------------
+#if CL_ROWSUM
+  {
+    __syncthreads();                                  // every wave is done with the tile images
+    float* red = reinterpret_cast<float*>(gd_b0);     // [BM][WN]
+#pragma unroll
+    for (int i = 0; i < GD_TM; ++i) {
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < GD_TN; ++j) sum += (acc[i][j][0] + acc[i][j][1]) + (acc[i][j][2] + acc[i][j][3]);
+      sum += lane_xor(sum, lane, 16);
+      sum += lane_xor(sum, lane, 32);
+      if (g == 0) red[(am + 16 * i + c) * CL_WN + wn] = sum;
+    }
+    __syncthreads();
+    for (int r = threadIdx.x; r < CL_BM; r += GD_THREADS) {
+      if (m0 + r >= CL_M) break;
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < CL_WN; ++w) sum += red[r * CL_WN + w];
+      CL_ARG_OUT[m0 + r] = to_elem(sum);
+    }
+    return;
+  }
+#endif
 #pragma unroll
   for (int i = 0; i < GD_TM; ++i) {
     const int m = m0 + am + 16 * i + c;

@@ -31,7 +31,7 @@ from .graph import ComputeOpNode, Graph, Node, OutputNode, PlaceHolderNode
 class Lowered:
     """A recognised operator: family, sizes and which placeholder plays which operand."""
 
-    family: str                       # matmul | rmsnorm_matmul | swiglu | attention | mla
+    family: str                       # matmul | rmsnorm_matmul | swiglu | matmul_rowsum | attention | mla
     problem: dict                     # sizes and flags the template needs
     operands: dict                    # role -> PlaceHolderNode
     outputs: list                     # OutputNodes in order
@@ -226,6 +226,26 @@ def _try_swiglu(view, out):
     return None
 
 
+def _try_matmul_rowsum(view, out):
+    """``(a @ b).sum(dim=-1)``: the row sums of a product that is never stored
+    (the reference's ``tests/_graphs.py:150-160``)."""
+    n = view.skip(out)
+    if not (_is(n, "reduce_sum") and view.reduce_dim(n) == -1):
+        return None
+    mm = view.ins(n)[0]
+    if not _is(mm, "matmul"):
+        return None
+    a, b = view.ins(mm)
+    if not (isinstance(a, PlaceHolderNode) and isinstance(b, PlaceHolderNode)):
+        return None
+    if view.is_split:
+        raise LoweringRejected("matmul + row sum has no split form here")
+    prob = _matmul_problem(a, b, mm.attrs["trans_A"], mm.attrs["trans_B"])
+    if prob["batch_A"] != 1 or prob["batch_B"] != 1:
+        raise LoweringRejected("matmul + row sum is built for 2-D operands")
+    return "matmul_rowsum", prob, {"A": a, "B": b}
+
+
 def _matmul_problem(a, b, trans_a, trans_b) -> dict:
     sa, sb = tuple(a.shape), tuple(b.shape)
     if len(sa) != len(sb) or len(sa) < 2:
@@ -377,7 +397,7 @@ def _try_attention(view, out):
     return "attention", prob, {"Q": q, "K": k, "V": v}
 
 
-_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_attention, _try_matmul)
+_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_matmul_rowsum, _try_attention, _try_matmul)
 
 
 def recognize(graph: Graph) -> Lowered:
@@ -399,7 +419,7 @@ def recognize(graph: Graph) -> Lowered:
                 _check_split_axes(family, operands, view.split_axes)
             return Lowered(family, problem, operands, outs, graph, dict(view.split_axes), split_dim)
     raise LoweringRejected(f"{graph.name}: ops {graph.op_kinds()} match no kernel family "
-                           "(matmul, rmsnorm_matmul, swiglu, attention, mla)")
+                           "(matmul, rmsnorm_matmul, swiglu, matmul_rowsum, attention, mla)")
 
 
 def _check_split_axes(family, operands, split_axes):

@@ -69,7 +69,7 @@ def make_inputs(graph, dtype=None, device: str = "cuda", seed: int | None = None
         else:
             x = torch.randn(tuple(ph.shape), generator=gen)
             low = getattr(graph, "lowered", None)
-            if low is not None and low.family in ("matmul", "rmsnorm_matmul", "swiglu") and getattr(graph, "role", "main") != "combine":
+            if low is not None and low.family in ("matmul", "rmsnorm_matmul", "swiglu", "matmul_rowsum") and getattr(graph, "role", "main") != "combine":
                 role = next((r for r, n in low.operands.items() if n is ph), None)
                 if role in ("B", "C"):
                     x = x / math.sqrt(low.problem["K"])  # keep products O(1) so tolerances mean something
@@ -213,6 +213,9 @@ def execute(graph, inputs, device=None) -> list:
         return [r.reshape(s) for r, s in zip(res, shapes)]
     if low.family == "swiglu":
         return [r.reshape(s) for r, s in zip(_eval_swiglu(low, feed, out_dtype), shapes)]
+    if low.family == "matmul_rowsum":
+        a, b = _mm_operands(low, feed)
+        return [(a @ b).sum(-1).to(out_dtype).reshape(shapes[0])]
     if low.family in ("attention", "mla"):
         if role == "combine":
             return _eval_attention_combine(feed, out_dtype, shapes[0])

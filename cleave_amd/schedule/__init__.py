@@ -30,6 +30,8 @@ def _candidates(graph, arch):
         return cands
     if fam == "swiglu":
         return policy.swiglu_candidates(low, role, factor, arch)
+    if fam == "matmul_rowsum":
+        return policy.rowsum_candidates(low, role, factor, arch)
     if fam == "attention":
         if not policy.attn_ok(low):
             raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "

@@ -184,6 +184,33 @@ def swiglu_candidates(low, role, factor, arch: Arch):
     return out
 
 
+def rowsum_candidates(low, role, factor, arch: Arch):
+    """Matmul + row sum: tilings of the direct-to-LDS matmul in which one workgroup owns BM rows and
+    walks all of N (whole column tiles), so the grid is the row tiles alone: ranked by how many
+    step sequences of ``(N / BN) * (K / 64)`` steps the machine runs one after another."""
+    import copy
+
+    if factor and factor > 1:
+        return []
+    p = low.problem
+    twin = copy.copy(low)
+    twin.family = "matmul"
+    out = []
+    for c in gemm_dma_candidates(twin, role, None, arch):
+        t = c.tiling
+        if p["N"] % t["BN"]:
+            continue
+        blocks = _ceil(p["M"], t["BM"])
+        steps = (p["N"] // t["BN"]) * (p["K"] // 64)
+        waves = t["WM"] * t["WN"]
+        mfma_clk = (t["BM"] // t["WM"] // 16) * (t["BN"] // t["WN"] // 16) * 2 * 16.4 * max(1.0, waves / 4.0)
+        c.score = _waves_time(blocks, 1, arch) * steps * (mfma_clk + 700)
+        c.tiling = dict(t, ROWSUM=1)
+        c.output_tile = [t["BM"], 1]
+        out.append(c)
+    return out
+
+
 # ----------------------------------------------------------------------------- few-row matmul
 def skinny_ok(low) -> bool:
     p = low.problem

@@ -36,6 +36,12 @@ def swiglu(x: cl.Tensor["M", "K"], w_up: cl.Tensor["K", "N"], w_gate: cl.Tensor[
 
 
 @cleave_amd.jit
+def matmul_rowsum(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
+    """Row sums of a product that is never stored (the reference's ``tests/_graphs.py:150-160``)."""
+    return (x @ w).sum(dim=-1, keepdim=True)
+
+
+@cleave_amd.jit
 def gqa_decode_exact(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
     return cl.softmax((q @ k.mT) / q.shape[-1] ** 0.5, dim=-1) @ v
 
@@ -59,6 +65,7 @@ FULL = {
     "c3": dict(HQ=256, HKV=64, SQ=1, SKV=8192, D=128),
     "c4": dict(B=16, H=128, D=512, PE=64, SKV=4096),
     "swiglu": dict(M=4096, N=14336, K=4096),
+    "matmul_rowsum": dict(M=4096, N=4096, K=64),
 }
 SMALL = {
     "c1": dict(M=32, N=64, K=256),

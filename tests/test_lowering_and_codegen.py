@@ -109,6 +109,18 @@ def test_swiglu_is_a_family_of_its_own():
         split_stages(g, 4)
 
 
+def test_matmul_rowsum_is_a_family_of_its_own():
+    g = stage_graph(C.matmul_rowsum.trace(cl.f16, **C.FULL["matmul_rowsum"]))
+    assert g.lowered.family == "matmul_rowsum" and g.outputs[0].shape == (4096, 1)
+    cands = search_tiling(g, topk=10_000)
+    assert cands and all(c.template == "gemm_dma" and c.tiling["ROWSUM"] == 1 and 4096 % c.tiling["BN"] == 0 for c in cands)
+    m = parse_manifest(source_for(C.matmul_rowsum.trace(cl.f16, **C.FULL["matmul_rowsum"]), template="gemm_dma",
+                                  tiling=dict(BM=16, BN=256, BK=64, WM=1, WN=4, ROWSUM=1)))
+    assert m["launches"][0]["grid"] == ["1", "256", "1"]           # one workgroup per 16 rows walks all of N
+    with pytest.raises(LoweringRejected, match="no split form"):
+        split_stages(g, 2)
+
+
 def test_unrecognised_program_is_refused():
     from cleave_amd.frontend import Program
 
