@@ -64,6 +64,10 @@ def op_table():
                        shapes=C.FULL["swiglu"], inputs=C.inputs_swiglu, split=False,
                        bytes=2 * (4096 * 4096 + 2 * 4096 * 14336 + 4096 * 14336), flops=4 * 4096 * 14336 * 4096,
                        bound="mfma", sets=2),
+        "attn": dict(title="dense GQA attention f16 B=1 Hq=32 Hkv=8 S=4096 SKV=4096 D=64 (the reference's gqa_bhsd case)",
+                     fn=C.gqa_decode_exact, dtype=cl.f16, shapes=dict(HQ=32, HKV=8, SQ=4096, SKV=4096, D=64),
+                     inputs=C.inputs_c3, split=False, bytes=2 * (2 * 32 * 4096 * 64 + 2 * 8 * 4096 * 64),
+                     flops=4 * 32 * 4096 * 4096 * 64, bound="mfma", sets=2),
         "mmrs": dict(title="matmul + row sum f16 (x@w).sum(-1) 4096x4096x64", fn=C.matmul_rowsum, dtype=cl.f16,
                      shapes=C.FULL["matmul_rowsum"], inputs=C.inputs_c1, split=False,
                      bytes=2 * (4096 * 64 + 64 * 4096 + 4096), flops=2 * 4096 * 4096 * 64, bound="mfma", sets=4),
@@ -387,7 +391,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,mmrs")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,mmrs,attn")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")

@@ -399,7 +399,32 @@ class HipCodeGen:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv({grid_rows} * {p['vdim'] // 4}, 256)", 1, 1), 256, 0, args)
 
+    def _emit_attn_dense_prefill(self, unit, plan, params, partial, combine):
+        """The LDS-shared prefill kernel over the dense attention family's operands: every unit
+        (batch entry x kv head) has ``group * sq`` query rows that all see all keys."""
+        p, op = plan.problem, plan.operands
+        if combine or (plan.split_factor or 1) > 1:
+            raise CodegenError("the many-row attention kernel has no split-KV form")
+        d, rows = p["head_dim"], p["group"] * p["sq"]
+        if d % 64 or d > 256 or p["vdim"] % 64 or p["vdim"] > 256:
+            raise CodegenError("the many-row attention kernel needs key and value widths in whole 64-feature panels (<= 256)")
+        self._attn_common(unit, plan, params, partial, combine, False, p["vdim"], p["units"] * rows, False)
+        for k, v in (("CL_DENSE", 1), ("CL_RAGGED", 1), ("CL_HEAD_DIM", d), ("CL_KV_HEADS", 1), ("CL_Q_HEADS", 1),
+                     ("CL_ROWS", rows), ("CL_SKV", p["skv"])):
+            unit.define(k, v)
+        unit.define("CL_SCALE", _f(float(p.get("scale", 1.0))))
+        for role, macro in (("Q", "CL_ARG_Q"), ("K", "CL_ARG_K"), ("V", "CL_ARG_V")):
+            unit.define(macro, op[role])
+        for k, v in plan.tiling.items():
+            if k != "SHARED":
+                unit.define(f"CL_PF_{k}", int(v))
+        unit.templates.append("attn_prefill_lds.hip")
+        items = -(-(-(-rows // 128)) // 8) * 8                  # padded to a multiple of 8 (one eighth of the space per XCD)
+        unit.launch(ENTRY, (items, p["units"], 1), 256, 0, self._partial_args)
+
     def _emit_attn_prefill(self, unit, plan, params, partial, combine, fused):
+        if not plan.problem.get("paged"):
+            return self._emit_attn_dense_prefill(unit, plan, params, partial, combine)
         """Causal prefill over ragged queries (token-table or packed keys): one item per 16-row tile
         (tokens x head group of one kv head), one wave per kv head."""
         p, op = plan.problem, plan.operands

@@ -21,6 +21,11 @@
 // boundary (item t = chunk w + request b for the one pair that overlaps); an item stops at the
 // last key any of its rows may see and writes zeros / -inf without reading when it sees none.
 //
+// CL_DENSE: the same kernel over dense operands Q (units, rows, d), K and V (units, keys, d), every
+// row seeing every key (the dense attention family with many query rows per unit): CL_ROWS,
+// CL_SKV and CL_SCALE are constants, an item is 128 consecutive rows of one unit, there are no
+// row pointers and no lse.
+//
 //   CL_HEAD_DIM (multiple of 64)  CL_KV_HEADS  CL_Q_HEADS (group divides 16)  CL_RAGGED
 //   run-time: batch, total_q, n_idx (table length / total_kv), num_pages (table form), sm_scale
 
@@ -30,20 +35,28 @@
 #ifndef CL_PF_REVERSE
 #define CL_PF_REVERSE 1
 #endif
+#ifndef CL_DENSE
+#define CL_DENSE 0
+#endif
+#if CL_DENSE && !CL_RAGGED
+#error "dense operands have consecutive key rows (CL_RAGGED)"
+#endif
 #define PL_STEP 32
 #define PL_GROUP (CL_Q_HEADS / CL_KV_HEADS)
 #define PL_ROWS 128
 #define PL_QT (PL_ROWS / PL_GROUP)            // query tokens per item
-#define PL_PANELS (CL_HEAD_DIM / 64)
+#define PL_KPANELS (CL_HEAD_DIM / 64)         // key width and value width (CL_VDIM) may differ
+#define PL_VPANELS (CL_VDIM / 64)
 #define PL_PANEL (PL_STEP * 64)               // elements of one 64-feature panel
-#define PL_IMG (PL_PANELS * PL_PANEL)         // elements of one operand image
-#define PL_STAGE (2 * PL_IMG)                 // K image, then V image
+#define PL_KIMG (PL_KPANELS * PL_PANEL)       // elements of the K image
+#define PL_STAGE ((PL_KPANELS + PL_VPANELS) * PL_PANEL)   // K image, then V image
 #define PL_STAGES 4
 #define PL_KJ (CL_HEAD_DIM / 32)
-#define PL_FB (CL_HEAD_DIM / 16)
-#define PL_UNITS_PER (2 * PL_PANELS)          // 1 KiB loads per wave and step: its 8-key group of every panel of K and V
+#define PL_FB (CL_VDIM / 16)
+#define PL_UNITS_PER (PL_KPANELS + PL_VPANELS)   // 1 KiB loads per wave and step: its 8-key group of every panel of K and V
 static_assert(CL_Q_HEADS % CL_KV_HEADS == 0 && 16 % PL_GROUP == 0, "the head group divides the 16-row query tile");
-static_assert(CL_HEAD_DIM % 64 == 0 && CL_HEAD_DIM <= 256, "head dim in whole 64-feature panels");
+static_assert(CL_HEAD_DIM % 64 == 0 && CL_HEAD_DIM <= 256 && CL_VDIM % 64 == 0 && CL_VDIM <= 256,
+              "key and value widths in whole 64-feature panels");
 static_assert(PL_UNITS_PER < 16, "load counter range");
 
 __shared__ __attribute__((aligned(1024))) elem_t pl_tiles[PL_STAGES * PL_STAGE];
@@ -69,13 +82,6 @@ CL_DEVICE void pl_dma16(const void* gptr, unsigned lds_byte) {
 CL_DEVICE void pl_dma4(const void* gptr, unsigned lds_byte) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)) : "memory");
-}
-template <int P>
-CL_DEVICE void pl_issue_panels(const char* src, unsigned group_byte) {
-  if constexpr (P < PL_PANELS) {
-    pl_dma16<128 * P>(src, group_byte + (unsigned)(P * PL_PANEL * 2) - 128 * P);
-    pl_issue_panels<P + 1>(src, group_byte);
-  }
 }
 
 template <int I> struct PlC { static constexpr int value = I; };
@@ -119,6 +125,18 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     item = lin % gx;
     head = lin / gx;
   }
+#if CL_DENSE
+  // dense operands: `head` is a unit (batch entry x kv head) with CL_ROWS query rows (its head group
+  // x the query positions, all seeing all CL_SKV keys); an item is 128 consecutive rows of them
+  const int lo = item * PL_ROWS;
+  if (lo >= CL_ROWS) return;                            // (the item axis is padded)
+  const int n_rows = CL_ROWS - lo < PL_ROWS ? CL_ROWS - lo : PL_ROWS;
+  const int q0 = 0, kv0 = 0, kv_len = CL_SKV, off = 0, ext = CL_SKV;
+  const float sm_scale = CL_SCALE;
+  (void)q0; (void)off;
+  auto row_index = [&](int m) __attribute__((always_inline)) { return (i64)head * CL_ROWS + lo + m; };
+  auto row_limit = [&](int m) __attribute__((always_inline)) { (void)m; return CL_SKV - 1; };
+#else
   // The request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item.
   // The condition holds for every request up to that one, so the lanes test 64 requests at a time
   // and count (one round trip to memory per 64 requests instead of one per halving); with up to
@@ -158,16 +176,23 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   ext = ext < kv_len ? ext : kv_len;
   ext = ext > 0 ? ext : 0;
 
-  // this lane's two query rows (column c of each of the wave's score tiles): token, head, last key it may see
+  // output (and query) row of the item's row m, and the last key it may see
+  auto row_index = [&](int m) __attribute__((always_inline)) {
+    return (i64)(lo + m / PL_GROUP) * CL_Q_HEADS + head * PL_GROUP + m % PL_GROUP;
+  };
+  auto row_limit = [&](int m) __attribute__((always_inline)) { return off + (lo + m / PL_GROUP - q0); };
+#endif
+
+  // this lane's two query rows (column c of each of the wave's score tiles): row index, last key it may see
   bool live[2];
-  int tok[2], qhead[2], limit[2];
+  i64 orow[2];
+  int limit[2];
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
     const int m = 32 * wave + 16 * rt + c;
     live[rt] = m < n_rows;
-    tok[rt] = lo + (live[rt] ? m / PL_GROUP : 0);
-    qhead[rt] = head * PL_GROUP + (live[rt] ? m % PL_GROUP : 0);
-    limit[rt] = live[rt] ? off + (tok[rt] - q0) : -1;
+    orow[rt] = row_index(live[rt] ? m : 0);
+    limit[rt] = live[rt] ? row_limit(m) : -1;
   }
 
   if (ext == 0) {
@@ -175,11 +200,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
       if (!live[rt]) continue;
-      elem_t* dst = CL_ARG_OUT + ((i64)tok[rt] * CL_Q_HEADS + qhead[rt]) * CL_HEAD_DIM + 16 * (g & 1) + 4 * (g & 2);
+      elem_t* dst = CL_ARG_OUT + orow[rt] * CL_VDIM + 16 * (g & 1) + 4 * (g & 2);
 #pragma unroll
       for (int fp = 0; fp < PL_FB / 2; ++fp) *reinterpret_cast<u32x4*>(dst + 32 * fp) = (u32x4){0u, 0u, 0u, 0u};
 #if CL_EMIT_LSE
-      if (g == 0) CL_ARG_LSE[(i64)tok[rt] * CL_Q_HEADS + qhead[rt]] = CL_NEG_INF;
+      if (g == 0) CL_ARG_LSE[orow[rt]] = CL_NEG_INF;
 #endif
     }
     return;
@@ -188,9 +213,16 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // the softmax scale as a positive factor of the raw scores (its sign goes into the Q rows, exactly)
   const float scale2 = fmaxf(fabsf(sm_scale) * 1.4426950408889634f, 1.0e-30f);
   const unsigned q_sign = sm_scale < 0.f ? 0x80008000u : 0u;
-  const i64 row_bytes = (i64)CL_KV_HEADS * CL_HEAD_DIM * 2;
+#if CL_DENSE
+  const i64 krow_bytes = (i64)CL_HEAD_DIM * 2, vrow_bytes = (i64)CL_VDIM * 2;       // K, V: (unit, key, feature)
+  const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_SKV * CL_HEAD_DIM * 2;
+  const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_SKV * CL_VDIM * 2;
+#else
+  // K, V: (key row, kv head, feature)
+  const i64 krow_bytes = (i64)CL_KV_HEADS * CL_HEAD_DIM * 2, vrow_bytes = (i64)CL_KV_HEADS * CL_VDIM * 2;
   const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_HEAD_DIM * 2;
-  const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_HEAD_DIM * 2;
+  const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_VDIM * 2;
+#endif
 #if CL_PF_DBG_ONESTEP
   const int n_steps = 1;
 #else
@@ -230,10 +262,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
   // load `part` of a step (its K panels, then its V panels) into stage `slot`
   auto issue_part = [&](int row, int slot, auto part_c) __attribute__((always_inline)) {
-    constexpr int PART = decltype(part_c)::value, P = PART % PL_PANELS;
+    constexpr int PART = decltype(part_c)::value;
+    constexpr bool IS_K = PART < PL_KPANELS;
+    constexpr int P = IS_K ? PART : PART - PL_KPANELS;
     const int chunk = (lane & 7) ^ pl_swz(my_r);
-    const char* src = (PART < PL_PANELS ? kbase : vbase) + (i64)row * row_bytes + 16 * chunk;
-    const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024) + (PART < PL_PANELS ? 0 : PL_IMG * 2);
+    const char* src = (IS_K ? kbase + (i64)row * krow_bytes : vbase + (i64)row * vrow_bytes) + 16 * chunk;
+    const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024) + (IS_K ? 0 : PL_KIMG * 2);
     pl_dma16<128 * P>(src, group_byte + (unsigned)(P * PL_PANEL * 2) - 128 * P);
   };
   // the quarter `place` (0..3) of a step's loads: the body spreads them between its matrix work,
@@ -265,7 +299,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   elem8 qf[2][PL_KJ];
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
-    const elem_t* row = CL_ARG_Q + ((i64)tok[rt] * CL_Q_HEADS + qhead[rt]) * CL_HEAD_DIM + 8 * g;
+    const elem_t* row = CL_ARG_Q + orow[rt] * CL_HEAD_DIM + 8 * g;
 #pragma unroll
     for (int j = 0; j < PL_KJ; ++j) {
 #if CL_PF_DBG_NOQ
@@ -296,7 +330,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // row has the smallest limit (a wave without live rows masks nothing: its rows are not written).
   int n_full = n_steps;
   if (32 * wave < n_rows) {
-    const int first_limit = off + (lo + (32 * wave) / PL_GROUP - q0);
+    const int first_limit = row_limit(32 * wave);
     n_full = first_limit < 0 ? 0 : (first_limit + 1) / PL_STEP;
     n_full = n_full < n_steps ? n_full : n_steps;
   }
@@ -313,7 +347,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // 16 fb + (0..15), slots = keys 4 g + (0..3), 16 + 4 g + (0..3)
   auto v_frag = [&](auto slot_c, int fb) __attribute__((always_inline)) {
     constexpr int SLOT = decltype(slot_c)::value;
-    const elem_t* p = pl_tiles + SLOT * PL_STAGE + PL_IMG + (fb >> 2) * PL_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
+    const elem_t* p = pl_tiles + SLOT * PL_STAGE + PL_KIMG + (fb >> 2) * PL_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
     const pl_s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p));
     const pl_s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p + 16 * 64));
     return __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -509,12 +543,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     if (l != 12345.f) continue;
 #endif
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
-    const i64 orow = (i64)(lo + m / PL_GROUP) * CL_Q_HEADS + head * PL_GROUP + m % PL_GROUP;
+    const i64 orow = row_index(m);
     // A lane holds features 16 fb + 4 g .. + 3 of its row for every block fb.  Lanes g and g ^ 1
     // trade halves of a pair of blocks (one row swap per register), so that each stores 16
     // contiguous bytes: even g the 8 features from 4 g of the even block, odd g those from
     // 4 (g - 1) of the odd one.
-    elem_t* dst = CL_ARG_OUT + orow * CL_HEAD_DIM + 16 * (g_e & 1) + 4 * (g_e & 2);
+    elem_t* dst = CL_ARG_OUT + orow * CL_VDIM + 16 * (g_e & 1) + 4 * (g_e & 2);
 #pragma unroll
     for (int fp = 0; fp < PL_FB / 2; ++fp) {
       elem4 y0, y1;

@@ -307,6 +307,23 @@ def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
     return out
 
 
+def attn_many_rows_candidates(low, role, factor, arch: Arch):
+    """Units with many query rows (prefill-shaped dense attention): the kernel whose four waves
+    share every key tile through LDS, 128 query rows per workgroup, instead of one 16-row tile per
+    workgroup streaming all keys.  Unsplit, key and value widths in 64-feature panels."""
+    p = low.problem
+    rows, d = p["group"] * p["sq"], p["head_dim"]
+    vd = p["vdim"]
+    if (factor or 1) > 1 or rows < 64 or d % 64 or d > 256 or vd % 64 or vd > 256 or p["skv"] < 1:
+        return []
+    items = p["units"] * _ceil(rows, 128)
+    steps = _ceil(p["skv"], 32)
+    # a workgroup-step is 32 matrix ops per wave beside as many vector ops; two workgroups per CU
+    score = _waves_time(items, 2, arch) * (steps * 2200 + 9000)
+    return [TileDict("attn_prefill", role, dict(SHARED=1), output_tile=[128, vd], rstep_map={"kv": 32}, n_threads=256,
+                     split_factor=factor, score=score, lds_bytes=4 * 32 * (d + vd) * 2, est_vgprs=230)]
+
+
 # ----------------------------------------------------------------------------- MLA decode
 def mla_lds_bytes(ckv, kpe, stages=3):
     """`stages` token-major images of a 32-token step: (ckv + kpe) / 64 panels of 32 x 64 elements."""

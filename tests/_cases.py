@@ -47,6 +47,13 @@ def gqa_decode_exact(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "
 
 
 @cleave_amd.jit
+def mla_prefill(q: cl.Tensor["H", "SQ", "DK"], k: cl.Tensor["H", "SKV", "DK"], v: cl.Tensor["H", "SKV", "DV"]):
+    """Attention with a key width that differs from the value width (the reference's
+    ``mla_prefill_bhsd`` case, 192 / 128: ``tests/schedule/end2end/test_end2end.py:33``)."""
+    return cl.softmax((q @ k.mT) / q.shape[-1] ** 0.5, dim=-1) @ v
+
+
+@cleave_amd.jit
 def gqa_decode_shift(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
     n = q.shape[-1] ** 0.5
     return cl.softmax((q @ k.mT) / n, dim=-1, shift=-50 / n) @ v

@@ -1,0 +1,99 @@
+"""GPU parity of the dense attention family with many query rows per unit (the reference's
+prefill-shaped end-to-end cases ``flash_attention_sd``, ``mha_bhsd``, ``gqa_bhsd``, ``mqa_bhsd``:
+``tests/schedule/end2end/test_end2end.py:14-43``) through the kernel whose four waves share
+every key tile: against the numpy oracle at small sizes (ragged row and key counts, head widths
+64 / 128 / 256, both element types), and at the reference's sizes against a sample of rows."""
+
+import numpy as np
+import pytest
+import torch
+
+import cleave_amd.lang as cl
+from cleave_amd import pipeline as P
+from oracle import program_oracle
+from tests import _cases as C
+from tests._lowlevel import kernel_for, stage_graph
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(fn, dtype, shapes, seed=7):
+    prog = fn.trace(dtype, **shapes)
+    args = prog.random_inputs(seed=seed)
+    print(f"dense prefill case {prog.name} {dtype} {shapes}", flush=True)
+    out = kernel_for(prog, template="attn_prefill", tiling=dict(SHARED=1))(*args)
+    torch.cuda.synchronize()
+    want = program_oracle.evaluate(prog, list(args))[0]
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("shapes", [
+    dict(HQ=8, HKV=2, SQ=200, SKV=300, D=64),          # GQA, ragged rows (800 per unit) and keys
+    dict(HQ=4, HKV=4, SQ=130, SKV=64, D=128),          # MHA, two items per unit with a 2-row tail
+    dict(HQ=8, HKV=1, SQ=40, SKV=1000, D=128),         # MQA, 320 rows on one key set
+    dict(HQ=2, HKV=2, SQ=64, SKV=33, D=256),           # widest head, one full step and a 1-key tail
+], ids=["gqa_d64", "mha_d128", "mqa_d128", "mha_d256"])
+def test_dense_prefill_against_the_oracle(shapes):
+    _check(C.gqa_decode_exact, cl.f16, shapes)
+
+
+def test_dense_prefill_bf16_and_the_shifted_softmax_form():
+    _check(C.gqa_decode_exact, cl.bf16, dict(HQ=8, HKV=2, SQ=96, SKV=257, D=128))
+    _check(C.gqa_decode_shift, cl.f16, dict(HQ=8, HKV=4, SQ=100, SKV=200, D=64))
+
+
+def test_key_width_differs_from_value_width():
+    """192-wide keys, 128-wide values (the reference's ``mla_prefill_bhsd`` case): small against
+    the oracle, then the reference's size on a sample of rows."""
+    _check(C.mla_prefill, cl.f16, dict(H=4, SQ=100, SKV=150, DK=192, DV=128))
+    _check(C.mla_prefill, cl.bf16, dict(H=2, SQ=64, SKV=64, DK=128, DV=64))
+    shapes = dict(H=128, SQ=4096, SKV=4096, DK=192, DV=128)
+    prog = C.mla_prefill.trace(cl.f16, **shapes)
+    q, k, v = prog.random_inputs(seed=17)
+    out = kernel_for(prog)(q, k, v)
+    torch.cuda.synchronize()
+    gen = np.random.default_rng(2)
+    for h, s in zip(gen.integers(0, 128, 32), gen.integers(0, 4096, 32)):
+        w = torch.softmax((k[h].double() @ q[h, s].double()) / 192 ** 0.5, dim=0)
+        np.testing.assert_allclose(out[h, s].float().cpu().numpy(), (w @ v[h].double()).float().cpu().numpy(),
+                                   rtol=1e-2, atol=1e-2)
+
+
+def test_search_prefers_the_shared_kernel_for_many_rows_and_keeps_decode_for_few():
+    from cleave_amd.schedule import search_tiling
+
+    many = search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=32, HKV=8, SQ=4096, SKV=4096, D=64)), topk=3)
+    assert many[0].template == "attn_prefill" and {c.template for c in many} == {"attn_prefill", "attn_decode"}
+    few = search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, **C.FULL["c3"])), topk=20)
+    assert {c.template for c in few} == {"attn_decode"}
+
+
+@pytest.mark.parametrize("shapes", [dict(HQ=32, HKV=8, SQ=4096, SKV=4096, D=64), dict(HQ=32, HKV=32, SQ=4096, SKV=4096, D=64),
+                                    dict(HQ=32, HKV=1, SQ=4096, SKV=4096, D=64), dict(HQ=1, HKV=1, SQ=4096, SKV=4096, D=64)],
+                         ids=["gqa_bhsd", "mha_bhsd", "mqa_bhsd", "flash_attention_sd"])
+def test_reference_end_to_end_sizes_on_a_sample_of_rows(shapes):
+    """The searched best kernel at the reference's sizes; 64 query rows spread over heads and
+    positions are recomputed in float64."""
+    prog = C.gqa_decode_exact.trace(cl.f16, **shapes)
+    q, k, v = prog.random_inputs(seed=13)
+    out = kernel_for(prog)(q, k, v)
+    torch.cuda.synchronize()
+    gen = np.random.default_rng(1)
+    group = shapes["HQ"] // shapes["HKV"]
+    for h, s in zip(gen.integers(0, shapes["HQ"], 64), gen.integers(0, shapes["SQ"], 64)):
+        kk, vv = k[h // group].double(), v[h // group].double()
+        w = torch.softmax((kk @ q[h, s].double()) / shapes["D"] ** 0.5, dim=0)
+        np.testing.assert_allclose(out[h, s].float().cpu().numpy(), (w @ vv).float().cpu().numpy(), rtol=1e-2, atol=1e-2)
+
+
+def test_dense_prefill_compiles_end_to_end(cache_root):
+    shapes = dict(HQ=8, HKV=2, SQ=512, SKV=512, D=128)
+    kernel = P.compile(C.gqa_decode_exact, shapes=shapes, dtype=cl.f16, split=False, schedule=P.ScheduleConfig(topk=4),
+                       eval=P.EvalConfig(warmup=2, iters=10, max_parallel=2))
+    # (at this size the streaming kernel with four waves may still win: both forms are searched and validated)
+    assert len(kernel.report.correct) == len(kernel.report) >= 2
+    assert {"attn_prefill", "attn_decode"} <= {r.label.split("#")[1].split()[1].split("[")[0] for r in kernel.report.correct}
+    prog = C.gqa_decode_exact.trace(cl.f16, **shapes)
+    args = prog.random_inputs(seed=2)
+    np.testing.assert_allclose(kernel(*args).float().cpu().numpy(), program_oracle.evaluate(prog, list(args))[0],
+                               rtol=1e-2, atol=1e-2)
