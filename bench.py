@@ -67,7 +67,16 @@ def op_table():
         "attn": dict(title="dense GQA attention f16 B=1 Hq=32 Hkv=8 S=4096 SKV=4096 D=64 (the reference's gqa_bhsd case)",
                      fn=C.gqa_decode_exact, dtype=cl.f16, shapes=dict(HQ=32, HKV=8, SQ=4096, SKV=4096, D=64),
                      inputs=C.inputs_c3, split=False, bytes=2 * (2 * 32 * 4096 * 64 + 2 * 8 * 4096 * 64),
-                     flops=4 * 32 * 4096 * 4096 * 64, bound="mfma", sets=2),
+                     flops=4 * 32 * 4096 * 4096 * 64, bound="mfma", sets=2, cpu=False),
+        "qknorm": dict(title="QK-norm GQA attention f16 Hq=64 Hkv=8 S=4096 SKV=4096 D=128 (the reference's qknorm case)",
+                       fn=C.qknorm, dtype=cl.f16, shapes=dict(HQ=64, HKV=8, SQ=4096, SKV=4096, D=128), inputs=C.inputs_c3,
+                       split=False, bytes=2 * (2 * 64 * 4096 * 128 + 2 * 8 * 4096 * 128), flops=4 * 64 * 4096 * 4096 * 128,
+                       bound="mfma", sets=2, cpu=False),
+        "mlapf": dict(title="attention f16 H=128 S=4096 SKV=4096 keys 192 / values 128 wide (the reference's mla_prefill_bhsd case)",
+                      fn=C.mla_prefill, dtype=cl.f16, shapes=dict(H=128, SQ=4096, SKV=4096, DK=192, DV=128),
+                      inputs=C.inputs_mla_prefill, split=False,
+                      bytes=2 * 128 * 4096 * (192 + 128 + 192 + 128), flops=2 * 128 * 4096 * 4096 * (192 + 128),
+                      bound="mfma", sets=2, cpu=False),
         "mmrs": dict(title="matmul + row sum f16 (x@w).sum(-1) 4096x4096x64", fn=C.matmul_rowsum, dtype=cl.f16,
                      shapes=C.FULL["matmul_rowsum"], inputs=C.inputs_c1, split=False,
                      bytes=2 * (4096 * 64 + 64 * 4096 + 4096), flops=2 * 4096 * 4096 * 64, bound="mfma", sets=4),
@@ -391,7 +400,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,mmrs,attn")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,mmrs,attn,qknorm,mlapf")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")
@@ -424,9 +433,9 @@ def main():
         if name == "c5":
             results[name] = run_paged(max(10, args.steps // 4), max(2, args.warmup // 4), not args.no_cpu, args.kernels)
             continue
-        steps = args.steps if name not in ("mm", "swiglu") else max(10, args.steps // 10)
+        steps = args.steps if name not in ("mm", "swiglu", "attn", "qknorm", "mlapf") else max(10, args.steps // 10)
         res, program = run_dense(name, ops[name], steps, args.warmup, args.search_iters, args.kernels)
-        if not args.no_cpu:
+        if not args.no_cpu and ops[name].get("cpu", True):     # (the large attention cases would take the oracle minutes)
             cpu_us, runs = cpu_dense(program, ops[name], budget_s=8.0 if name != "c4" else 15.0)
             res["cpu_us"] = round(cpu_us, 1)
             res["cpu_sample"] = f"full workload, median of {runs} runs"

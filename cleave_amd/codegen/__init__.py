@@ -351,6 +351,8 @@ class HipCodeGen:
 
     def _emit_attn_decode(self, unit, plan, params, partial, combine, fused):
         p, t, op = plan.problem, plan.tiling, plan.operands
+        if p.get("norm_eps"):
+            raise CodegenError("the streaming attention kernel has no QK-norm form")
         paged = bool(p.get("paged"))
         rows = p["group"] * p["sq"]
         emit_lse = bool(p.get("emit_lse"))
@@ -413,6 +415,11 @@ class HipCodeGen:
                      ("CL_ROWS", rows), ("CL_SKV", p["skv"])):
             unit.define(k, v)
         unit.define("CL_SCALE", _f(float(p.get("scale", 1.0))))
+        norm = p.get("norm_eps") or {}
+        unit.define("CL_QNORM", "q" in norm)
+        unit.define("CL_KNORM", "k" in norm)
+        unit.define("CL_QNORM_EPS", _f(float(norm.get("q", 0.0))))
+        unit.define("CL_KNORM_EPS", _f(float(norm.get("k", 0.0))))
         for role, macro in (("Q", "CL_ARG_Q"), ("K", "CL_ARG_K"), ("V", "CL_ARG_V")):
             unit.define(macro, op[role])
         for k, v in plan.tiling.items():

@@ -26,6 +26,14 @@
 // CL_SKV and CL_SCALE are constants, an item is 128 consecutive rows of one unit, there are no
 // row pointers and no lse.
 //
+// CL_QNORM / CL_KNORM (QK-norm attention): query / key rows enter the scores RMS-normalised over
+// their features, x * rsqrt(mean(x^2) + eps).  Query rows are normalised once when they are loaded.
+// Key rows cannot be touched on their way into LDS, so their factors multiply the scores instead:
+// the sum of squares of the 16 keys of a score tile is the diagonal of K K^T, which the matrix
+// unit makes from the key fragments already in registers (A and B operand are the same
+// registers); the lanes on the diagonal take the reciprocal root and the lanes of each score
+// fetch the factor of its key.
+//
 //   CL_HEAD_DIM (multiple of 64)  CL_KV_HEADS  CL_Q_HEADS (group divides 16)  CL_RAGGED
 //   run-time: batch, total_q, n_idx (table length / total_kv), num_pages (table form), sm_scale
 
@@ -37,6 +45,12 @@
 #endif
 #ifndef CL_DENSE
 #define CL_DENSE 0
+#endif
+#ifndef CL_QNORM
+#define CL_QNORM 0
+#endif
+#ifndef CL_KNORM
+#define CL_KNORM 0
 #endif
 #if CL_DENSE && !CL_RAGGED
 #error "dense operands have consecutive key rows (CL_RAGGED)"
@@ -310,6 +324,20 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       if (!live[rt]) raw = (u32x4){0u, 0u, 0u, 0u};
       qf[rt][j] = as_elem8(raw ^ q_sign);
     }
+#if CL_QNORM
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PL_KJ; ++j)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += to_f32(qf[rt][j][i]) * to_f32(qf[rt][j][i]);
+    ss += lane_xor(ss, lane, 16);
+    ss += lane_xor(ss, lane, 32);
+    const float rq = fast_rsqrt(ss * (1.0f / CL_HEAD_DIM) + CL_QNORM_EPS);
+#pragma unroll
+    for (int j = 0; j < PL_KJ; ++j)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[rt][j][i] = to_elem(to_f32(qf[rt][j][i]) * rq);
+#endif
   }
 
   float m_run[2] = {CL_NEG_BIG, CL_NEG_BIG};   // running max of the scaled scores (log2 domain), uniform over g
@@ -353,6 +381,28 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     return __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
+#if CL_KNORM
+  // Factors of the keys of one step onto its raw scores.  gram[h] = K_h K_h^T for the 16 keys of
+  // half h: lane (c, g) holds rows 4 g .. 4 g + 3 of column c, so the lanes with c / 4 == g hold
+  // the diagonal entry of key c in register c % 4; score slot q of lane (c, g) belongs to key
+  // 4 g + q, whose factor is in lane 20 g + q.
+  const int kn_src[4] = {(20 * g + 0) << 2, (20 * g + 1) << 2, (20 * g + 2) << 2, (20 * g + 3) << 2};
+  auto scale_by_key_norms = [&](const f32x4 (&gram)[2], f32x4 (&sc)[2][2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int sel = c & 3;
+      const float d01 = sel & 1 ? gram[h][1] : gram[h][0], d23 = sel & 1 ? gram[h][3] : gram[h][2];
+      const float rk = fast_rsqrt((sel & 2 ? d23 : d01) * (1.0f / CL_HEAD_DIM) + CL_KNORM_EPS);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float f = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(kn_src[q], __builtin_bit_cast(int, rk)));
+        sc[0][h][q] *= f;
+        sc[1][h][q] *= f;
+      }
+    }
+  };
+#endif
+
   // The loop is skewed by one step: body s turns the scores of step s (made in body s - 1) into
   // weights and adds their value product, and between those vector instructions it issues the
   // score products of step s + 1, so that the matrix unit works in the shadow of the softmax.
@@ -366,6 +416,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   {
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) st[rt][0] = st[rt][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#if CL_KNORM
+    f32x4 gram[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};
+#endif
 #pragma unroll
     for (int j = 0; j < PL_KJ; ++j)
 #pragma unroll
@@ -373,7 +426,13 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         const elem8 a = k_frag(PlC<0>{}, j, h);
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) st[rt][h] = mfma16(a, qf[rt][j], st[rt][h]);
+#if CL_KNORM
+        gram[h] = mfma16(a, a, gram[h]);
+#endif
       }
+#if CL_KNORM
+    scale_by_key_norms(gram, st);
+#endif
   }
 
   // Body of step `step`, whose images are in stage SLOT (compile-time: every LDS address is a
@@ -507,6 +566,16 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // ---- value product of the second row tile ------------------------------------------------
 #pragma unroll
     for (int fb = 0; fb < PL_FB; ++fb) acc[1][fb] = mfma16(vf[fb], pf[1], acc[1][fb]);
+#if CL_KNORM
+    // (and the sums of squares of the keys of step + 1, whose factors go onto its scores)
+    f32x4 gram[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int j = 0; j < PL_KJ; ++j)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) gram[h] = mfma16(kf[j][h], kf[j][h], gram[h]);
+    __builtin_amdgcn_sched_barrier(0);
+    scale_by_key_norms(gram, sn);
+#endif
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll

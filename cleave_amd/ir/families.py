@@ -333,14 +333,37 @@ def _match_scores(view, n):
         parts = view.ins(core)
     else:
         parts = [core]
+    norms = {}
     for p in parts:
         if not (_is(p, "matmul") and not p.attrs["trans_A"] and p.attrs["trans_B"]):
             return None
         q, k = view.ins(p)
+        # RMSNorm over the feature axis on either operand (QK-norm attention): x * rnorm(x)
+        for side, t in (("q", q), ("k", k)):
+            hit = _normed(view, t)
+            if hit is not None:
+                if len(parts) != 1:
+                    return None
+                norms[side] = hit[1]
+                q, k = (hit[0], k) if side == "q" else (q, hit[0])
         if not (isinstance(q, PlaceHolderNode) and isinstance(k, PlaceHolderNode)):
             return None
         terms.append((q, k))
-    return {"terms": terms, "scale": scale, "exact": exact, "shift": shift}
+    return {"terms": terms, "scale": scale, "exact": exact, "shift": shift, "norms": norms}
+
+
+def _normed(view, n):
+    """``n`` = ``x * rnorm(x)`` for a graph input x -> ``(x, eps)`` or None."""
+    n = view.skip(n)
+    if not (_is(n, "mul") and n.scalar is None and len(n.inputs) == 2):
+        return None
+    a, b = view.ins(n)
+    for x, rn in ((a, b), (b, a)):
+        if isinstance(x, PlaceHolderNode):
+            hit = _match_rnorm(view, rn)
+            if hit is not None and hit[0] is x:
+                return x, hit[2]
+    return None
 
 
 def _try_attention(view, out):
@@ -394,6 +417,10 @@ def _try_attention(view, out):
     group = math.prod(bq) // units
     prob = {"units": units, "group": group, "sq": sq_[-2], "skv": sk_[-2], "head_dim": sq_[-1],
             "vdim": v.shape[-1], "scale": sc["scale"], "exact": sc["exact"], "shift": sc["shift"]}
+    if sc["norms"]:
+        if view.is_split:
+            raise LoweringRejected("QK-norm attention has no split-KV form here")
+        prob["norm_eps"] = dict(sc["norms"])      # {"q": eps, "k": eps} for the normalised operands
     return "attention", prob, {"Q": q, "K": k, "V": v}
 
 

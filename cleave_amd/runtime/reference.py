@@ -144,6 +144,8 @@ def _eval_matmul_combine(low, feed, out_dtype, out_shape):
 
 def _attn_scores(low, feed):
     """``(scores (units, rows, skv) scaled to the log2 domain, values (units, skv, vdim))``."""
+    import torch
+
     p = low.problem
     if low.family == "mla":
         q, qpe = feed[low.operands["Q"].name].float(), feed[low.operands["QPE"].name].float()
@@ -153,6 +155,11 @@ def _attn_scores(low, feed):
     q = feed[low.operands["Q"].name].float()
     k = feed[low.operands["K"].name].float()
     v = feed[low.operands["V"].name].float()
+    norm = p.get("norm_eps") or {}
+    if "q" in norm:
+        q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + norm["q"])
+    if "k" in norm:
+        k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + norm["k"])
     units, rows = p["units"], p["group"] * p["sq"]
     q = q.reshape(units, rows, p["head_dim"])
     k = k.reshape(units, p["skv"], p["head_dim"])

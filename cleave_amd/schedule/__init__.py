@@ -36,7 +36,13 @@ def _candidates(graph, arch):
         if not policy.attn_ok(low):
             raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "
                                    f"a multiple of 128, got {low.problem['head_dim']}/{low.problem['vdim']}")
-        return policy.attn_candidates(low, role, factor, arch) + policy.attn_many_rows_candidates(low, role, factor, arch)
+        many = policy.attn_many_rows_candidates(low, role, factor, arch)
+        if low.problem.get("norm_eps"):
+            if not many:
+                raise ScheduleRejected("QK-norm attention runs on the many-row kernel only: at least 64 query rows per "
+                                       "unit, widths in 64-feature panels, unsplit")
+            return many
+        return policy.attn_candidates(low, role, factor, arch) + many
     if fam == "mla":
         if not policy.mla_ok(low):
             raise ScheduleRejected("MLA template needs heads % 16 == 0 and widths that are multiples of 32")

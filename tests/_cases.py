@@ -54,6 +54,14 @@ def mla_prefill(q: cl.Tensor["H", "SQ", "DK"], k: cl.Tensor["H", "SKV", "DK"], v
 
 
 @cleave_amd.jit
+def qknorm(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
+    """Grouped-query attention over RMS-normalised queries and keys (the reference's
+    ``demo/qknorm.py`` / ``tests/_graphs.py:542-640``)."""
+    qn, kn = cl.rms_norm(q, dim=-1, eps=1e-6), cl.rms_norm(k, dim=-1, eps=1e-6)
+    return cl.softmax((qn @ kn.mT) / q.shape[-1] ** 0.5, dim=-1) @ v
+
+
+@cleave_amd.jit
 def gqa_decode_shift(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
     n = q.shape[-1] ** 0.5
     return cl.softmax((q @ k.mT) / n, dim=-1, shift=-50 / n) @ v
@@ -117,6 +125,15 @@ def inputs_c3(shapes, seed=3, device="cpu"):
     q = torch.randn(s["HQ"], s["SQ"], s["D"], generator=g)
     k = torch.randn(s["HKV"], s["SKV"], s["D"], generator=g)
     v = torch.randn(s["HKV"], s["SKV"], s["D"], generator=g)
+    return [t.to(torch.float16).to(device) for t in (q, k, v)]
+
+
+def inputs_mla_prefill(shapes, seed=8, device="cpu"):
+    g = _gen(seed)
+    s = shapes
+    q = torch.randn(s["H"], s["SQ"], s["DK"], generator=g)
+    k = torch.randn(s["H"], s["SKV"], s["DK"], generator=g)
+    v = torch.randn(s["H"], s["SKV"], s["DV"], generator=g)
     return [t.to(torch.float16).to(device) for t in (q, k, v)]
 
 

@@ -59,6 +59,37 @@ def test_key_width_differs_from_value_width():
                                    rtol=1e-2, atol=1e-2)
 
 
+def test_qk_norm_attention():
+    """RMSNorm of queries and keys fused into the attention (the reference's ``qknorm`` case,
+    (1, 64, 8, 4096, 4096, 128)): small against the oracle with both, only the keys and only the
+    queries normalised; then the reference's size on a sample of rows."""
+    import cleave_amd
+
+    @cleave_amd.jit
+    def k_only(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
+        return cl.softmax((q @ cl.rms_norm(k, dim=-1, eps=1e-5).mT) * 0.25, dim=-1) @ v
+
+    @cleave_amd.jit
+    def q_only(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
+        return cl.softmax((cl.rms_norm(q, dim=-1) @ k.mT) * 0.25, dim=-1) @ v
+
+    _check(C.qknorm, cl.f16, dict(HQ=8, HKV=2, SQ=100, SKV=300, D=128))
+    _check(C.qknorm, cl.bf16, dict(HQ=4, HKV=4, SQ=70, SKV=45, D=64))
+    _check(k_only, cl.f16, dict(HQ=8, HKV=1, SQ=33, SKV=200, D=128))
+    _check(q_only, cl.f16, dict(HQ=2, HKV=2, SQ=96, SKV=64, D=64))
+    shapes = dict(HQ=64, HKV=8, SQ=4096, SKV=4096, D=128)
+    prog = C.qknorm.trace(cl.f16, **shapes)
+    q, k, v = prog.random_inputs(seed=19)
+    out = kernel_for(prog)(q, k, v)
+    torch.cuda.synchronize()
+    gen = np.random.default_rng(3)
+    norm = lambda x: x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)   # noqa: E731
+    for h, s in zip(gen.integers(0, 64, 32), gen.integers(0, 4096, 32)):
+        w = torch.softmax((norm(k[h // 8].double()) @ norm(q[h, s].double())) / 128 ** 0.5, dim=0)
+        np.testing.assert_allclose(out[h, s].float().cpu().numpy(), (w @ v[h // 8].double()).float().cpu().numpy(),
+                                   rtol=1e-2, atol=1e-2)
+
+
 def test_search_prefers_the_shared_kernel_for_many_rows_and_keeps_decode_for_few():
     from cleave_amd.schedule import search_tiling
 

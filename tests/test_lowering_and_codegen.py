@@ -121,6 +121,18 @@ def test_matmul_rowsum_is_a_family_of_its_own():
         split_stages(g, 2)
 
 
+def test_qk_norm_attention_is_attention_with_normalised_operands():
+    g = stage_graph(C.qknorm.trace(cl.f16, HQ=64, HKV=8, SQ=4096, SKV=4096, D=128))
+    low = g.lowered
+    assert low.family == "attention" and low.problem["norm_eps"] == {"q": pytest.approx(1e-6), "k": pytest.approx(1e-6)}
+    assert (low.problem["units"], low.problem["group"]) == (8, 8)
+    assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}     # the streaming kernel has no norm form
+    with pytest.raises(ScheduleRejected, match="many-row kernel"):
+        search_tiling(stage_graph(C.qknorm.trace(cl.f16, HQ=4, HKV=4, SQ=1, SKV=256, D=128)))
+    m = parse_manifest(source_for(C.qknorm.trace(cl.f16, HQ=64, HKV=8, SQ=4096, SKV=4096, D=128)))
+    assert m["launches"][0]["grid"] == ["256", "8", "1"] and m["launches"][0]["block"][0] == 256
+
+
 def test_unrecognised_program_is_refused():
     from cleave_amd.frontend import Program
 
