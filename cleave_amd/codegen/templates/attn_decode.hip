@@ -38,7 +38,7 @@ struct AttUnit {
   const elem_t* q;      // first query row of this tile (row stride CL_HEAD_DIM)
   const elem_t* k;      // dense: first K row of the unit; paged: cache base + head offset
   const elem_t* v;
-  i64 row_stride;       // elements between consecutive tokens
+  i64 k_stride, v_stride;   // elements between consecutive tokens of K and of V (their widths may differ)
   int kv_len;           // valid tokens
   int rows;             // real rows in this tile (1..16)
   const int* pages;     // paged: this request's slice of the page table
@@ -52,24 +52,24 @@ struct AttUnit {
 // An item's page ids were read once into one register per lane; a token's page id comes from
 // the lane that holds it.  A page-table load per token would sit in the same in-order load
 // queue as the K/V rows and make every prefetch wait for the rows of the step before it.
-CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) {
+CL_DEVICE i64 att_token_row(const AttUnit& u, int t) {
   int pi = t / CL_PAGE_SIZE;
   pi = pi < u.n_pages ? pi : u.n_pages - 1;
   const i64 page = __builtin_amdgcn_ds_bpermute(pi << 2, u.page_reg);
-  return (page * CL_PAGE_SIZE + (t % CL_PAGE_SIZE)) * u.row_stride;
+  return page * CL_PAGE_SIZE + (t % CL_PAGE_SIZE);
 }
 #elif CL_PAGED
-CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) {
+CL_DEVICE i64 att_token_row(const AttUnit& u, int t) {
   int pi = t / CL_PAGE_SIZE;
   pi = pi < u.n_pages ? pi : u.n_pages - 1;
   int pid = u.pages[pi];
   pid = pid < u.pool_pages - 1 ? pid : u.pool_pages - 1;
   pid = pid > 0 ? pid : 0;
   const i64 page = pid;
-  return (page * CL_PAGE_SIZE + (t % CL_PAGE_SIZE)) * u.row_stride;
+  return page * CL_PAGE_SIZE + (t % CL_PAGE_SIZE);
 }
 #else
-CL_DEVICE i64 att_token_offset(const AttUnit& u, int t) { return (i64)t * u.row_stride; }
+CL_DEVICE i64 att_token_row(const AttUnit& u, int t) { (void)u; return (i64)t; }
 #endif
 
 struct AttTile {               // one 32-token step's K and V, as loaded
@@ -85,7 +85,7 @@ CL_DEVICE void att_load(const AttUnit& u, int t0, int c, int g, AttTile& tile) {
   for (int h = 0; h < 2; ++h) {
     int t = t0 + 16 * h + c;
     t = t < last ? t : last;
-    const elem_t* row = u.k + att_token_offset(u, t) + 8 * g;
+    const elem_t* row = u.k + att_token_row(u, t) * u.k_stride + 8 * g;
 #pragma unroll
     for (int j = 0; j < ATT_KJ; ++j) tile.k[h][j] = ld16(row + 32 * j);
   }
@@ -93,7 +93,7 @@ CL_DEVICE void att_load(const AttUnit& u, int t0, int c, int g, AttTile& tile) {
   for (int e = 0; e < 8; ++e) {
     int t = t0 + (e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4));
     t = t < last ? t : last;
-    const elem_t* row = u.v + att_token_offset(u, t);
+    const elem_t* row = u.v + att_token_row(u, t) * u.v_stride;
 #pragma unroll
     for (int vc = 0; vc < ATT_VC; ++vc) {
       int col = 128 * vc + 8 * c;
@@ -154,7 +154,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     pid = pid < num_pages - 1 ? pid : num_pages - 1;
     u.page_reg = pid > 0 ? pid : 0;
   }
-  u.row_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
+  u.k_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
+  u.v_stride = (i64)CL_KV_HEADS * CL_VDIM;
   u.k = CL_ARG_K + (i64)head * CL_HEAD_DIM;
   u.v = CL_ARG_V + (i64)head * CL_VDIM;
   u.out_row = (i64)req * CL_Q_HEADS + (i64)head * CL_ROWS;
@@ -186,7 +187,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   u.page_reg = 0;
   u.n_pages = n_pages;
   u.pool_pages = num_pages;
-  u.row_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
+  u.k_stride = (i64)CL_KV_HEADS * CL_HEAD_DIM;
+  u.v_stride = (i64)CL_KV_HEADS * CL_VDIM;
   u.k = CL_ARG_K + (i64)head * CL_HEAD_DIM;
   u.v = CL_ARG_V + (i64)head * CL_VDIM;
   u.out_row = ((i64)req * CL_Q_HEADS + (i64)head * CL_ROWS) + 16 * tile_id;
@@ -198,7 +200,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   u.pages = nullptr;
   u.n_pages = 0;
   u.pool_pages = 0;
-  u.row_stride = CL_HEAD_DIM;
+  u.k_stride = CL_HEAD_DIM;
+  u.v_stride = CL_VDIM;
   u.k = CL_ARG_K + (i64)unit * CL_SKV * CL_HEAD_DIM;
   u.v = CL_ARG_V + (i64)unit * CL_SKV * CL_VDIM;
   u.out_row = (i64)unit * CL_ROWS + 16 * tile_id;

@@ -90,6 +90,20 @@ def test_qk_norm_attention():
                                    rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("waves", [1, 2, 4])
+def test_streaming_kernel_strides_keys_and_values_by_their_own_widths(waves):
+    """The streaming (decode) kernel on operands whose key width is not the value width: K rows
+    are 192 or 64 elements apart, V rows 128.  (It once walked V with the key stride.)"""
+    for shapes in (dict(H=3, SQ=20, SKV=150, DK=192, DV=128), dict(H=2, SQ=5, SKV=70, DK=64, DV=128)):
+        prog = C.mla_prefill.trace(cl.f16, **shapes)
+        args = prog.random_inputs(seed=23)
+        print(f"streaming kernel, widths {shapes['DK']}/{shapes['DV']}, waves {waves}: {shapes}", flush=True)
+        out = kernel_for(prog, template="attn_decode", tiling=dict(WAVES=waves))(*args)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(out.float().cpu().numpy(), program_oracle.evaluate(prog, list(args))[0],
+                                   rtol=1e-2, atol=1e-2)
+
+
 def test_search_prefers_the_shared_kernel_for_many_rows_and_keeps_decode_for_few():
     from cleave_amd.schedule import search_tiling
 
