@@ -77,6 +77,10 @@ def op_table():
                       inputs=C.inputs_mla_prefill, split=False,
                       bytes=2 * 128 * 4096 * (192 + 128 + 192 + 128), flops=2 * 128 * 4096 * 4096 * (192 + 128),
                       bound="mfma", sets=2, cpu=False),
+        "lora": dict(title="LoRA f16 x@w + (x@a)@b M=16 N=4096 K=4096 R=16", fn=C.lora, dtype=cl.f16,
+                     shapes=C.FULL["lora"], inputs=C.inputs_lora, split=False,
+                     bytes=2 * (16 * 4096 + 4096 * 4096 + 4096 * 16 + 16 * 4096 + 16 * 4096),
+                     flops=2 * 16 * 4096 * 4096 + 2 * 16 * 4096 * 16 * 2, bound="hbm", sets=6),
         "mmrs": dict(title="matmul + row sum f16 (x@w).sum(-1) 4096x4096x64", fn=C.matmul_rowsum, dtype=cl.f16,
                      shapes=C.FULL["matmul_rowsum"], inputs=C.inputs_c1, split=False,
                      bytes=2 * (4096 * 64 + 64 * 4096 + 4096), flops=2 * 4096 * 4096 * 64, bound="mfma", sets=4),
@@ -400,7 +404,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,mmrs,attn,qknorm,mlapf")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,lora,mmrs,attn,qknorm,mlapf")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")

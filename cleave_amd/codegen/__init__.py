@@ -196,7 +196,8 @@ class HipCodeGen:
                 unit.define("CL_ARG_PACC", op["PACC"])
                 if norm:
                     unit.define("CL_ARG_PSS", op["PSS"])
-            for role, macro in (("A", "CL_ARG_A"), ("B", "CL_ARG_B"), ("C", "CL_ARG_C"), ("GAMMA", "CL_ARG_GAMMA")):
+            for role, macro in (("A", "CL_ARG_A"), ("B", "CL_ARG_B"), ("C", "CL_ARG_C"), ("GAMMA", "CL_ARG_GAMMA"),
+                                ("LA", "CL_ARG_LA"), ("LB", "CL_ARG_LB")):
                 if role in op:
                     unit.define(macro, op[role])
             unit.define("CL_ARG_X", op["A"])
@@ -289,13 +290,22 @@ class HipCodeGen:
             unit.define(f"CL_{k}", v)
         unit.templates.append("skinny_matmul.hip")
         splits = plan.split_factor or 1
+        lora = plan.family == "lora"
+        if lora != bool(tile.get("LORA")) or (lora and (splits > 1 or combine)):
+            raise CodegenError("LoRA is the LORA tiling of the few-row matmul, unsplit")
+        if lora:
+            if p["R"] % 8 or p["R"] > 64:
+                raise CodegenError("LoRA rank must be a multiple of 8 up to 64")
+            unit.define("CL_R", p["R"])
         if partial:
-            from ..schedule.policy import skinny_lds_bytes
+            from ..schedule.policy import lora_lds_bytes, skinny_lds_bytes
 
             if p["M"] > 64 or p["K"] % 32 or p["N"] % 8:
                 raise CodegenError("the few-row matmul template needs M <= 64, K % 32 == 0, N % 8 == 0")
             grid = (-(-p["N"] // (128 * tile["WAVES_N"])), splits, 1)
             lds = skinny_lds_bytes(-(-p["M"] // 16), tile["WAVES_N"], tile["WAVES_K"])
+            if lora:
+                lds = lora_lds_bytes(-(-p["M"] // 16), tile["WAVES_N"], tile["WAVES_K"], p["R"])
             unit.launch(ENTRY, grid, tile["WAVES_N"] * tile["WAVES_K"] * 64, lds, self._partial_args)
         if combine:
             entry, args, blocks = self._combine_args

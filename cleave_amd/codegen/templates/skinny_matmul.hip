@@ -18,6 +18,14 @@
 //   CL_NORM            0 plain, 1 RMSNorm epilogue; CL_GAMMA: 1 when a (K) weight multiplies X
 //   CL_EPS             epsilon inside the rsqrt
 //   CL_PREFETCH        steps of loads in flight ahead of the one being computed (1..3)
+//
+// CL_LORA: Y = X * W + (X * LA) * LB with LA (K, CL_R) and LB (CL_R, N), unsplit.  The rank-R
+// product D = X * LA rides along: the lanes of the first CL_R / 8 column groups load their 8x8
+// blocks of LA with the W blocks (same ring, same transpose, eight more MFMAs per step into a
+// second accumulator set of which only those column groups mean anything), D is reduced over the
+// K-sharing waves with the main accumulators, rounded to the element type like the input of the
+// reference's second product, parked in LDS, and the epilogue adds D * LB to each lane's outputs
+// with plain multiply-adds (CL_R per output).
 
 #define SK_MT ((CL_M + 15) / 16)
 #define SK_COLS 128
@@ -26,6 +34,12 @@
 
 #ifndef CL_PREFETCH
 #define CL_PREFETCH 2
+#endif
+#ifndef CL_LORA
+#define CL_LORA 0
+#endif
+#if CL_LORA
+static_assert(CL_R % 8 == 0 && CL_R <= 128 && CL_SPLITS == 1 && !CL_NORM, "LoRA: rank in whole 8-column blocks, unsplit");
 #endif
 // Everything one 32-row step needs, as loaded: the lane's 8x8 block of W, its X fragments
 // (lane (c, g) holds X[16 mt + c][k0 + 8 g .. +8]) and the matching gamma chunk.  X and gamma
@@ -37,10 +51,13 @@ struct SkTile {
 #if CL_NORM && CL_GAMMA
   u32x4 gm;
 #endif
+#if CL_LORA
+  u32x4 la[8];
+#endif
 };
 
 CL_DEVICE void sk_load(const elem_t* __restrict__ W, const elem_t* __restrict__ X, const elem_t* __restrict__ G,
-                       int k0, int ncol, int c, int g, SkTile& t) {
+                       const elem_t* __restrict__ LA, int k0, int ncol, int c, int g, SkTile& t) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) t.w[e] = ld16(W + (i64)(k0 + 8 * g + e) * CL_N + ncol);
 #pragma unroll
@@ -52,6 +69,13 @@ CL_DEVICE void sk_load(const elem_t* __restrict__ W, const elem_t* __restrict__ 
   t.gm = ld16(G + k0 + 8 * g);
 #else
   (void)G;
+#endif
+#if CL_LORA
+#pragma unroll
+  for (int e = 0; e < 8; ++e)   // (only the lanes of the first CL_R / 8 column groups fetch anything)
+    t.la[e] = 8 * c < CL_R ? ld16(LA + (i64)(k0 + 8 * g + e) * CL_R + 8 * c) : (u32x4){0u, 0u, 0u, 0u};
+#else
+  (void)LA;
 #endif
 }
 
@@ -90,6 +114,13 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   float ss[SK_MT];
 #pragma unroll
   for (int mt = 0; mt < SK_MT; ++mt) ss[mt] = 0.f;
+#if CL_LORA
+  f32x4 dacc[SK_MT][8];        // dacc[mt][j][r] = D[16 mt + 4 g + r][8 c + j] in the lanes with 8 c < CL_R
+#pragma unroll
+  for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dacc[mt][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#endif
 
   // Ring of CL_PREFETCH + 1 register tiles: while step n is in the matrix cores the loads of
   // steps n+1 .. n+CL_PREFETCH are in flight.
@@ -97,6 +128,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const elem_t* gamma_ptr = CL_ARG_GAMMA;
 #else
   const elem_t* gamma_ptr = nullptr;
+#endif
+#if CL_LORA
+  const elem_t* la_ptr = CL_ARG_LA;
+#else
+  const elem_t* la_ptr = nullptr;
 #endif
   SkTile ring[CL_PREFETCH + 1];
   // one step on the tile `cur`: row sums of squares, gamma, 8x8 transpose of W, eight MFMAs per row tile
@@ -115,7 +151,20 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     _Pragma("unroll") for (int j = 0; j < 8; ++j)                                         \
       _Pragma("unroll") for (int mt = 0; mt < SK_MT; ++mt)                                \
         acc[mt][j] = mfma16(xa[mt], as_elem8(wt[j]), acc[mt][j]);                         \
+    SK_LORA_STEP(cur)                                                                     \
   }
+#if CL_LORA
+#define SK_LORA_STEP(cur)                                                                 \
+    {                                                                                     \
+      u32x4 lt[8];                                                                        \
+      transpose8x8((cur).la, lt);                                                         \
+      _Pragma("unroll") for (int j = 0; j < 8; ++j)                                       \
+        _Pragma("unroll") for (int mt = 0; mt < SK_MT; ++mt)                              \
+          dacc[mt][j] = mfma16(xa[mt], as_elem8(lt[j]), dacc[mt][j]);                     \
+    }
+#else
+#define SK_LORA_STEP(cur)
+#endif
 #if CL_NORM
 #if CL_GAMMA
 #define SK_GAMMA_X(x, cur)                                                                \
@@ -141,11 +190,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // load issued CL_PREFETCH steps ahead of its use and none past the end
 #pragma unroll
     for (int i = 0; i < CL_PREFETCH && i < steps_per_wave; ++i)
-      sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, (s_begin + i) * SK_STEP, ncol, c, g, ring[i % (CL_PREFETCH + 1)]);
+      sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, la_ptr, (s_begin + i) * SK_STEP, ncol, c, g, ring[i % (CL_PREFETCH + 1)]);
 #pragma unroll
     for (int i = 0; i < steps_per_wave; ++i) {
       if (i + CL_PREFETCH < steps_per_wave)
-        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, (s_begin + i + CL_PREFETCH) * SK_STEP, ncol, c, g,
+        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, la_ptr, (s_begin + i + CL_PREFETCH) * SK_STEP, ncol, c, g,
                 ring[(i + CL_PREFETCH) % (CL_PREFETCH + 1)]);
       SK_CONSUME(ring[i % (CL_PREFETCH + 1)])
     }
@@ -159,7 +208,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int i = 0; i < CL_PREFETCH; ++i) {
         int sidx = s_begin + i;
         sidx = sidx < last_step ? sidx : last_step;
-        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, sidx * SK_STEP, ncol, c, g, ring[i]);
+        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, la_ptr, sidx * SK_STEP, ncol, c, g, ring[i]);
       }
     }
     for (int base = s_begin; base < s_end; base += CL_PREFETCH + 1) {
@@ -169,7 +218,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         if (s >= s_end) break;
         int ahead = s + CL_PREFETCH;
         ahead = ahead < last_step ? ahead : last_step;
-        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, ahead * SK_STEP, ncol, c, g, ring[(r + CL_PREFETCH) % (CL_PREFETCH + 1)]);
+        sk_load(CL_ARG_W, CL_ARG_X, gamma_ptr, la_ptr, ahead * SK_STEP, ncol, c, g, ring[(r + CL_PREFETCH) % (CL_PREFETCH + 1)]);
         SK_CONSUME(ring[r])
       }
     }
@@ -187,6 +236,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   extern __shared__ float sk_lds[];
   float* sh_acc = sk_lds;                                     // [WAVES_K-1][WAVES_N][MT*8*4][64]
   float* sh_ss = sk_lds + (CL_WAVES_K - 1) * CL_WAVES_N * SK_MT * 32 * 64;  // [WAVES_K][MT*16]
+#if CL_LORA
+  float* sh_dacc = sh_ss + CL_WAVES_K * SK_MT * 16 + 4;       // like sh_acc, for the rank-R accumulators
+  float* sh_d = sh_dacc + (CL_WAVES_K - 1) * CL_WAVES_N * SK_MT * 32 * 64;  // [WAVES_N][16 MT][CL_R]
+#endif
 #if CL_WAVES_K > 1
   if (wk > 0) {
     float* dst = sh_acc + ((i64)((wk - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
@@ -196,6 +249,15 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int j = 0; j < 8; ++j)
 #pragma unroll
         for (int r = 0; r < 4; ++r) dst[((mt * 8 + j) * 4 + r) * 64 + lane] = acc[mt][j][r];
+#if CL_LORA
+    float* ddst = sh_dacc + ((i64)((wk - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ddst[((mt * 8 + j) * 4 + r) * 64 + lane] = dacc[mt][j][r];
+#endif
   }
 #endif
 #if CL_NORM
@@ -205,17 +267,56 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 #endif
   __syncthreads();
+#if !CL_LORA
   if (wk != 0) return;
+#endif
 #if CL_WAVES_K > 1
+  if (wk == 0) {
 #pragma unroll
-  for (int w = 1; w < CL_WAVES_K; ++w) {
-    const float* src = sh_acc + ((i64)((w - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
+    for (int w = 1; w < CL_WAVES_K; ++w) {
+      const float* src = sh_acc + ((i64)((w - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
+#pragma unroll
+      for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[mt][j][r] += src[((mt * 8 + j) * 4 + r) * 64 + lane];
+#if CL_LORA
+      const float* dsrc = sh_dacc + ((i64)((w - 1) * CL_WAVES_N + wn) * SK_MT * 32) * 64;
+#pragma unroll
+      for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) dacc[mt][j][r] += dsrc[((mt * 8 + j) * 4 + r) * 64 + lane];
+#endif
+    }
+  }
+#endif
+#if CL_LORA
+  // D (rounded to the element type, as the input of a second product is) goes to LDS for this
+  // wave's epilogue; the workgroup-wide barrier is the simplest fence between its lanes
+  if (wk == 0 && 8 * c < CL_R) {
 #pragma unroll
     for (int mt = 0; mt < SK_MT; ++mt)
 #pragma unroll
       for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[mt][j][r] += src[((mt * 8 + j) * 4 + r) * 64 + lane];
+        for (int r = 0; r < 4; ++r)
+          sh_d[((wn * SK_MT + mt) * 16 + 4 * g + r) * CL_R + 8 * c + j] = to_f32(to_elem(dacc[mt][j][r]));
+  }
+  __syncthreads();
+  if (wk != 0) return;
+  for (int rr = 0; rr < CL_R; ++rr) {
+    const elem8 bv = as_elem8(ld16(CL_ARG_LB + (i64)rr * CL_N + ncol));
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float d = sh_d[((wn * SK_MT + mt) * 16 + 4 * g + r) * CL_R + rr];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[mt][j][r] += d * to_f32(bv[j]);
+      }
   }
 #endif
 

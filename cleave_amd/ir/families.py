@@ -31,7 +31,7 @@ from .graph import ComputeOpNode, Graph, Node, OutputNode, PlaceHolderNode
 class Lowered:
     """A recognised operator: family, sizes and which placeholder plays which operand."""
 
-    family: str                       # matmul | rmsnorm_matmul | swiglu | matmul_rowsum | attention | mla
+    family: str                       # matmul | rmsnorm_matmul | swiglu | lora | matmul_rowsum | attention | mla
     problem: dict                     # sizes and flags the template needs
     operands: dict                    # role -> PlaceHolderNode
     outputs: list                     # OutputNodes in order
@@ -246,6 +246,35 @@ def _try_matmul_rowsum(view, out):
     return "matmul_rowsum", prob, {"A": a, "B": b}
 
 
+def _try_lora(view, out):
+    """``x @ w + (x @ la) @ lb``: a base product plus a rank-R update through a shared activation
+    (the reference's ``tests/_graphs.py:438-480``): operands A (x), B (w), LA (K, R), LB (R, N)."""
+    n = view.skip(out)
+    if not (_is(n, "add") and n.scalar is None and len(n.inputs) == 2):
+        return None
+    for base, up in (view.ins(n), view.ins(n)[::-1]):
+        if not (_is(base, "matmul") and _is(up, "matmul")):
+            continue
+        down, lb = view.ins(up)
+        if not _is(down, "matmul"):
+            continue
+        (x, w), (x2, la) = view.ins(base), view.ins(down)
+        if x is not x2 or not all(isinstance(t, PlaceHolderNode) for t in (x, w, la, lb)):
+            continue
+        if any(m.attrs["trans_A"] or m.attrs["trans_B"] for m in (base, up, down)):
+            raise LoweringRejected("LoRA is built for row-major operands: x (M, K), w (K, N), a (K, R), b (R, N)")
+        if view.is_split:
+            raise LoweringRejected("LoRA has no split-K form here")
+        prob = _matmul_problem(x, w, False, False)
+        if prob["batch_A"] != 1 or prob["batch_B"] != 1 or len(la.shape) != 2 or len(lb.shape) != 2:
+            raise LoweringRejected("LoRA is built for 2-D operands")
+        if la.shape != (prob["K"], lb.shape[0]) or lb.shape[1] != prob["N"]:
+            raise LoweringRejected(f"LoRA factors do not line up: a {tuple(la.shape)}, b {tuple(lb.shape)}")
+        prob["R"] = int(lb.shape[0])
+        return "lora", prob, {"A": x, "B": w, "LA": la, "LB": lb}
+    return None
+
+
 def _matmul_problem(a, b, trans_a, trans_b) -> dict:
     sa, sb = tuple(a.shape), tuple(b.shape)
     if len(sa) != len(sb) or len(sa) < 2:
@@ -424,7 +453,7 @@ def _try_attention(view, out):
     return "attention", prob, {"Q": q, "K": k, "V": v}
 
 
-_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_matmul_rowsum, _try_attention, _try_matmul)
+_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_lora, _try_matmul_rowsum, _try_attention, _try_matmul)
 
 
 def recognize(graph: Graph) -> Lowered:
@@ -446,7 +475,7 @@ def recognize(graph: Graph) -> Lowered:
                 _check_split_axes(family, operands, view.split_axes)
             return Lowered(family, problem, operands, outs, graph, dict(view.split_axes), split_dim)
     raise LoweringRejected(f"{graph.name}: ops {graph.op_kinds()} match no kernel family "
-                           "(matmul, rmsnorm_matmul, swiglu, matmul_rowsum, attention, mla)")
+                           "(matmul, rmsnorm_matmul, swiglu, lora, matmul_rowsum, attention, mla)")
 
 
 def _check_split_axes(family, operands, split_axes):

@@ -69,9 +69,9 @@ def make_inputs(graph, dtype=None, device: str = "cuda", seed: int | None = None
         else:
             x = torch.randn(tuple(ph.shape), generator=gen)
             low = getattr(graph, "lowered", None)
-            if low is not None and low.family in ("matmul", "rmsnorm_matmul", "swiglu", "matmul_rowsum") and getattr(graph, "role", "main") != "combine":
+            if low is not None and low.family in ("matmul", "rmsnorm_matmul", "swiglu", "matmul_rowsum", "lora") and getattr(graph, "role", "main") != "combine":
                 role = next((r for r, n in low.operands.items() if n is ph), None)
-                if role in ("B", "C"):
+                if role in ("B", "C", "LA"):
                     x = x / math.sqrt(low.problem["K"])  # keep products O(1) so tolerances mean something
         made.append(x.to(dtype=torch_dtype(ph.dtype), device=device))
     return made
@@ -220,6 +220,12 @@ def execute(graph, inputs, device=None) -> list:
         return [r.reshape(s) for r, s in zip(res, shapes)]
     if low.family == "swiglu":
         return [r.reshape(s) for r, s in zip(_eval_swiglu(low, feed, out_dtype), shapes)]
+    if low.family == "lora":
+        # x @ w + (x @ a) @ b, the down product rounded to the storage type before the up product
+        a, b = _mm_operands(low, feed)
+        la, lb = feed[low.operands["LA"].name].float(), feed[low.operands["LB"].name].float()
+        down = (a @ la).to(torch_dtype(graph.dtype)).float()
+        return [(a @ b + down @ lb).to(out_dtype).reshape(shapes[0])]
     if low.family == "matmul_rowsum":
         a, b = _mm_operands(low, feed)
         return [(a @ b).sum(-1).to(out_dtype).reshape(shapes[0])]

@@ -32,6 +32,12 @@ def _candidates(graph, arch):
         return policy.swiglu_candidates(low, role, factor, arch)
     if fam == "matmul_rowsum":
         return policy.rowsum_candidates(low, role, factor, arch)
+    if fam == "lora":
+        cands = policy.lora_candidates(low, role, factor, arch)
+        if not cands:
+            raise ScheduleRejected("LoRA runs on the few-row matmul kernel only: M <= 64, K % 32 == 0, N % 8 == 0, "
+                                   "rank a multiple of 8 up to 64, unsplit")
+        return cands
     if fam == "attention":
         if not policy.attn_ok(low):
             raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "

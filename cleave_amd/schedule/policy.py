@@ -211,6 +211,38 @@ def rowsum_candidates(low, role, factor, arch: Arch):
     return out
 
 
+def lora_lds_bytes(mt, waves_n, waves_k, rank):
+    """The few-row kernel's reduction buffers twice (main and rank-R accumulators) plus the D tile."""
+    return 2 * skinny_lds_bytes(mt, waves_n, waves_k) + waves_n * 16 * mt * rank * 4 + 16
+
+
+def lora_candidates(low, role, factor, arch: Arch):
+    """LoRA: the few-row matmul with the rank-R product riding along (unsplit: the rank update needs
+    the whole of ``x @ a``)."""
+    import copy
+
+    p = low.problem
+    if (factor or 1) > 1 or p["R"] % 8 or p["R"] > 64:
+        return []
+    twin = copy.copy(low)
+    twin.family = "matmul"
+    if not skinny_ok(twin):
+        return []
+    out = []
+    for c in skinny_candidates(twin, role, None, arch):
+        t = c.tiling
+        lds = lora_lds_bytes(_ceil(p["M"], 16), t["WAVES_N"], t["WAVES_K"], p["R"])
+        if lds > arch.lds_bytes:
+            continue
+        c.tiling, c.lds_bytes = dict(t, LORA=1), lds
+        if t["WAVES_N"] * t["WAVES_K"] > 4:
+            # more than four waves have 256 registers each: the ring of tiles (each now carries a block
+            # of the rank-R factor too) is one tile shallower so that nothing spills
+            c.tiling["PREFETCH"] = 1
+        out.append(c)
+    return out
+
+
 # ----------------------------------------------------------------------------- few-row matmul
 def skinny_ok(low) -> bool:
     p = low.problem

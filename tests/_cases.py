@@ -36,6 +36,12 @@ def swiglu(x: cl.Tensor["M", "K"], w_up: cl.Tensor["K", "N"], w_gate: cl.Tensor[
 
 
 @cleave_amd.jit
+def lora(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"], a: cl.Tensor["K", "R"], b: cl.Tensor["R", "N"]):
+    """``x @ w + (x @ a) @ b`` (the reference's ``demo/lora.py`` / ``tests/_graphs.py:438-480``)."""
+    return x @ w + (x @ a) @ b
+
+
+@cleave_amd.jit
 def matmul_rowsum(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
     """Row sums of a product that is never stored (the reference's ``tests/_graphs.py:150-160``)."""
     return (x @ w).sum(dim=-1, keepdim=True)
@@ -81,6 +87,7 @@ FULL = {
     "c4": dict(B=16, H=128, D=512, PE=64, SKV=4096),
     "swiglu": dict(M=4096, N=14336, K=4096),
     "matmul_rowsum": dict(M=4096, N=4096, K=64),
+    "lora": dict(M=16, N=4096, K=4096, R=16),
 }
 SMALL = {
     "c1": dict(M=32, N=64, K=256),
@@ -108,6 +115,16 @@ def inputs_swiglu(shapes, seed=6, device="cpu"):
     x = torch.randn(M, K, generator=g)
     ws = [torch.randn(K, N, generator=g) / math.sqrt(K) for _ in range(2)]
     return [t.to(torch.float16).to(device) for t in (x, *ws)]
+
+
+def inputs_lora(shapes, seed=9, device="cpu"):
+    g = _gen(seed)
+    M, N, K, R = shapes["M"], shapes["N"], shapes["K"], shapes["R"]
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(K, N, generator=g) / math.sqrt(K)
+    a = torch.randn(K, R, generator=g) / math.sqrt(K)
+    b = torch.randn(R, N, generator=g) / math.sqrt(R)
+    return [t.to(torch.float16).to(device) for t in (x, w, a, b)]
 
 
 def inputs_c2(shapes, seed=2, device="cpu"):

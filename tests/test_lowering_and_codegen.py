@@ -133,6 +133,23 @@ def test_qk_norm_attention_is_attention_with_normalised_operands():
     assert m["launches"][0]["grid"] == ["256", "8", "1"] and m["launches"][0]["block"][0] == 256
 
 
+def test_lora_is_a_family_of_its_own():
+    g = stage_graph(C.lora.trace(cl.f16, **C.FULL["lora"]))
+    low = g.lowered
+    assert low.family == "lora" and low.problem["R"] == 16
+    assert {r: n.name for r, n in low.operands.items()} == {"A": "PlaceHolder_x", "B": "PlaceHolder_w",
+                                                            "LA": "PlaceHolder_a", "LB": "PlaceHolder_b"}
+    cands = search_tiling(g, topk=100)
+    assert cands and all(c.template == "skinny" and c.tiling["LORA"] == 1 for c in cands)
+    m = parse_manifest(source_for(C.lora.trace(cl.f16, **C.FULL["lora"])))
+    assert [p["name"] for p in m["params"]] == ["PlaceHolder_x", "PlaceHolder_w", "PlaceHolder_a", "PlaceHolder_b",
+                                                 "OutputNode_0"]
+    with pytest.raises(ScheduleRejected, match="few-row matmul kernel only"):
+        search_tiling(stage_graph(C.lora.trace(cl.f16, M=256, N=512, K=512, R=16)))
+    with pytest.raises(LoweringRejected, match="no split form"):
+        split_stages(g, 4)
+
+
 def test_unrecognised_program_is_refused():
     from cleave_amd.frontend import Program
 
