@@ -34,6 +34,9 @@
 // registers); the lanes on the diagonal take the reciprocal root and the lanes of each score
 // fetch the factor of its key.
 //
+// CL_PF_XCD / CL_PF_REVERSE (default 1) switch the XCD mapping and the walking order; the
+// CL_PF_DBG_* switches leave parts of the kernel out for measurement (wrong results by design).
+//
 //   CL_HEAD_DIM (multiple of 64)  CL_KV_HEADS  CL_Q_HEADS (group divides 16)  CL_RAGGED
 //   run-time: batch, total_q, n_idx (table length / total_kv), num_pages (table form), sm_scale
 
