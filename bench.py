@@ -52,7 +52,7 @@ def op_table():
                    shapes=C.FULL["c2"], inputs=C.inputs_c2, split=cl.Split("K", (2, 4, 8, 16)), bytes=90_669_056,
                    flops=1_442_840_576, bound="hbm", sets=6),
         "c3": dict(title="GQA decode f16 B=8 Hq=32 Hkv=8 D=128 SKV=8192 exact softmax", fn=C.gqa_decode_exact,
-                   dtype=cl.f16, shapes=C.FULL["c3"], inputs=C.inputs_c3, split=cl.Split("SKV", (8, 16, 32)),
+                   dtype=cl.f16, shapes=C.FULL["c3"], inputs=C.inputs_c3, split=cl.Split("SKV", (4, 8, 16)),
                    bytes=268_566_528, flops=1_073_741_824, bound="hbm", sets=3),
         "c4": dict(title="MLA decode bf16 B=16 H=128 512+64 SKV=4096", fn=C.mla_decode, dtype=cl.bf16,
                    shapes=C.FULL["c4"], inputs=C.inputs_c4, split=cl.Split("SKV", (2, 4, 8, 16)), bytes=79_953_920,

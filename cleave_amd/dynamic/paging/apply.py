@@ -105,7 +105,7 @@ def read_dense_attention(plan: KernelPlan) -> DenseAttention:
     waves = int(plan.tiling.get("WAVES", 4))
     return DenseAttention(query_rows=-(-rows // 16) * 16, kv_tile=KV_STEP, head_dim=p["head_dim"],
                           n_threads=waves * 64, dtype=plan.dtype, out_dtype=plan.dtype, waves=waves,
-                          split=plan.split_factor)
+                          split=plan.split_factor, prefetch=int(plan.tiling.get("PREFETCH", 1)))
 
 
 def read_dense_partial(plan: KernelPlan):

@@ -336,6 +336,12 @@ def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
         tiling = dict(WAVES=waves)
         out.append(TileDict("attn_decode", role, tiling, output_tile=[16, vd], rstep_map={"kv": 32},
                             n_threads=waves * 64, split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+        # a second step of loads in flight (measured on the 8192-key decode: with about two waves per CU
+        # streaming, the deeper ring is worth a few percent; with many waves it is not)
+        if waves <= 2 and vgprs + kv_regs <= arch.vgprs_per_lane and steps_per_wave >= 8:
+            out.append(TileDict("attn_decode", role, dict(WAVES=waves, PREFETCH=2), output_tile=[16, vd],
+                                rstep_map={"kv": 32}, n_threads=waves * 64, split_factor=factor, score=score * 1.001,
+                                lds_bytes=lds, est_vgprs=vgprs + kv_regs))
     return out
 
 
