@@ -43,14 +43,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int c = lane & 15, g = lane >> 4;
   const int item = blockIdx.x;
   // the request whose items include `item`: the last b with b + qo_indptr[b] / PF_TOK <= item
-  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, PF_TOK, 1, item, lane);
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, PF_TOK, 1, item, lane, CL_ARG_INDPTR, n_idx);
   const int req = found.req, q0 = found.p0, q1 = found.p1;
   const int chunk = item - req;
   const int lo = q0 > chunk * PF_TOK ? q0 : chunk * PF_TOK;
   const int hi = q1 < (chunk + 1) * PF_TOK ? q1 : (chunk + 1) * PF_TOK;
   if (hi <= lo) return;                                 // an index no (chunk, request) pair maps to
-  const int kv0 = pf_clamp(CL_ARG_INDPTR[req], 0, n_idx);
-  int kv_len = pf_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx) - kv0;
+  const int kv0 = found.s0;
+  int kv_len = found.s1 - kv0;
   kv_len = kv_len > 0 ? kv_len : 0;
   const int off = kv_len - (q1 - q0);                   // key position of the request's first query row
   const int n_rows = (hi - lo) * PF_GROUP;

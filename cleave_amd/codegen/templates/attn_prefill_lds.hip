@@ -154,33 +154,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   auto row_index = [&](int m) __attribute__((always_inline)) { return (i64)head * CL_ROWS + lo + m; };
   auto row_limit = [&](int m) __attribute__((always_inline)) { (void)m; return CL_SKV - 1; };
 #else
-  // The request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item.
-  // The condition holds for every request up to that one, so the lanes test 64 requests at a time
-  // and count (one round trip to memory per 64 requests instead of one per halving); with up to
-  // 63 requests the row pointers the item needs are already in the lanes.
-  int req, q0, q1, kv0, kv1;
-  {
-    const int b0 = lane < batch ? lane : batch;
-    const int qp0 = pl_clamp(CL_ARG_QINDPTR[b0], 0, total_q), kp0 = pl_clamp(CL_ARG_INDPTR[b0], 0, n_idx);
-    int count = __builtin_popcountll(__builtin_amdgcn_ballot_w64(lane < batch && lane + qp0 / PL_QT <= item));
-    for (int base = 64; base < batch; base += 64) {
-      const int b = base + lane < batch ? base + lane : batch;
-      const int qp = pl_clamp(CL_ARG_QINDPTR[b], 0, total_q);
-      count += __builtin_popcountll(__builtin_amdgcn_ballot_w64(base + lane < batch && b + qp / PL_QT <= item));
-    }
-    req = count > 0 ? count - 1 : 0;
-    if (batch < 64) {
-      q0 = __builtin_amdgcn_readlane(qp0, req);
-      q1 = __builtin_amdgcn_readlane(qp0, req + 1);
-      kv0 = __builtin_amdgcn_readlane(kp0, req);
-      kv1 = __builtin_amdgcn_readlane(kp0, req + 1);
-    } else {
-      q0 = pl_clamp(CL_ARG_QINDPTR[req], 0, total_q);
-      q1 = pl_clamp(CL_ARG_QINDPTR[req + 1], 0, total_q);
-      kv0 = pl_clamp(CL_ARG_INDPTR[req], 0, n_idx);
-      kv1 = pl_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx);
-    }
-  }
+  // The request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item, found by
+  // all lanes at once (one round trip to memory, which also brings the key row pointers).
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, PL_QT, 1, item, lane, CL_ARG_INDPTR, n_idx);
+  const int req = found.req, q0 = found.p0, q1 = found.p1, kv0 = found.s0, kv1 = found.s1;
   const int chunk = item - req;
   const int lo = q0 > chunk * PL_QT ? q0 : chunk * PL_QT;
   const int hi = q1 < (chunk + 1) * PL_QT ? q1 : (chunk + 1) * PL_QT;

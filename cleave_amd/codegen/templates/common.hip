@@ -50,11 +50,15 @@ CL_DEVICE float lane_read(float v, int src_lane) {
 // (true for every request up to that one, so the lanes test 64 requests at a time and count:
 // one round trip to memory per 256 requests where a bisection makes one per halving), and the
 // clamped ptr[b], ptr[b + 1] -- out of the lanes when there are fewer than 64 requests.
-struct ClRequest { int req, p0, p1; };
+struct ClRequest { int req, p0, p1, s0, s1; };   // s0, s1: the same two entries of a second pointer array
 CL_DEVICE int cl_clamp_ptr(int p, int limit) { return p < 0 ? 0 : (p > limit ? limit : p); }
+// `second` (may be null): another row-pointer array of the same requests, clamped into [0, limit2];
+// its entries for the request found come back as s0, s1 -- read in the same round trip as the
+// searched array when there are fewer than 64 requests.
 CL_DEVICE ClRequest cl_find_request(const int* __restrict__ ptr, int batch, int limit, int div, int with_b,
-                                    int item, int lane) {
+                                    int item, int lane, const int* __restrict__ second = nullptr, int limit2 = 0) {
   const int v0 = cl_clamp_ptr(ptr[lane < batch ? lane : batch], limit);
+  const int w0 = second ? cl_clamp_ptr(second[lane < batch ? lane : batch], limit2) : 0;
   int count = __builtin_popcountll(__builtin_amdgcn_ballot_w64(lane < batch && with_b * lane + v0 / div <= item));
   for (int base = 64; base < batch; base += 256) {
     int v[4];
@@ -71,12 +75,19 @@ CL_DEVICE ClRequest cl_find_request(const int* __restrict__ ptr, int batch, int 
   }
   ClRequest r;
   r.req = count > 0 ? count - 1 : 0;
+  r.s0 = r.s1 = 0;
   if (batch < 64) {
     r.p0 = __builtin_amdgcn_readlane(v0, r.req);
     r.p1 = __builtin_amdgcn_readlane(v0, r.req + 1);
+    r.s0 = __builtin_amdgcn_readlane(w0, r.req);
+    r.s1 = __builtin_amdgcn_readlane(w0, r.req + 1);
   } else {
     r.p0 = cl_clamp_ptr(ptr[r.req], limit);
     r.p1 = cl_clamp_ptr(ptr[r.req + 1], limit);
+    if (second) {
+      r.s0 = cl_clamp_ptr(second[r.req], limit2);
+      r.s1 = cl_clamp_ptr(second[r.req + 1], limit2);
+    }
   }
   return r;
 }

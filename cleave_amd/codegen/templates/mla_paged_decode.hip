@@ -88,12 +88,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // kv_pos <= kv_len - q_len + q_pos of its request
   const int qtok = blockIdx.x;
   // its request: the last b with qo_indptr[b] <= qtok
-  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, 1, 0, qtok, lane);
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, 1, 0, qtok, lane, CL_ARG_INDPTR, n_idx);
   const int req = found.req, q0 = found.p0, q1 = found.p1;
-  const int lo = mp_clamp(CL_ARG_INDPTR[req], 0, n_idx);
+  const int lo = found.s0;
   int hi;
   {
-    int kv_len = mp_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx) - lo;
+    int kv_len = found.s1 - lo;
     kv_len = kv_len > 0 ? kv_len : 0;
     int ext = kv_len - (q1 - q0) + (qtok - q0) + 1;
     ext = qtok < q1 ? ext : 0;                          // (a token past its request's rows: nothing)
