@@ -102,6 +102,49 @@ def test_every_record_kind_against_scalar_loops():
         close(x, y.astype(np.float64), 1e-6)
 
 
+def test_demo_programs_against_float64_restatements_and_identities():
+    """The oracle on the later operators (SwiGLU, LoRA, matmul + row sum, QK-norm attention, attention
+    with unlike key / value widths): against float64 formulas written from the reference's graph
+    docstrings (``tests/_graphs.py:150-160, 403-436, 438-480, 542-640``), and against what the
+    mathematics fixes -- the row sum of a product is the product with the row sums of B; SwiGLU is
+    linear in the bare weight; LoRA with a zero factor is the base product; RMS-normalised rows
+    do not change when a row is scaled."""
+    rng = np.random.default_rng(7)
+    f = lambda *s: rng.normal(size=s).astype(np.float32)          # noqa: E731
+    d = lambda x: x.astype(np.float64)                            # noqa: E731
+    x, wu, wg = f(5, 12), f(12, 7), f(12, 7)
+    prog = C.swiglu.trace(cl.f32, M=5, K=12, N=7)
+    got = po.evaluate(prog, [x, wu, wg])[0]
+    gate = d(x) @ d(wg)
+    close(got, (d(x) @ d(wu)) * gate / (1 + np.exp(-gate)), 1e-5)
+    close(po.evaluate(prog, [x, 3 * wu, wg])[0], 3 * d(got), 1e-5)                       # linear in w_up
+    a, b = f(12, 4), f(4, 7)
+    prog = C.lora.trace(cl.f32, M=5, K=12, N=7, R=4)
+    close(po.evaluate(prog, [x, wu, a, b])[0], d(x) @ d(wu) + (d(x) @ d(a)) @ d(b), 1e-5)
+    close(po.evaluate(prog, [x, wu, a, 0 * b])[0], d(x) @ d(wu), 1e-5)                   # zero factor: the base product
+    prog = C.matmul_rowsum.trace(cl.f32, M=5, K=12, N=7)
+    got = po.evaluate(prog, [x, wu])[0]
+    assert got.shape == (5, 1)
+    close(got[:, 0], d(x) @ d(wu).sum(1), 1e-5)                                          # (x w) 1 = x (w 1)
+    q, k, v = f(4, 6, 8), f(2, 9, 8), f(2, 9, 8)
+    prog = C.qknorm.trace(cl.f32, HQ=4, HKV=2, SQ=6, SKV=9, D=8)
+    got = po.evaluate(prog, [q, k, v])[0]
+    nrm = lambda t: d(t) / np.sqrt((d(t) ** 2).mean(-1, keepdims=True) + 1e-6)           # noqa: E731
+    for h in range(4):
+        s_ = (nrm(q[h]) @ nrm(k[h // 2]).T) / np.sqrt(8)
+        w_ = np.exp(s_ - s_.max(-1, keepdims=True))
+        close(got[h], (w_ / w_.sum(-1, keepdims=True)) @ d(v[h // 2]), 1e-5)
+    q2, k2 = q.copy(), k.copy()
+    q2[1, 3] *= 5.0
+    k2[0, 2] *= 0.25
+    close(po.evaluate(prog, [q2, k2, v])[0], d(got), 1e-4)                               # scale-free rows
+    kk, vv = f(3, 9, 12), f(3, 9, 4)
+    prog = C.mla_prefill.trace(cl.f32, H=3, SQ=6, SKV=9, DK=12, DV=4)
+    got = po.evaluate(prog, [f(3, 6, 12) * 0 + 1, kk, vv])[0]                            # equal queries: rows of a head agree
+    close(got[:, 0], d(got[:, 5]), 1e-6)
+    assert got.shape == (3, 6, 4)
+
+
 def test_grouped_matmul_is_repeat_interleave_not_tile():
     rng = np.random.default_rng(1)
     a, b = rng.normal(size=(6, 2, 4)).astype(np.float32), rng.normal(size=(2, 4, 5)).astype(np.float32)
