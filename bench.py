@@ -78,7 +78,7 @@ def op_table():
                       bytes=2 * 128 * 4096 * (192 + 128 + 192 + 128), flops=2 * 128 * 4096 * 4096 * (192 + 128),
                       bound="mfma", sets=2, cpu=False),
         "lora": dict(title="LoRA f16 x@w + (x@a)@b M=16 N=4096 K=4096 R=16", fn=C.lora, dtype=cl.f16,
-                     shapes=C.FULL["lora"], inputs=C.inputs_lora, split=False,
+                     shapes=C.FULL["lora"], inputs=C.inputs_lora, split=cl.Split("K", (4, 8, 16)),
                      bytes=2 * (16 * 4096 + 4096 * 4096 + 4096 * 16 + 16 * 4096 + 16 * 4096),
                      flops=2 * 16 * 4096 * 4096 + 2 * 16 * 4096 * 16 * 2, bound="hbm", sets=6),
         "mmrs": dict(title="matmul + row sum f16 (x@w).sum(-1) 4096x4096x64", fn=C.matmul_rowsum, dtype=cl.f16,

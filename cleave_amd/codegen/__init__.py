@@ -170,8 +170,12 @@ class HipCodeGen:
         p, op = plan.problem, plan.operands
         self._common(unit, plan, partial, combine)
         norm = plan.family == "rmsnorm_matmul"
+        lora = plan.family == "lora"
         for k in ("M", "N", "K"):
             unit.define(f"CL_{k}", p[k])
+        if lora:
+            unit.define("CL_LORA", 1)
+            unit.define("CL_R", p["R"])
         unit.define("CL_NORM", norm)
         unit.define("CL_GAMMA", bool(norm and p.get("gamma")))
         unit.define("CL_EPS", _f(p.get("eps", 0.0)))
@@ -191,11 +195,13 @@ class HipCodeGen:
             elif plan.role == "partial":
                 sig = ins + outs
             else:  # fused
-                sig = ins + [names[op["PACC"]]] + ([names[op["PSS"]]] if norm else [])
+                sig = ins + [names[op["PACC"]]] + ([names[op["PSS"]]] if norm else []) + ([names[op["PD"]]] if lora else [])
             if splits > 1:
                 unit.define("CL_ARG_PACC", op["PACC"])
                 if norm:
                     unit.define("CL_ARG_PSS", op["PSS"])
+                if lora:
+                    unit.define("CL_ARG_PD", op["PD"])
             for role, macro in (("A", "CL_ARG_A"), ("B", "CL_ARG_B"), ("C", "CL_ARG_C"), ("GAMMA", "CL_ARG_GAMMA"),
                                 ("LA", "CL_ARG_LA"), ("LB", "CL_ARG_LB")):
                 if role in op:
@@ -209,16 +215,25 @@ class HipCodeGen:
                 sig, entry, suffix = ins + outs, ENTRY, ""
             else:
                 # the combine reads the same allocation under its `_combine` name
-                sig = [names[op["PACC_COMBINE"]]] + ([names[op["PSS_COMBINE"]]] if norm else []) + outs
+                sig = [names[op["PACC_COMBINE"]]] + ([names[op["PSS_COMBINE"]]] if norm else []) \
+                    + ([names[op["PD_COMBINE"]], names[op["LB"]]] if lora else []) + outs
                 entry, suffix = COMBINE_ENTRY, "_COMBINE"
             unit.define("CL_CARG_PACC", op["PACC" + suffix])
             if norm:
                 unit.define("CL_CARG_PSS", op["PSS" + suffix])
+            if lora:
+                unit.define("CL_CARG_PD", op["PD" + suffix])
+                unit.define("CL_CARG_LB", op["LB"])
             unit.define("CL_CARG_OUT", op["OUT"])
             args = unit.signature("CL_COMBINE_PARAMS", "CL_COMBINE_NAME", entry, sig, ())
             # columns per thread: the most that still leaves the chip a few hundred workgroups
             total = batch * p["M"] * p["N"]
             cols = next((c for c in (4, 2, 1) if p["N"] % c == 0 and total // c // 256 >= 256), 1)
+            if lora:
+                # a workgroup of the LoRA combine works on one row (it sums that row's rank-R partials once, in LDS)
+                cols = next((c for c in (4, 2, 1) if p["N"] % (256 * c) == 0), None)
+                if cols is None:
+                    raise CodegenError("the LoRA combine needs N to be a multiple of 256")
             unit.define("CL_COMBINE_ROWS", batch * p["M"])
             unit.define("CL_COMBINE_COLS", cols)
             self._combine_args = (entry, args, -(-(total // cols) // 256))
@@ -291,12 +306,10 @@ class HipCodeGen:
         unit.templates.append("skinny_matmul.hip")
         splits = plan.split_factor or 1
         lora = plan.family == "lora"
-        if lora != bool(tile.get("LORA")) or (lora and (splits > 1 or combine)):
-            raise CodegenError("LoRA is the LORA tiling of the few-row matmul, unsplit")
-        if lora:
-            if p["R"] % 8 or p["R"] > 64:
-                raise CodegenError("LoRA rank must be a multiple of 8 up to 64")
-            unit.define("CL_R", p["R"])
+        if lora != bool(tile.get("LORA")):
+            raise CodegenError("LoRA is the LORA tiling of the few-row matmul")
+        if lora and (p["R"] % 8 or p["R"] > 64):
+            raise CodegenError("LoRA rank must be a multiple of 8 up to 64")
         if partial:
             from ..schedule.policy import lora_lds_bytes, skinny_lds_bytes
 

@@ -19,13 +19,15 @@
 //   CL_EPS             epsilon inside the rsqrt
 //   CL_PREFETCH        steps of loads in flight ahead of the one being computed (1..3)
 //
-// CL_LORA: Y = X * W + (X * LA) * LB with LA (K, CL_R) and LB (CL_R, N), unsplit.  The rank-R
+// CL_LORA: Y = X * W + (X * LA) * LB with LA (K, CL_R) and LB (CL_R, N).  The rank-R
 // product D = X * LA rides along: the lanes of the first CL_R / 8 column groups load their 8x8
 // blocks of LA with the W blocks (same ring, same transpose, eight more MFMAs per step into a
 // second accumulator set of which only those column groups mean anything), D is reduced over the
 // K-sharing waves with the main accumulators, rounded to the element type like the input of the
 // reference's second product, parked in LDS, and the epilogue adds D * LB to each lane's outputs
-// with plain multiply-adds (CL_R per output).
+// with plain multiply-adds (CL_R per output).  Split over K (CL_SPLITS > 1) the rank update cannot
+// happen here (it needs all of D): the first column slab's workgroups write their partial sums
+// of D beside the partial products (CL_ARG_PD[split][M][CL_R]) and the combine applies it.
 
 #define SK_MT ((CL_M + 15) / 16)
 #define SK_COLS 128
@@ -39,7 +41,7 @@
 #define CL_LORA 0
 #endif
 #if CL_LORA
-static_assert(CL_R % 8 == 0 && CL_R <= 128 && CL_SPLITS == 1 && !CL_NORM, "LoRA: rank in whole 8-column blocks, unsplit");
+static_assert(CL_R % 8 == 0 && CL_R <= 128 && !CL_NORM, "LoRA: rank in whole 8-column blocks");
 #endif
 // Everything one 32-row step needs, as loaded: the lane's 8x8 block of W, its X fragments
 // (lane (c, g) holds X[16 mt + c][k0 + 8 g .. +8]) and the matching gamma chunk.  X and gamma
@@ -293,7 +295,21 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
   }
 #endif
-#if CL_LORA
+#if CL_LORA && CL_SPLITS > 1
+  if (wk != 0) return;
+  if (blockIdx.x == 0 && wn == 0 && 8 * c < CL_R) {
+#pragma unroll
+    for (int mt = 0; mt < SK_MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = 16 * mt + 4 * g + r;
+        if (m >= CL_M) continue;
+        float* drow = CL_ARG_PD + ((i64)split * CL_M + m) * CL_R + 8 * c;
+        *reinterpret_cast<f32x4*>(drow) = (f32x4){dacc[mt][0][r], dacc[mt][1][r], dacc[mt][2][r], dacc[mt][3][r]};
+        *reinterpret_cast<f32x4*>(drow + 4) = (f32x4){dacc[mt][4][r], dacc[mt][5][r], dacc[mt][6][r], dacc[mt][7][r]};
+      }
+  }
+#elif CL_LORA
   // D (rounded to the element type, as the input of a second product is) goes to LDS for this
   // wave's epilogue; the workgroup-wide barrier is the simplest fence between its lanes
   if (wk == 0 && 8 * c < CL_R) {

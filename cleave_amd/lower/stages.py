@@ -39,11 +39,13 @@ def partial_buffers(low: Lowered, factor: int) -> list:
     like the reference's ``(split, batch, heads[, D])`` layout
     (``python/cleave/dynamic/paging/tensor_maps.py:41-69``); f32 except the MLA value partials."""
     p = low.problem
-    if low.family in ("matmul", "rmsnorm_matmul"):
+    if low.family in ("matmul", "rmsnorm_matmul", "lora"):
         batch = max(p["batch_A"], p["batch_B"])
         bufs = [("PACC", (factor, batch * p["M"], p["N"]), "float32")]
         if low.family == "rmsnorm_matmul":
             bufs.append(("PSS", (factor, batch * p["M"]), "float32"))
+        if low.family == "lora":
+            bufs.append(("PD", (factor, p["M"], p["R"]), "float32"))     # partial sums of the rank-R product x @ a
         return bufs
     if low.family == "attention":
         rows, width = p["units"] * p["group"] * p["sq"], p["vdim"]
@@ -73,6 +75,9 @@ def split_stages(graph: StageGraph, factor: int) -> list:
     bufs = partial_buffers(low, factor)
     part_outs = [irg.OutputNode(f"OutputNode_{i}", shape, dt) for i, (_, shape, dt) in enumerate(bufs)]
     comb_ins = [irg.PlaceHolderNode(f"PlaceHolder_{n}", shape, dt) for n, shape, dt in bufs]
+    if low.family == "lora":
+        # the rank update happens in the combine, which therefore also reads the up factor
+        comb_ins.append(low.operands["LB"])
     partial = StageGraph(graph, low, "partial", factor, outputs=part_outs)
     combine = StageGraph(graph, low, "combine", factor, placeholders=comb_ins)
     partial.name, combine.name = f"{graph.name}.partial", f"{graph.name}.combine"

@@ -117,7 +117,7 @@ def _split_dim_of(program, lowered) -> str | None:
     """Name of the program dim the recognised family can be split over (K or the KV length)."""
     from ..frontend.tensor import Dim
 
-    if lowered.family in ("matmul", "rmsnorm_matmul"):
+    if lowered.family in ("matmul", "rmsnorm_matmul", "lora"):
         node, axis = lowered.operands["A"], (-2 if lowered.problem["trans_A"] else -1)
     elif lowered.family == "attention":
         node, axis = lowered.operands["K"], -2

@@ -221,9 +221,22 @@ def execute(graph, inputs, device=None) -> list:
     if low.family == "swiglu":
         return [r.reshape(s) for r, s in zip(_eval_swiglu(low, feed, out_dtype), shapes)]
     if low.family == "lora":
-        # x @ w + (x @ a) @ b, the down product rounded to the storage type before the up product
+        # x @ w + (x @ a) @ b, the down product rounded to the storage type before the up product;
+        # split over K: partial sums of x @ w and of x @ a, and a combine that applies the rank update
+        import torch
+
+        if role == "combine":
+            down = feed["PlaceHolder_PD"].float().sum(0).to(torch_dtype(graph.dtype)).float()
+            lb = feed[low.operands["LB"].name].float()
+            return [(feed["PlaceHolder_PACC"].float().sum(0) + down @ lb).to(out_dtype).reshape(shapes[0])]
         a, b = _mm_operands(low, feed)
-        la, lb = feed[low.operands["LA"].name].float(), feed[low.operands["LB"].name].float()
+        la = feed[low.operands["LA"].name].float()
+        if role == "partial":
+            kc = low.problem["K"] // factor
+            pacc = torch.stack([a[0, :, s * kc:(s + 1) * kc] @ b[0, s * kc:(s + 1) * kc] for s in range(factor)])
+            pd = torch.stack([a[0, :, s * kc:(s + 1) * kc] @ la[s * kc:(s + 1) * kc] for s in range(factor)])
+            return [pacc.reshape(shapes[0]), pd.reshape(shapes[1])]
+        lb = feed[low.operands["LB"].name].float()
         down = (a @ la).to(torch_dtype(graph.dtype)).float()
         return [(a @ b + down @ lb).to(out_dtype).reshape(shapes[0])]
     if low.family == "matmul_rowsum":

@@ -35,8 +35,8 @@ def _candidates(graph, arch):
     if fam == "lora":
         cands = policy.lora_candidates(low, role, factor, arch)
         if not cands:
-            raise ScheduleRejected("LoRA runs on the few-row matmul kernel only: M <= 64, K % 32 == 0, N % 8 == 0, "
-                                   "rank a multiple of 8 up to 64, unsplit")
+            raise ScheduleRejected("LoRA runs on the few-row matmul kernel only: M <= 64, K % 32 == 0, N % 8 == 0 "
+                                   "(N % 256 == 0 when split), rank a multiple of 8 up to 64")
         return cands
     if fam == "attention":
         if not policy.attn_ok(low):
@@ -115,9 +115,10 @@ def apply_tiling(cand: TileDict) -> KernelPlan:
             params.append(ParamSpec(ph.name, ph.dtype, tuple(ph.shape), "input"))
             operands[by_node[id(ph)]] = ph.name
     else:
+        keep_role = {id(n): r for r, n in low.operands.items()}      # an original input a combine reads (LoRA's up factor)
         for ph in graph.placeholders:
             params.append(ParamSpec(ph.name, ph.dtype, tuple(ph.shape), "input"))
-            operands[ph.name.replace("PlaceHolder_", "")] = ph.name
+            operands[keep_role.get(id(ph), ph.name.replace("PlaceHolder_", ""))] = ph.name
     if role == "partial":
         for out, (bname, shape, dt) in zip(graph.outputs, partial_buffers(low, cand.split_factor)):
             params.append(ParamSpec(out.name, dt, tuple(shape), "output"))

@@ -217,19 +217,20 @@ def lora_lds_bytes(mt, waves_n, waves_k, rank):
 
 
 def lora_candidates(low, role, factor, arch: Arch):
-    """LoRA: the few-row matmul with the rank-R product riding along (unsplit: the rank update needs
-    the whole of ``x @ a``)."""
+    """LoRA: the few-row matmul with the rank-R product ``x @ a`` riding along.  Unsplit, the epilogue
+    applies the rank update; split over K, the partial kernel writes partial sums of both products
+    and the combine applies it (it needs the whole of ``x @ a``)."""
     import copy
 
     p = low.problem
-    if (factor or 1) > 1 or p["R"] % 8 or p["R"] > 64:
+    if p["R"] % 8 or p["R"] > 64 or ((factor or 1) > 1 and p["N"] % 256):
         return []
     twin = copy.copy(low)
     twin.family = "matmul"
     if not skinny_ok(twin):
         return []
     out = []
-    for c in skinny_candidates(twin, role, None, arch):
+    for c in skinny_candidates(twin, role, factor, arch):
         t = c.tiling
         lds = lora_lds_bytes(_ceil(p["M"], 16), t["WAVES_N"], t["WAVES_K"], p["R"])
         if lds > arch.lds_bytes:
@@ -446,6 +447,7 @@ def mla_candidates(low, role, factor, arch: Arch):
 def combine_candidates(low, factor, arch: Arch):
     """The combine of a split has one shape: one thread per 4 (attention) or 4/8 (matmul)
     output columns, 256 threads; it is memory-trivial next to its partial."""
-    family = {"matmul": "gemm", "rmsnorm_matmul": "gemm", "attention": "attn_decode", "mla": "mla_decode"}[low.family]
+    family = {"matmul": "gemm", "rmsnorm_matmul": "gemm", "lora": "gemm", "attention": "attn_decode",
+              "mla": "mla_decode"}[low.family]
     return [TileDict(family, "combine", {}, output_tile=[1, 256], rstep_map={"split": factor}, n_threads=256,
                      split_factor=factor, score=1.0, lds_bytes=0, est_vgprs=32)]

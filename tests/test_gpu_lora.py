@@ -52,6 +52,31 @@ def test_lora_ranks_types_and_benchmark_size():
     _check(cl.f16, C.FULL["lora"])
 
 
+@pytest.mark.parametrize("split,tiling", [(2, dict(WAVES_N=1, WAVES_K=1)), (4, dict(WAVES_N=1, WAVES_K=2)),
+                                          (8, dict(WAVES_N=2, WAVES_K=2))], ids=["s2", "s4", "s8"])
+def test_lora_split_over_k(split, tiling):
+    """Partial sums of both products per K split; the combine adds them up and applies the rank update."""
+    for dtype, shapes in ((cl.f16, dict(M=16, N=512, K=1024, R=16)), (cl.bf16, dict(M=40, N=256, K=512, R=32))):
+        prog = C.lora.trace(dtype, **shapes)
+        args = _inputs(prog, 8)
+        print(f"lora split case {dtype} {shapes} split={split} {tiling}", flush=True)
+        out = kernel_for(prog, template="skinny", tiling=dict(tiling, LORA=1), split=split)(*args)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(out.float().cpu().numpy(), program_oracle.evaluate(prog, list(args))[0],
+                                   rtol=1e-2, atol=1e-2)
+
+
+def test_lora_benchmark_size_picks_a_split_variant(cache_root):
+    kernel = P.compile(C.lora, shapes=C.FULL["lora"], dtype=cl.f16, split=cl.Split("K", (4, 8)),
+                       schedule=P.ScheduleConfig(topk=3, split_k=(4, 8)), eval=P.EvalConfig(warmup=2, iters=20, max_parallel=2))
+    rep = kernel.report
+    assert len(rep.correct) == len(rep) and kernel.variant.startswith("split")
+    prog = cleave_amd.trace(C.lora, C.FULL["lora"], cl.f16)
+    args = _inputs(prog, 10)
+    np.testing.assert_allclose(kernel(*args).float().cpu().numpy(), program_oracle.evaluate(prog, list(args))[0],
+                               rtol=1e-2, atol=1e-2)
+
+
 def test_lora_compiles_end_to_end(cache_root):
     shapes = dict(M=16, N=1024, K=1024, R=16)
     kernel = P.compile(C.lora, shapes=shapes, dtype=cl.f16, split=False, schedule=P.ScheduleConfig(topk=4),

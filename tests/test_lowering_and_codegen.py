@@ -146,8 +146,15 @@ def test_lora_is_a_family_of_its_own():
                                                  "OutputNode_0"]
     with pytest.raises(ScheduleRejected, match="few-row matmul kernel only"):
         search_tiling(stage_graph(C.lora.trace(cl.f16, M=256, N=512, K=512, R=16)))
-    with pytest.raises(LoweringRejected, match="no split form"):
-        split_stages(g, 4)
+    # split over K: partial sums of both products; the combine applies the rank update, so it also reads the up factor
+    partial, combine = split_stages(g, 8)
+    assert [o.shape for o in partial.outputs] == [(8, 16, 4096), (8, 16, 16)]
+    assert [p.name for p in combine.placeholders] == ["PlaceHolder_PACC", "PlaceHolder_PD", "PlaceHolder_b"]
+    fused = parse_manifest(source_for(C.lora.trace(cl.f16, **C.FULL["lora"]), template="skinny",
+                                      tiling=dict(WAVES_N=1, WAVES_K=2, LORA=1), split=8))
+    assert [l["args"] for l in fused["launches"]] == [
+        ["PlaceHolder_x", "PlaceHolder_w", "PlaceHolder_a", "PlaceHolder_b", "Partial_PACC_split", "Partial_PD_split"],
+        ["Partial_PACC_combine", "Partial_PD_combine", "PlaceHolder_b", "OutputNode_0"]]
 
 
 def test_unrecognised_program_is_refused():
