@@ -555,8 +555,12 @@ class HipCodeGen:
         for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_CHUNKED", chunked),
                      ("CL_CHUNK_PAGES", chunked), ("CL_Q_HEADS", p["heads"]), ("CL_PREFILL", prefill)):
             unit.define(k, v)
+        tok = int(t.get("TOK", 1)) if prefill else 1
+        if tok not in (1, 2, 4):
+            raise CodegenError("a paged MLA prefill item holds 1, 2 or 4 query tokens")
         if prefill:
             unit.define("CL_ARG_QINDPTR", op["QINDPTR"])
+            unit.define("CL_MP_TOK", tok)
         if "LDS_AHEAD" in t:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
         for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE"),
@@ -566,8 +570,8 @@ class HipCodeGen:
         if partial:
             items = f"ceildiv({p['dim_names']['n_idx']}, chunk_pages) + {batch_name}" if chunked else batch_name
             if prefill:
-                items = p["dim_names"]["total_q"]
-            unit.launch(ENTRY, (items, p["heads"] // 16, 1), 64, 0, self._partial_args)
+                items = f"ceildiv({p['dim_names']['total_q']}, {tok}) + batch"
+            unit.launch(ENTRY, (items, p["heads"] // 16, 1), 64 * tok, 0, self._partial_args)
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv(({batch_name} * {p['heads']}) * {p['ckv'] // 4}, 256)", 1, 1), 256, 0, args)

@@ -14,8 +14,13 @@
 // read.  Scores, softmax and value product are the dense kernel's (16 heads per wave, Q fragments
 // resident, fixed softmax reference raised outside the hot loop).
 //
-// CL_PREFILL: causal prefill over ragged query rows -- an item is one query token (rows = its 16
-// heads) and the keys its causal limit admits; out and lse are per query token.
+// CL_PREFILL: causal prefill over ragged query rows -- an item is up to CL_MP_TOK consecutive query
+// tokens of one request (a new item at every multiple of CL_MP_TOK packed tokens and at every
+// request boundary), one wave per token (rows = its 16 heads), and the keys the item's last token
+// may see: the waves of an item share the two images (each loads a share of a step's rows, one
+// barrier per step) and every wave masks by its own token's causal limit; out and lse are per
+// query token.  Four tokens per item quarter the traffic into the CU and put eight waves on a CU
+// where single-token items have two (an item's images take 72 KB of LDS whatever its wave count).
 //
 //   CL_HEADS (multiple of 16)  CL_CKV  CL_KPE (multiples of 64)  CL_CHUNKED  CL_PREFILL
 //   run-time: batch, num_pages, n_idx [, chunk_pages]; scalar sm_scale (> 0 or not: the
@@ -24,6 +29,11 @@
 #ifndef CL_PREFILL
 #define CL_PREFILL 0
 #endif
+#ifndef CL_MP_TOK
+#define CL_MP_TOK 1
+#endif
+#define MP_WAVES (CL_PREFILL ? CL_MP_TOK : 1)   // waves per workgroup
+static_assert(MP_WAVES == 1 || MP_WAVES == 2 || MP_WAVES == 4, "1, 2 or 4 tokens per prefill item");
 #define MP_STEP 32
 #define MP_D (CL_CKV + CL_KPE)
 #define MP_PANEL (MP_STEP * 64)
@@ -69,9 +79,9 @@ CL_DEVICE void mp_issue_row_group(const char* lat_src, const char* pe_src, unsig
 }
 
 #if CL_EMIT_PARTIAL
-extern "C" __global__ void __launch_bounds__(64)
+extern "C" __global__ void __launch_bounds__(64 * MP_WAVES)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
-  const int lane = threadIdx.x & 63;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int head0 = 16 * blockIdx.y;
 #if CL_CHUNKED
@@ -84,20 +94,25 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int hi = p1 < (chunk + 1) * chunk_pages ? p1 : (chunk + 1) * chunk_pages;
   if (hi <= lo) return;                               // an index no (chunk, request) pair maps to
 #elif CL_PREFILL
-  // causal prefill: an item is one query token (its 16 heads are the tile); it sees the keys
-  // kv_pos <= kv_len - q_len + q_pos of its request
-  const int qtok = blockIdx.x;
-  // its request: the last b with qo_indptr[b] <= qtok
-  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, 1, 0, qtok, lane, CL_ARG_INDPTR, n_idx);
+  // causal prefill: the request whose items include `item` is the last b with
+  // b + qo_indptr[b] / MP_WAVES <= item; token t of it sees the keys kv_pos <= kv_len - q_len + (t - q0)
+  const int item = blockIdx.x;
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, MP_WAVES, 1, item, lane, CL_ARG_INDPTR, n_idx);
   const int req = found.req, q0 = found.p0, q1 = found.p1;
+  const int chunk = item - req;
+  const int t_lo = q0 > chunk * MP_WAVES ? q0 : chunk * MP_WAVES;
+  const int t_hi = q1 < (chunk + 1) * MP_WAVES ? q1 : (chunk + 1) * MP_WAVES;
+  if (t_hi <= t_lo) return;                           // an index no (chunk, request) pair maps to
+  const bool tok_live = t_lo + wave < t_hi;           // this wave's token (a wave past the item's tokens only helps load)
+  const int qtok = tok_live ? t_lo + wave : t_lo;
   const int lo = found.s0;
-  int hi;
+  int hi, n_tok_own;
   {
     int kv_len = found.s1 - lo;
     kv_len = kv_len > 0 ? kv_len : 0;
-    int ext = kv_len - (q1 - q0) + (qtok - q0) + 1;
-    ext = qtok < q1 ? ext : 0;                          // (a token past its request's rows: nothing)
-    hi = lo + mp_clamp(ext, 0, kv_len);
+    const int ext_own = kv_len - (q1 - q0) + (qtok - q0) + 1, ext_all = kv_len - (q1 - q0) + (t_hi - 1 - q0) + 1;
+    n_tok_own = tok_live ? mp_clamp(ext_own, 0, kv_len) : 0;
+    hi = lo + mp_clamp(ext_all, 0, kv_len);           // the item's last token sees the most
   }
 #else
   const int req = blockIdx.x;
@@ -105,8 +120,13 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   int hi = mp_clamp(CL_ARG_INDPTR[req + 1], 0, n_idx);
   hi = hi > lo ? hi : lo;
 #endif
+#if CL_PREFILL
+  const int n_tok = n_tok_own;                        // keys this wave's token weighs
+  const int n_steps = (hi - lo + MP_STEP - 1) / MP_STEP;   // steps of the item (the same for all its waves)
+#else
   const int n_tok = hi - lo;
   const int n_steps = (n_tok + MP_STEP - 1) / MP_STEP;
+#endif
   const float scale_log2e = sm_scale * 1.4426950408889634f;
 #if CL_PREFILL
   const i64 qrow = (i64)qtok * CL_HEADS + head0 + c;
@@ -151,7 +171,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       const int held = k == 0 ? ids[0] : k == 1 ? ids[1] : k == 2 ? ids[2] : ids[3];
       const unsigned stage_byte = tiles_byte + (unsigned)((s & 1) * MP_TILE * 2);
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
+      for (int i = 0; i < 4 / MP_WAVES; ++i) {
+        const int rg = wave + i * MP_WAVES;             // (the waves of an item share a step's four row groups)
         const int r = 8 * rg + (lane >> 3);
         const int src_lane = 32 * (in_window & 1) + r;
         const int id = __builtin_amdgcn_ds_bpermute(src_lane << 2, held);
@@ -195,7 +216,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           // ops of step - 1, all issued)
           __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
           __syncthreads();
-          if (step % (MP_WINDOW / MP_STEP) == 0 && (step / (MP_WINDOW / MP_STEP) + 1) * MP_WINDOW < n_tok)
+          if (step % (MP_WINDOW / MP_STEP) == 0 && (step / (MP_WINDOW / MP_STEP) + 1) * MP_WINDOW < hi - lo)
             load_window(step / (MP_WINDOW / MP_STEP) + 1, ids_next);
           if (step + 1 < n_steps) {
             if ((step + 1) % (MP_WINDOW / MP_STEP) == 0) {
@@ -207,6 +228,15 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           front_done = true;
         }
         const elem_t* tile = mp_tiles + (step & 1) * MP_TILE;
+#if CL_PREFILL
+        // a wave whose token sees none of this step's keys (or that has no token: it only helps
+        // load) leaves the images to the waves that need them
+        if (step * MP_STEP >= n_tok) {
+          ++step;
+          front_done = false;
+          continue;
+        }
+#endif
 
         // scores^T: rows = tokens 16 h + (0..15), columns = heads
         f32x4 st[2];
@@ -255,7 +285,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
+#if CL_PREFILL
+            // (a wave whose token sees none of a step's keys has no reference yet: test the mask itself)
+            const float p = st[h][r] > 0.5f * CL_NEG_BIG ? fast_exp2(st[h][r] - m_run) : 0.f;
+#else
             const float p = fast_exp2(st[h][r] - m_run);
+#endif
             l_exact += p;
             pf[4 * h + r] = to_elem(p);
           }
@@ -301,6 +336,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 
   // ---- write this wave's heads ------------------------------------------------------------------
+#if CL_PREFILL
+  if (!tok_live) return;
+#endif
   const float l = l_acc[0];
   const int f0 = 4 * g;
 #if CL_CHUNKED

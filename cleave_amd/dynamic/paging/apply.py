@@ -316,7 +316,7 @@ def mla_chunk_pages_expr(spec: MLASpec, chunk_pages: int) -> str:
     return f"max(32, min(512, ceildiv({spec.index_dim}, max(1, {2 * cus} - {spec.batch_dim}))))"
 
 
-def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None) -> KernelPlan:
+def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None, tok: int = 1) -> KernelPlan:
     prefill = spec.kind == MLA_PAGED_PREFILL_CAUSAL
     dim_names = {"total_q": spec.tokens_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim} if prefill else \
         {"batch": spec.batch_dim, "num_pages": spec.pages_dim, "n_idx": spec.index_dim}
@@ -327,12 +327,14 @@ def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None
     tiling, extra = {}, {}
     if prefill:     # the request count follows from the row pointers
         extra["derived_dims"] = [("batch", f"{spec.indptr_dim} - 1")]
+        tiling["TOK"] = int(tok)          # query tokens (= waves) per work item
     if split:
         tiling["CHUNK_PAGES"] = dense.chunk_pages
         extra["derived_dims"] = [("chunk_pages", mla_chunk_pages_expr(spec, dense.chunk_pages))]
+    threads = dense.n_threads * (int(tok) if prefill else 1)
     return KernelPlan(template="mla_decode", role=role, family="mla", dtype=dense.dtype, extra=extra, problem=problem,
                       tiling=tiling, params=params, operands=operands, split_factor=split, dyn_dims=dyn,
-                      n_threads=dense.n_threads, label=f"kv={dense.kv_tile} q={dense.heads} thr={dense.n_threads}")
+                      n_threads=threads, label=f"kv={dense.kv_tile} q={dense.heads * (int(tok) if prefill else 1)} thr={threads}")
 
 
 def _mla_split_decode(spec: MLASpec, dense: DenseMLA, split: int) -> list:
@@ -354,15 +356,24 @@ def _mla_split_decode(spec: MLASpec, dense: DenseMLA, split: int) -> list:
     return [partial, combine]
 
 
-def apply_paging(plan: KernelPlan, spec) -> KernelPlan:
-    """A single paged decode kernel at ``plan``'s tiling."""
+def mla_prefill_variants(plan: KernelPlan, spec) -> list:
+    """The paged MLA causal prefill kernel with two, four and one query tokens per work item (the
+    search times each: an item's waves share its key images, which divides the traffic into the
+    CU and raises the number of waves a CU holds, but they also share the LDS bandwidth that
+    bounds this kernel's matrix work; two tokens per item measured best on the captured workloads)."""
+    return [apply_paging(plan, spec, tok=t) for t in (2, 4, 1)]
+
+
+def apply_paging(plan: KernelPlan, spec, tok: int = 2) -> KernelPlan:
+    """A single paged kernel at ``plan``'s tiling (``tok``: query tokens per work item of the
+    paged MLA causal prefill layer)."""
     spec.validate()
     if isinstance(spec, MLASpec):
         dense = read_dense_mla(plan)
         _check_tiling(spec, dense)
         params, operands = _mla_params(spec, dense)
         outs, out_ops = _mla_outputs(spec, dense)
-        return _mla_plan(spec, dense, "main", params + outs, {**operands, **out_ops})
+        return _mla_plan(spec, dense, "main", params + outs, {**operands, **out_ops}, tok=tok)
     dense = read_dense_attention(plan)
     _check_tiling(spec, dense)
     if spec.kind in CAUSAL_KINDS:

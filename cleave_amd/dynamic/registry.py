@@ -70,7 +70,7 @@ class DynamicOperator:
             dense = DenseMLA(self.dims[0], self.dims[1], self.dims[2], "bfloat16", "bfloat16")
             params, ops = _mla_params(self.spec, dense)
             outs, out_ops = _mla_outputs(self.spec, dense)
-            return HipCodeGen().gen(_mla_plan(self.spec, dense, "main", params + outs, {**ops, **out_ops}))
+            return HipCodeGen().gen(_mla_plan(self.spec, dense, "main", params + outs, {**ops, **out_ops}, tok=2))
         dense = DenseAttention(t["query_rows"], t["kv_tile"], t["head_dim"], t["waves"] * 64, "bfloat16", "bfloat16",
                                waves=t["waves"])
         params, ops = _paged_params(self.spec, dense)

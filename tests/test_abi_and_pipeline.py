@@ -157,7 +157,9 @@ def test_paged_mla_layer_plans_and_signature():
     assert [p["name"] for p in pre["params"]] == ["PlaceHolder_Q_NOPE", "PlaceHolder_Q_PE", "PlaceHolder_CKV_CACHE",
                                                  "PlaceHolder_KPE_CACHE", "PlaceHolder_QO_INDPTR", "PlaceHolder_KV_INDPTR",
                                                  "PlaceHolder_KV_INDICES", "sm_scale", "OutputNode_0", "OutputNode_1"]
-    assert pre["launches"][0]["grid"][0] == "total_q" and dict(pre["derived_dims"]) == {"batch": "len_indptr - 1"}
+    # two query tokens (waves) per work item: a new item at every second packed token and at every request boundary
+    assert pre["launches"][0]["grid"][0] == "ceildiv(total_q, 2) + batch" and pre["launches"][0]["block"][0] == 128
+    assert dict(pre["derived_dims"]) == {"batch": "len_indptr - 1"} and pre["tiling"]["TOK"] == 2
     gqa = parse_manifest(registry.OPERATORS["gqa_ragged_prefill_causal_h32_kv8_d128"].kernel_source())
     assert [p["name"] for p in gqa["params"]] == ["PlaceHolder_Q", "PlaceHolder_K", "PlaceHolder_V", "PlaceHolder_QO_INDPTR",
                                                  "PlaceHolder_KV_INDPTR", "sm_scale", "OutputNode_0", "OutputNode_1"]

@@ -106,26 +106,29 @@ def test_registry_mla_operator_workloads(axes):
         check(mla_kernel(split=split), args, lens, f"registry axes {axes} split={split}")
 
 
-def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16"):
+def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4):
     spec = MLASpec(num_qo_heads=heads, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True)
     spec.validate()
     dense = DenseMLA(heads, ckv, kpe, dtype, dtype)
     params, ops = _mla_params(spec, dense)
     outs, out_ops = _mla_outputs(spec, dense)
-    loaded = _load_main_kernel_from_code(HipCodeGen().gen(_mla_plan(spec, dense, "main", params + outs, {**ops, **out_ops})))
+    loaded = _load_main_kernel_from_code(HipCodeGen().gen(_mla_plan(spec, dense, "main", params + outs, {**ops, **out_ops},
+                                                                    tok=tok)))
     return _compile(loaded, loaded.manifest["out_idx"])
 
 
+@pytest.mark.parametrize("tok", [1, 2, 4], ids=lambda t: f"tok{t}")
 @pytest.mark.parametrize("q_lens,kv_lens", [([1, 4, 5, 33, 0, 40, 7], [1, 4, 40, 33, 9, 300, 3]), ([6, 0, 3], [0, 5, 3]),
-                                            ([90], [700])])
-def test_paged_mla_causal_prefill(q_lens, kv_lens):
-    """Ragged query rows, one item per query token: equal lengths, a cached prefix, windows shorter
-    than the query run (fully masked rows), requests without queries or without keys, a long
-    prefix (table windows reloaded)."""
+                                            ([90], [700]), ([3, 9], [2, 5])])
+def test_paged_mla_causal_prefill(q_lens, kv_lens, tok):
+    """Ragged query rows, one, two or four query tokens per item (one wave each, sharing the
+    item's key images): equal lengths, a cached prefix, windows shorter than the query run (fully
+    masked rows beside live ones in one item), requests without queries or without keys, a long
+    prefix (table windows reloaded), items cut by request boundaries."""
     tq, tk = sum(q_lens), sum(kv_lens)
     args = dref.mla_paged_prefill_inputs((16, 512, 64, 4 * tk + 64, tk + 3, tq), q_lens, kv_lens, device="cpu")
-    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens}", flush=True)
-    out, lse = mla_prefill_kernel()(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens} tok={tok}", flush=True)
+    out, lse = mla_prefill_kernel(tok=tok)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
     torch.cuda.synchronize()
     got_o, got_l = out.float().cpu().numpy(), lse.cpu().numpy()
     want_o, want_l = paged_oracle.mla_prefill(*args[:7], q_lens, kv_lens, args[7])
