@@ -374,8 +374,8 @@ class HipCodeGen:
 
     def _emit_attn_decode(self, unit, plan, params, partial, combine, fused):
         p, t, op = plan.problem, plan.tiling, plan.operands
-        if p.get("norm_eps"):
-            raise CodegenError("the streaming attention kernel has no QK-norm form")
+        if p.get("norm_eps") or p.get("linear"):
+            raise CodegenError("the streaming attention kernel has no QK-norm form and no softmax-free form")
         paged = bool(p.get("paged"))
         rows = p["group"] * p["sq"]
         emit_lse = bool(p.get("emit_lse"))
@@ -439,6 +439,7 @@ class HipCodeGen:
             unit.define(k, v)
         unit.define("CL_SCALE", _f(float(p.get("scale", 1.0))))
         norm = p.get("norm_eps") or {}
+        unit.define("CL_LINEAR", bool(p.get("linear")))
         unit.define("CL_QNORM", "q" in norm)
         unit.define("CL_KNORM", "k" in norm)
         unit.define("CL_QNORM_EPS", _f(float(norm.get("q", 0.0))))

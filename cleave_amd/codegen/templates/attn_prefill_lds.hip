@@ -26,6 +26,9 @@
 // CL_SKV and CL_SCALE are constants, an item is 128 consecutive rows of one unit, there are no
 // row pointers and no lse.
 //
+// CL_LINEAR (dense mode): no softmax -- out = (q k^T) v, the raw scores times CL_SCALE, rounded to the
+// element type, are the weights; no maxima, no reference, no normalisation.
+//
 // CL_QNORM / CL_KNORM (QK-norm attention): query / key rows enter the scores RMS-normalised over
 // their features, x * rsqrt(mean(x^2) + eps).  Query rows are normalised once when they are loaded.
 // Key rows cannot be touched on their way into LDS, so their factors multiply the scores instead:
@@ -48,6 +51,9 @@
 #endif
 #ifndef CL_DENSE
 #define CL_DENSE 0
+#endif
+#ifndef CL_LINEAR
+#define CL_LINEAR 0
 #endif
 #ifndef CL_QNORM
 #define CL_QNORM 0
@@ -462,7 +468,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int rt = 0; rt < 2; ++rt) {
         const int room = lim_rel[rt] - step * PL_STEP;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) s[rt][i] = 16 * (i >> 2) + (i & 3) <= room ? s[rt][i] : CL_NEG_INF;
+        for (int i = 0; i < 8; ++i) s[rt][i] = 16 * (i >> 2) + (i & 3) <= room ? s[rt][i] : (CL_LINEAR ? 0.f : CL_NEG_INF);
       }
     }
     // (first half of the score products of step + 1 in the shadow of the maxima)
@@ -475,6 +481,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[j][h], qf[rt][j], sn[rt][h]);
+#if !CL_LINEAR
     float mx[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
@@ -501,6 +508,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         for (int fb = 0; fb < PL_FB; ++fb) acc[rt][fb] *= alpha;
       }
     }
+#endif  // !CL_LINEAR
     __builtin_amdgcn_sched_barrier(0);
     PL_ISSUE(1);
 
@@ -510,7 +518,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       float psum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
+#if CL_LINEAR
+        const float p = s[rt][i] * sm_scale;
+#else
         const float p = fast_exp2(__builtin_fmaf(s[rt][i], scale2, -m_run[rt]));
+#endif
         psum += p;
         pf[rt][i] = to_elem(p);
       }
@@ -591,7 +603,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #if CL_PF_DBG_NOSTORE
     if (l != 12345.f) continue;
 #endif
+#if CL_LINEAR
+    const float inv = 1.0f;
+#else
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
+#endif
     const i64 orow = row_index(m);
     // A lane holds features 16 fb + 4 g .. + 3 of its row for every block fb.  Lanes g and g ^ 1
     // trade halves of a pair of blocks (one row swap per register), so that each stores 16

@@ -43,10 +43,10 @@ def _candidates(graph, arch):
             raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "
                                    f"a multiple of 128, got {low.problem['head_dim']}/{low.problem['vdim']}")
         many = policy.attn_many_rows_candidates(low, role, factor, arch)
-        if low.problem.get("norm_eps"):
+        if low.problem.get("norm_eps") or low.problem.get("linear"):
             if not many:
-                raise ScheduleRejected("QK-norm attention runs on the many-row kernel only: at least 64 query rows per "
-                                       "unit, widths in 64-feature panels, unsplit")
+                raise ScheduleRejected("QK-norm attention and chained matmuls run on the many-row kernel only: at least "
+                                       "64 query rows per unit, widths in 64-feature panels, unsplit")
             return many
         return policy.attn_candidates(low, role, factor, arch) + many
     if fam == "mla":

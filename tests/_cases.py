@@ -68,6 +68,13 @@ def qknorm(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl
 
 
 @cleave_amd.jit
+def matmul_matmul(q: cl.Tensor["H", "SQ", "D"], k: cl.Tensor["H", "SKV", "D"], v: cl.Tensor["H", "SKV", "D"]):
+    """``(q @ k^T) @ v`` with nothing in between (the reference's ``matmul_matmul_bhsd`` case,
+    ``tests/_graphs.py:78-101``)."""
+    return (q @ k.mT) @ v
+
+
+@cleave_amd.jit
 def gqa_decode_shift(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
     n = q.shape[-1] ** 0.5
     return cl.softmax((q @ k.mT) / n, dim=-1, shift=-50 / n) @ v

@@ -104,6 +104,37 @@ def test_streaming_kernel_strides_keys_and_values_by_their_own_widths(waves):
                                    rtol=1e-2, atol=1e-2)
 
 
+def test_chained_matmul_is_attention_without_softmax():
+    """``(q @ k^T) @ v`` (the reference's ``matmul_matmul_bhsd`` case, (1, 32, 4096, 4096, 64)):
+    small against the oracle (ragged rows and keys), then the reference's size on a sample of rows
+    with the scores rounded to the element type as the second product's input is."""
+    def scaled(prog, seed):
+        q, k, v = prog.random_inputs(seed=seed)
+        return (q.float() / 8).to(q.dtype), k, v            # keeps sums of thousands of products inside f16
+
+    for dtype, shapes in ((cl.f16, dict(H=3, SQ=100, SKV=150, D=64)), (cl.bf16, dict(H=2, SQ=64, SKV=33, D=128))):
+        prog = C.matmul_matmul.trace(dtype, **shapes)
+        args = scaled(prog, 29)
+        print(f"chained matmul case {dtype} {shapes}", flush=True)
+        out = kernel_for(prog)(*args)
+        torch.cuda.synchronize()
+        want = program_oracle.evaluate(prog, list(args))[0]
+        # the weights here are raw scores of magnitude well above 1 kept to 11 (f16) or 8 (bf16) bits, and the sums
+        # cancel: the absolute tolerance follows the magnitude of the outputs and the width of the element type
+        atol = 1e-2 + np.abs(want).max() * (2.0 ** -6 if dtype is cl.bf16 else 2.0 ** -9)
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=atol)
+    shapes = dict(H=32, SQ=4096, SKV=4096, D=64)
+    prog = C.matmul_matmul.trace(cl.f16, **shapes)
+    q, k, v = scaled(prog, 31)
+    out = kernel_for(prog)(q, k, v)
+    torch.cuda.synchronize()
+    gen = np.random.default_rng(4)
+    for h, s in zip(gen.integers(0, 32, 32), gen.integers(0, 4096, 32)):
+        w = (k[h].float() @ q[h, s].float()).to(torch.float16).double()
+        want = (w @ v[h].double()).float().cpu().numpy()
+        np.testing.assert_allclose(out[h, s].float().cpu().numpy(), want, rtol=1e-2, atol=1e-2 * max(1.0, np.abs(want).max() / 16))
+
+
 def test_search_prefers_the_shared_kernel_for_many_rows_and_keeps_decode_for_few():
     from cleave_amd.schedule import search_tiling
 

@@ -157,6 +157,12 @@ def test_lora_is_a_family_of_its_own():
         ["Partial_PACC_combine", "Partial_PD_combine", "PlaceHolder_b", "OutputNode_0"]]
 
 
+def test_chained_matmul_is_attention_marked_linear():
+    g = stage_graph(C.matmul_matmul.trace(cl.f16, H=32, SQ=4096, SKV=4096, D=64))
+    assert g.lowered.family == "attention" and g.lowered.problem["linear"] and g.lowered.problem["scale"] == 1.0
+    assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}
+
+
 def test_unrecognised_program_is_refused():
     from cleave_amd.frontend import Program
 
