@@ -81,6 +81,9 @@ def op_table():
                      shapes=C.FULL["lora"], inputs=C.inputs_lora, split=cl.Split("K", (4, 8, 16)),
                      bytes=2 * (16 * 4096 + 4096 * 4096 + 4096 * 16 + 16 * 4096 + 16 * 4096),
                      flops=2 * 16 * 4096 * 4096 + 2 * 16 * 4096 * 16 * 2, bound="hbm", sets=6),
+        "rsdiv": dict(title="rows divided by their sums f16 4096x4096 (the reference's rowsum_div case)", fn=C.rowsum_div,
+                      dtype=cl.f16, shapes=dict(M=4096, N=4096), inputs=C.inputs_rows, split=False,
+                      bytes=2 * 2 * 4096 * 4096, flops=2 * 4096 * 4096, bound="hbm", sets=6),
         "mmrs": dict(title="matmul + row sum f16 (x@w).sum(-1) 4096x4096x64", fn=C.matmul_rowsum, dtype=cl.f16,
                      shapes=C.FULL["matmul_rowsum"], inputs=C.inputs_c1, split=False,
                      bytes=2 * (4096 * 64 + 64 * 4096 + 4096), flops=2 * 4096 * 4096 * 64, bound="mfma", sets=4),
@@ -404,7 +407,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,lora,mmrs,attn,qknorm,mlapf")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,lora,mmrs,rsdiv,attn,qknorm,mlapf")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")

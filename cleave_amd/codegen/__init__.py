@@ -296,6 +296,26 @@ class HipCodeGen:
             unit.templates.append("matmul_combine.hip")
             unit.launch(entry, (blocks, 1, 1), 256, 0, args)
 
+    def _emit_rowsum(self, unit, plan, params, partial, combine, fused):
+        p, op = plan.problem, plan.operands
+        if combine or (plan.split_factor or 1) > 1:
+            raise CodegenError("row reductions have no split form")
+        if p["N"] % 8:
+            raise CodegenError("row reductions read 16-byte chunks: the row length must be a multiple of 8")
+        rows = int(plan.tiling.get("ROWS_PER_BLOCK", 4))
+        if rows not in (1, 2, 4):
+            raise CodegenError("1, 2 or 4 rows per workgroup")
+        self._common(unit, plan, partial, combine)
+        for k, v in (("CL_M", p["M"]), ("CL_N", p["N"]), ("CL_DIV", bool(p["div"])), ("CL_ROWS_PER_BLOCK", rows)):
+            unit.define(k, v)
+        unit.define("CL_ARG_X", op["X"])
+        unit.define("CL_ARG_OUT", op["OUT"])
+        ins = [q for q in params if q.role in ("input", "scalar")]
+        outs = [q for q in params if q.role == "output"]
+        args = unit.signature("CL_PARTIAL_PARAMS", "CL_PARTIAL_NAME", ENTRY, ins + outs, ())
+        unit.templates.append("rowsum.hip")
+        unit.launch(ENTRY, (-(-p["M"] // rows), 1, 1), 64 * rows, 0, args)
+
     def _emit_skinny(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
         self._matmul_common(unit, plan, params, partial, combine, fused)

@@ -31,7 +31,7 @@ from .graph import ComputeOpNode, Graph, Node, OutputNode, PlaceHolderNode
 class Lowered:
     """A recognised operator: family, sizes and which placeholder plays which operand."""
 
-    family: str                       # matmul | rmsnorm_matmul | swiglu | lora | matmul_rowsum | attention | mla
+    family: str                       # matmul | rmsnorm_matmul | swiglu | lora | matmul_rowsum | rowsum | attention | mla
     problem: dict                     # sizes and flags the template needs
     operands: dict                    # role -> PlaceHolderNode
     outputs: list                     # OutputNodes in order
@@ -395,6 +395,28 @@ def _normed(view, n):
     return None
 
 
+def _try_rowsum(view, out):
+    """``x.sum(-1)`` and ``x / x.sum(-1)`` over a 2-D input (the reference's ``rowsum`` and
+    ``rowsum_div`` cases, ``tests/_graphs.py:1238-1275``)."""
+    n = view.skip(out)
+    div = False
+    if _is(n, "div") and n.scalar is None and len(n.inputs) == 2:
+        x, rs = view.ins(n)
+        if not (_is(rs, "reduce_sum") and view.ins(rs)[0] is x):
+            return None
+        div, n = True, rs
+    if not (_is(n, "reduce_sum") and view.reduce_dim(n) == -1):
+        return None
+    x = view.ins(n)[0]
+    if not isinstance(x, PlaceHolderNode):
+        return None
+    if view.is_split:
+        raise LoweringRejected("a row reduction has no split form here")
+    if len(x.shape) != 2:
+        raise LoweringRejected("row reductions are built for 2-D inputs")
+    return "rowsum", {"M": int(x.shape[0]), "N": int(x.shape[1]), "div": div}, {"X": x}
+
+
 def _try_chained_matmul(view, out):
     """``(q @ k^T) @ v`` with nothing between the products (the reference's ``matmul_matmul_bhsd``
     case, ``tests/_graphs.py:78-101``): attention without a softmax.  It is the attention family
@@ -481,8 +503,8 @@ def _try_attention(view, out):
     return "attention", prob, {"Q": q, "K": k, "V": v}
 
 
-_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_lora, _try_matmul_rowsum, _try_attention, _try_chained_matmul,
-             _try_matmul)
+_MATCHERS = (_try_rmsnorm_matmul, _try_swiglu, _try_lora, _try_matmul_rowsum, _try_rowsum, _try_attention,
+             _try_chained_matmul, _try_matmul)
 
 
 def recognize(graph: Graph) -> Lowered:
@@ -504,7 +526,7 @@ def recognize(graph: Graph) -> Lowered:
                 _check_split_axes(family, operands, view.split_axes)
             return Lowered(family, problem, operands, outs, graph, dict(view.split_axes), split_dim)
     raise LoweringRejected(f"{graph.name}: ops {graph.op_kinds()} match no kernel family "
-                           "(matmul, rmsnorm_matmul, swiglu, lora, matmul_rowsum, attention, mla)")
+                           "(matmul, rmsnorm_matmul, swiglu, lora, matmul_rowsum, rowsum, attention, mla)")
 
 
 def _check_split_axes(family, operands, split_axes):

@@ -220,6 +220,10 @@ def execute(graph, inputs, device=None) -> list:
             return _eval_matmul_combine(low, feed, out_dtype, shapes[0])
         res = _eval_matmul(low, feed, role, factor, torch_dtype(graph.dtype))
         return [r.reshape(s) for r, s in zip(res, shapes)]
+    if low.family == "rowsum":
+        x = feed[low.operands["X"].name].float()
+        total = x.sum(-1, keepdim=True)
+        return [((x / total) if low.problem["div"] else total).to(out_dtype).reshape(shapes[0])]
     if low.family == "swiglu":
         return [r.reshape(s) for r, s in zip(_eval_swiglu(low, feed, out_dtype), shapes)]
     if low.family == "lora":

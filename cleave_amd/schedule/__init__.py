@@ -32,6 +32,8 @@ def _candidates(graph, arch):
         return policy.swiglu_candidates(low, role, factor, arch)
     if fam == "matmul_rowsum":
         return policy.rowsum_candidates(low, role, factor, arch)
+    if fam == "rowsum":
+        return policy.rowsum_only_candidates(low, role, factor, arch)
     if fam == "lora":
         cands = policy.lora_candidates(low, role, factor, arch)
         if not cands:

@@ -244,6 +244,22 @@ def lora_candidates(low, role, factor, arch: Arch):
     return out
 
 
+def rowsum_only_candidates(low, role, factor, arch: Arch):
+    """Row reductions: one wave per row, 1, 2 or 4 rows per workgroup; the cost is the stream."""
+    p = low.problem
+    if (factor or 1) > 1 or p["N"] % 8:
+        return []
+    out = []
+    for rows in (4, 2, 1):
+        blocks = _ceil(p["M"], rows)
+        nbytes = p["M"] * p["N"] * 2 * (3 if p["div"] else 1)
+        score = nbytes / (arch.hbm_gbps * 1e3 * 0.6) * 2400 + 3000 + 200 * _waves_time(blocks, 8, arch) + rows
+        out.append(TileDict("rowsum", role, dict(ROWS_PER_BLOCK=rows), output_tile=[rows, p["N"] if p["div"] else 1],
+                            rstep_map={"n": 512}, n_threads=64 * rows, split_factor=factor, score=score, lds_bytes=0,
+                            est_vgprs=40))
+    return out
+
+
 # ----------------------------------------------------------------------------- few-row matmul
 def skinny_ok(low) -> bool:
     p = low.problem

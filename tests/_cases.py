@@ -42,6 +42,18 @@ def lora(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"], a: cl.Tensor["K", "R"],
 
 
 @cleave_amd.jit
+def rowsum(x: cl.Tensor["M", "N"]):
+    """Row sums (the reference's ``rowsum`` case, ``tests/_graphs.py:1238-1249``)."""
+    return x.sum(dim=-1, keepdim=True)
+
+
+@cleave_amd.jit
+def rowsum_div(x: cl.Tensor["M", "N"]):
+    """Rows divided by their sums (the reference's ``rowsum_div`` case, ``tests/_graphs.py:1252-1275``)."""
+    return x / x.sum(dim=-1, keepdim=True)
+
+
+@cleave_amd.jit
 def matmul_rowsum(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
     """Row sums of a product that is never stored (the reference's ``tests/_graphs.py:150-160``)."""
     return (x @ w).sum(dim=-1, keepdim=True)
@@ -122,6 +134,11 @@ def inputs_swiglu(shapes, seed=6, device="cpu"):
     x = torch.randn(M, K, generator=g)
     ws = [torch.randn(K, N, generator=g) / math.sqrt(K) for _ in range(2)]
     return [t.to(torch.float16).to(device) for t in (x, *ws)]
+
+
+def inputs_rows(shapes, seed=12, device="cpu"):
+    g = _gen(seed)
+    return [(torch.rand(shapes["M"], shapes["N"], generator=g) + 0.25).to(torch.float16).to(device)]
 
 
 def inputs_lora(shapes, seed=9, device="cpu"):

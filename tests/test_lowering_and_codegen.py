@@ -163,6 +163,16 @@ def test_chained_matmul_is_attention_marked_linear():
     assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}
 
 
+def test_row_reductions_are_a_family():
+    for fn, div, out_shape in ((C.rowsum, False, (4096, 1)), (C.rowsum_div, True, (4096, 4096))):
+        g = stage_graph(fn.trace(cl.f16, M=4096, N=4096))
+        assert g.lowered.family == "rowsum" and g.lowered.problem == {"M": 4096, "N": 4096, "div": div}
+        assert g.outputs[0].shape == out_shape
+        assert sorted(c.tiling["ROWS_PER_BLOCK"] for c in search_tiling(g, topk=10)) == [1, 2, 4]
+        m = parse_manifest(source_for(fn.trace(cl.f16, M=4096, N=4096), template="rowsum", tiling=dict(ROWS_PER_BLOCK=4)))
+        assert m["launches"][0]["grid"] == ["1024", "1", "1"] and m["launches"][0]["block"][0] == 256
+
+
 def test_unrecognised_program_is_refused():
     from cleave_amd.frontend import Program
 
