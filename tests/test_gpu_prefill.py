@@ -80,3 +80,23 @@ def test_causal_prefill_long_request(shared):
     check(True, [700], [700], shared=shared)
     check(False, [300, 2], [1000, 900], what="long cached prefix", shared=shared)
     check(False, [40, 33], [600, 290], what="table windows", shared=shared)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_causal_prefill_random_shapes(seed):
+    """Seeded random request lists (lengths 0..300, cached prefixes 0..500 or key windows shorter
+    than the query run, 1..6 requests, either head grouping, either key form) through the
+    LDS-shared kernel; every odd seed also through the 16-row kernel."""
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(1, 7))
+    q_lens = [int(x) for x in rng.integers(0, 301, n)]
+    kv_lens = [max(0, q + int(rng.integers(-40, 500))) if rng.random() < 0.8 else int(rng.integers(0, 60)) for q in q_lens]
+    if sum(q_lens) == 0:
+        q_lens[0] = 5
+    if sum(kv_lens) == 0:
+        kv_lens[0] = 7
+    hkv = 8 if seed % 2 else 4
+    ragged = bool((seed // 2) % 2)
+    check(ragged, q_lens, kv_lens, hkv=hkv, pad=int(rng.integers(0, 9)), what=f"random seed {seed}", shared=True)
+    if seed % 2:
+        check(ragged, q_lens, kv_lens, hkv=hkv, what=f"random seed {seed}", shared=False)
