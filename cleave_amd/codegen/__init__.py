@@ -289,6 +289,13 @@ class HipCodeGen:
             if (not p["trans_B"] and p["N"] % 8) or (p["trans_A"] and p["M"] % 8) or p["K"] % 8:
                 raise CodegenError("16-byte global chunks need the minor extent of each operand to be a multiple of 8")
             grid = (1 if rowsum else -(-p["N"] // out_bn), -(-p["M"] // tile["BM"]), batch * splits)
+            tail = int(tile.get("TAIL", 0))
+            if tail:
+                # the last `tail` tiles run as two half-height workgroups each, on a one-dimensional grid
+                if (rowsum or p["trans_A"] or batch * splits != 1 or not 0 < tail <= grid[0] * grid[1]
+                        or tile["BM"] % (32 * tile["WM"]) or p["M"] % tile["BM"]):
+                    raise CodegenError("the tail split needs row-major A, whole row tiles that halve, one batch and one split")
+                grid = (grid[0] * grid[1] + tail, 1, 1)
             # the tile images are static LDS arrays of the kernel: no dynamic LDS at launch
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, 0, self._partial_args)
         if combine:

@@ -51,6 +51,12 @@
 #ifndef CL_ROWSUM
 #define CL_ROWSUM 0
 #endif
+#ifndef CL_TAIL
+#define CL_TAIL 0
+#endif
+#ifndef CL_ASM_MFMA
+#define CL_ASM_MFMA (GD_TM * GD_TN * 4 > 128)   // wave tiles whose accumulators fill a register half
+#endif
 static_assert(CL_BK == 64, "K steps are 64 wide (128-byte K-minor rows)");
 static_assert((GD_TM & (GD_TM - 1)) == 0 && (GD_TN & (GD_TN - 1)) == 0, "wave tiles are powers of two");
 static_assert(CL_BM % 16 == 0 && CL_BN % 16 == 0, "tiles are multiples of 16");
@@ -85,6 +91,7 @@ CL_DEVICE int gd_swz_kmaj(int k) {
 // One operand of the product: how its tile is fetched and how fragments are read.
 //   EXT      tile extent along the operand's own axis (BM for A, BN for B)
 //   KMAJOR   stored with K as the major axis
+template <int V> struct GdInt { static constexpr int value = V; };
 template <bool WIDE> struct GdOffset { typedef u32 type; };
 template <> struct GdOffset<true> { typedef i64 type; };
 //   DUAL     the tile's second half (rows / columns EXT/2 ..) comes from a second tensor of the
@@ -168,25 +175,58 @@ CL_DEVICE elem8 gd_read_kmaj(const elem_t* tile, int off0, int j, int s) {
   return __builtin_bit_cast(elem8, v);
 }
 
+// The matrix op.  Through the compiler's builtin, a wave tile whose accumulators fill a whole
+// register half (8 x 8 fragments = 256 registers) comes out with the accumulators renamed from op
+// to op and copied back inside the loop (three copies per matrix op), and with the load addresses
+// spilled and reloaded between the tile loads, each reload waiting for the loads before it: 1900 us
+// on the 4096 x 14336 x 4096 product.  Written as assembly with the accumulator tied to one
+// accumulation register quadruple every op updates its registers in place (520 us).  The compiler
+// does not know such a statement is a matrix op, so what it would insert is written here: two idle
+// states ahead of the op (an operand written by a vector instruction just before), and the drain
+// between the last matrix op and the first read of an accumulator (gd_acc_drain).  Smaller wave
+// tiles compile well through the builtin (measured equal or a little faster), which stays their
+// default.
+#if CL_ASM_MFMA
+#if CL_BF16
+#define GD_MFMA_OP "v_mfma_f32_16x16x32_bf16"
+#else
+#define GD_MFMA_OP "v_mfma_f32_16x16x32_f16"
+#endif
+#define GD_MFMA(acc, a, b) asm volatile("s_nop 1\n\t" GD_MFMA_OP " %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+CL_DEVICE void gd_acc_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+CL_DEVICE f32x4 gd_acc_read(const f32x4& acc) {
+  float r0, r1, r2, r3;
+  asm volatile("v_accvgpr_read_b32 %0, %4\n\tv_accvgpr_read_b32 %1, %5\n\t"
+               "v_accvgpr_read_b32 %2, %6\n\tv_accvgpr_read_b32 %3, %7"
+               : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+               : "a"(acc[0]), "a"(acc[1]), "a"(acc[2]), "a"(acc[3]));
+  return (f32x4){r0, r1, r2, r3};
+}
+#else
+#define GD_MFMA(acc, a, b) acc = mfma16(a, b, acc)
+CL_DEVICE void gd_acc_drain() {}
+CL_DEVICE f32x4 gd_acc_read(const f32x4& acc) { return acc; }
+#endif
+
 // LDS read instructions per fragment, and the reads issued under the cover of row `i` of k block
 // `s` in GD_COMPUTE
 #define GD_A_READS (CL_TRANS_A ? 2 : 1)
 #define GD_B_READS (CL_TRANS_B ? 1 : 2)
-constexpr int gd_reads_after(int s, int i) {
+constexpr int gd_reads_after(int TM, int s, int i) {
   int n = 0;
-  if (s * GD_TM + i + 2 < 2 * GD_TM) n += GD_A_READS;
+  if (s * TM + i + 2 < 2 * TM) n += GD_A_READS;
   if (s == 0)
     for (int j = 0; j < GD_TN; ++j)
-      if (j % GD_TM == i) n += GD_B_READS;
+      if (j % TM == i) n += GD_B_READS;
   return n;
 }
-template <int S, int I>
+template <int TM, int S, int I>
 CL_DEVICE void gd_sched_rows() {
   __builtin_amdgcn_sched_group_barrier(0x008, GD_TN, 0);
-  constexpr int n = gd_reads_after(S, I);
+  constexpr int n = gd_reads_after(TM, S, I);
   if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);
-  if constexpr (I + 1 < GD_TM) gd_sched_rows<S, I + 1>();
-  else if constexpr (S == 0) gd_sched_rows<1, 0>();
+  if constexpr (I + 1 < TM) gd_sched_rows<TM, S, I + 1>();
+  else if constexpr (S == 0) gd_sched_rows<TM, 1, 0>();
 }
 
 #if CL_EMIT_PARTIAL
@@ -200,17 +240,33 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // XCD (L % 8)'s contiguous share, tiles ordered in patches of CL_GROUP_M row-tiles.
   constexpr int tiles_m = (CL_M + CL_BM - 1) / CL_BM, tiles_n = CL_ROWSUM ? 1 : (CL_N + GD_OUT_BN - 1) / GD_OUT_BN;
   constexpr int tiles = tiles_m * tiles_n;
-  int tile_id = blockIdx.y * tiles_n + blockIdx.x;
-  {
+  // CL_TAIL: the last CL_TAIL tiles (the partly filled final round of a launch that does not divide
+  // among the compute units) are each run as two workgroups of half the rows, so that the round
+  // keeps twice as many compute units busy for half as long.  The grid is then one-dimensional:
+  // the whole tiles first, two workgroups per tail tile after them, the halves of a tile on one XCD.
+  constexpr int whole = tiles - CL_TAIL;
+  int tile_id = CL_TAIL ? blockIdx.x : blockIdx.y * tiles_n + blockIdx.x;
+  int half = -1;
+  if (tile_id < whole) {
     const int xcd = tile_id % GD_XCDS, nth = tile_id / GD_XCDS;
-    constexpr int share = tiles / GD_XCDS, extra = tiles % GD_XCDS;
+    constexpr int share = whole / GD_XCDS, extra = whole % GD_XCDS;
     tile_id = xcd * share + (xcd < extra ? xcd : extra) + nth;
+  } else {
+    const int t = tile_id - whole;
+    if (CL_TAIL % GD_XCDS == 0) {
+      const int xcd = t % GD_XCDS, nth = t / GD_XCDS;
+      tile_id = whole + (nth >> 1) * GD_XCDS + xcd;
+      half = nth & 1;
+    } else {
+      tile_id = whole + (t >> 1);
+      half = t & 1;
+    }
   }
   constexpr int group_m = CL_GROUP_M < tiles_m ? CL_GROUP_M : tiles_m;
   const int band = tile_id / (group_m * tiles_n);
   const int band_rows = (tiles_m - band * group_m) < group_m ? (tiles_m - band * group_m) : group_m;
   const int in_band = tile_id - band * group_m * tiles_n;
-  const int m0 = (band * group_m + in_band % band_rows) * CL_BM, n0 = (in_band / band_rows) * GD_OUT_BN;
+  const int tile_m0 = (band * group_m + in_band % band_rows) * CL_BM, n0 = (in_band / band_rows) * GD_OUT_BN;
   const int batch = blockIdx.z / CL_SPLITS, split = blockIdx.z % CL_SPLITS;
   constexpr int k_per_split = CL_K / CL_SPLITS;
   const int k_begin = split * k_per_split;
@@ -223,8 +279,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const elem_t* A = CL_ARG_A + (i64)(batch / (GD_BATCH / CL_BATCH_A)) * CL_M * CL_K;
   const elem_t* B = CL_ARG_B + (i64)(batch / (GD_BATCH / CL_BATCH_B)) * CL_K * CL_N;
 
+  // The rest of the kernel for a workgroup that owns BM rows from m0 (BM = CL_BM, or half of it for
+  // a tail half): TM row fragments per wave.
+  auto body = [&](auto bm_tag, const int m0) {
+  constexpr int BM = decltype(bm_tag)::value;
+  constexpr int TM = BM / CL_WM / 16;
+  static_assert(TM >= 1 && (TM & (TM - 1)) == 0, "wave tiles are powers of two");
   // ---- operand movers: tile origin at K step 0 and the uniform advance per step ---------------
-  GdOperand<CL_BM, CL_TRANS_A != 0> opa;
+  GdOperand<BM, CL_TRANS_A != 0> opa;
   GdOperand<CL_BN, CL_TRANS_B == 0, CL_SWIGLU != 0> opb;
 #if CL_SWIGLU
   const i64 b_twin = reinterpret_cast<const char*>(CL_ARG_C) - reinterpret_cast<const char*>(CL_ARG_B);
@@ -253,7 +315,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // ---- this lane's fragment offsets -------------------------------------------------------------
   // wave origin inside the tile (SwiGLU: inside each half of the B tile; fragments j < TN/2 come
   // from the first half, the others from the same columns of the second)
-  const int am = wm * (CL_BM / CL_WM), bn = wn * (GD_OUT_BN / CL_WN);
+  const int am = wm * (BM / CL_WM), bn = wn * (GD_OUT_BN / CL_WN);
 #if CL_SWIGLU
 #define GD_BSEL(j, x, y) ((j) < GD_TN / 2 ? (x) : (y))
 #define GD_BJ(j) ((j) % (GD_TN / 2))
@@ -262,9 +324,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GD_BJ(j) (j)
 #endif
 #if CL_TRANS_A
-  const int a_f = gd_swz_kmaj<CL_BM>(8 * g + (c >> 2));
-  const int a_off = (8 * g + (c >> 2)) * CL_BM + 8 * (((am / 8) ^ a_f) + ((c & 3) >> 1)) + 4 * (c & 1);
-#define GD_AFRAG(tile, i, s) gd_read_kmaj<CL_BM>(tile, a_off, i, s)
+  const int a_f = gd_swz_kmaj<BM>(8 * g + (c >> 2));
+  const int a_off = (8 * g + (c >> 2)) * BM + 8 * (((am / 8) ^ a_f) + ((c & 3) >> 1)) + 4 * (c & 1);
+#define GD_AFRAG(tile, i, s) gd_read_kmaj<BM>(tile, a_off, i, s)
 #else
   const int a_off = (am + c) * 64 + ((g ^ gd_swz_kmin(am + c)) << 3);
 #define GD_AFRAG(tile, i, s) gd_read_kmin(tile, a_off, i, s)
@@ -280,9 +342,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GD_BFRAG(tile, j, s) gd_read_kmaj<CL_BN>(tile, GD_BSEL(j, b_off, b_off2), GD_BJ(j), s)
 #endif
 
-  f32x4 acc[GD_TM][GD_TN];
+  f32x4 acc[TM][GD_TN];
 #pragma unroll
-  for (int i = 0; i < GD_TM; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < GD_TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
@@ -294,27 +356,27 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // under their cover" so that no LDS latency is waited for with the matrix cores idle.
 #define GD_COMPUTE(a_tile, b_tile, NEXT)                                                            \
   {                                                                                                 \
-    elem8 af[2][GD_TM], bf[2][GD_TN];                                                               \
+    elem8 af[2][TM], bf[2][GD_TN];                                                               \
     _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) bf[0][j] = GD_BFRAG(b_tile, j, 0);           \
     af[0][0] = GD_AFRAG(a_tile, 0, 0);                                                              \
-    af[1 / GD_TM][1 % GD_TM] = GD_AFRAG(a_tile, 1 % GD_TM, 1 / GD_TM);                              \
+    af[1 / TM][1 % TM] = GD_AFRAG(a_tile, 1 % TM, 1 / TM);                              \
     _Pragma("unroll") for (int s = 0; s < 2; ++s) {                                                \
-      _Pragma("unroll") for (int i = 0; i < GD_TM; ++i) {                                          \
-        NEXT(s * GD_TM + i)                                                                         \
-        _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) acc[i][j] = mfma16(bf[s][j], af[s][i], acc[i][j]); \
-        if (s * GD_TM + i + 2 < 2 * GD_TM)                                                          \
-          af[(s * GD_TM + i + 2) / GD_TM][(i + 2) % GD_TM] =                                        \
-              GD_AFRAG(a_tile, (i + 2) % GD_TM, (s * GD_TM + i + 2) / GD_TM);                       \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                          \
+        NEXT(s * TM + i)                                                                         \
+        _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) GD_MFMA(acc[i][j], bf[s][j], af[s][i]);              \
+        if (s * TM + i + 2 < 2 * TM)                                                          \
+          af[(s * TM + i + 2) / TM][(i + 2) % TM] =                                        \
+              GD_AFRAG(a_tile, (i + 2) % TM, (s * TM + i + 2) / TM);                       \
         if (s == 0) {                                                                               \
           _Pragma("unroll") for (int j = 0; j < GD_TN; ++j)                                        \
-            if (j % GD_TM == i) bf[1][j] = GD_BFRAG(b_tile, j, 1);                                  \
+            if (j % TM == i) bf[1][j] = GD_BFRAG(b_tile, j, 1);                                  \
         }                                                                                           \
         GD_ROW_END()                                                                                \
       }                                                                                             \
     }                                                                                               \
     GD_STEP_SCHED()                                                                                 \
   }
-#if CL_SPREAD_LOADS
+#if CL_SPREAD_LOADS || CL_ASM_MFMA
 // every row of matrix ops closes with a scheduling barrier: the order of the source (this row's
 // loads of the next step, its matrix ops, the fragment reads for two rows on) is the order of the
 // instruction stream
@@ -324,7 +386,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GD_ROW_END()
 #define GD_STEP_SCHED()                                                                             \
     __builtin_amdgcn_sched_group_barrier(0x100, GD_B_READS * GD_TN + 2 * GD_A_READS, 0);            \
-    gd_sched_rows<0, 0>();
+    gd_sched_rows<TM, 0, 0>();
 #endif
   // everything this wave loaded has landed; after the barrier, everything every wave loaded
 #define GD_STEP_END()                           \
@@ -342,6 +404,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #if CL_ROWSUM
 #define GD_A_AT(kt) (a_base + (i64)((kt) % KT_K) * a_step)
 #define GD_B_AT(kt) (b_base + (i64)((kt) % KT_K) * b_step + (i64)((kt) / KT_K) * (CL_TRANS_B ? (i64)CL_BN * CL_K : (i64)CL_BN))
+#elif defined(CL_DBG_HOT)
+// (timing probe: every workgroup fetches the first tile's first two steps, which stay in L2)
+#define GD_A_AT(kt) (A + (i64)((kt) & 1) * a_step)
+#define GD_B_AT(kt) (B + (i64)((kt) & 1) * b_step)
 #else
 #define GD_A_AT(kt) (a_base + (i64)(kt) * a_step)
 #define GD_B_AT(kt) (b_base + (i64)(kt) * b_step)
@@ -353,7 +419,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)                                                         \
   {                                                                                                 \
     constexpr int ua_ = decltype(opa)::PER, ub_ = decltype(opb)::PER;                               \
-    constexpr int per_row_ = (ua_ + ub_ + 2 * GD_TM - 1) / (2 * GD_TM);                             \
+    constexpr int per_row_ = (ua_ + ub_ + 2 * TM - 1) / (2 * TM);                             \
     _Pragma("unroll") for (int q_ = (r) * per_row_; q_ < ((r) + 1) * per_row_; ++q_) {             \
       if (q_ < ua_) opa.issue_unit(q_, GD_A_AT(kt), a_lds);                                         \
       else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, GD_B_AT(kt), b_lds);                        \
@@ -393,21 +459,25 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   if constexpr (KT % 2 == 1) GD_COMPUTE(gd_a0, gd_b0, GD_NO_NEXT)     // an odd number of steps ends on stage 0
 
   // ---- epilogue: acc[i][j][r] = C[m0 + am + 16 i + c][n0 + bn + 16 j + 4 g + r] ----------------
+  gd_acc_drain();
 #if CL_ROWSUM
   {
     __syncthreads();                                  // every wave is done with the tile images
     float* red = reinterpret_cast<float*>(gd_b0);     // [BM][WN]
 #pragma unroll
-    for (int i = 0; i < GD_TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
       float sum = 0.f;
 #pragma unroll
-      for (int j = 0; j < GD_TN; ++j) sum += (acc[i][j][0] + acc[i][j][1]) + (acc[i][j][2] + acc[i][j][3]);
+      for (int j = 0; j < GD_TN; ++j) {
+        const f32x4 v = gd_acc_read(acc[i][j]);
+        sum += (v[0] + v[1]) + (v[2] + v[3]);
+      }
       sum += lane_xor(sum, lane, 16);
       sum += lane_xor(sum, lane, 32);
       if (g == 0) red[(am + 16 * i + c) * CL_WN + wn] = sum;
     }
     __syncthreads();
-    for (int r = threadIdx.x; r < CL_BM; r += GD_THREADS) {
+    for (int r = threadIdx.x; r < BM; r += GD_THREADS) {
       if (m0 + r >= CL_M) break;
       float sum = 0.f;
 #pragma unroll
@@ -418,7 +488,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 #endif
 #pragma unroll
-  for (int i = 0; i < GD_TM; ++i) {
+  for (int i = 0; i < TM; ++i) {
     const int m = m0 + am + 16 * i + c;
     if (m >= CL_M) continue;
 #if CL_SWIGLU
@@ -427,10 +497,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       const int n = n0 + bn + 16 * j + 4 * g;
       if (n >= CL_N) continue;
       elem4 y;
+      const f32x4 up = gd_acc_read(acc[i][j]), gates = gd_acc_read(acc[i][j + GD_TN / 2]);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float gate = acc[i][j + GD_TN / 2][r];
-        y[r] = to_elem(acc[i][j][r] * gate / (1.0f + __expf(-gate)));
+        const float gate = gates[r];
+        y[r] = to_elem(up[r] * gate / (1.0f + __expf(-gate)));
       }
       *reinterpret_cast<elem4*>(CL_ARG_OUT + (i64)m * CL_N + n) = y;
     }
@@ -439,16 +510,26 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     for (int j = 0; j < GD_TN; ++j) {
       const int n = n0 + bn + 16 * j + 4 * g;
       if (n >= CL_N) continue;
+      const f32x4 v = gd_acc_read(acc[i][j]);
 #if CL_SPLITS > 1
-      *reinterpret_cast<f32x4*>(CL_ARG_PACC + (((i64)split * GD_BATCH + batch) * CL_M + m) * CL_N + n) = acc[i][j];
+      *reinterpret_cast<f32x4*>(CL_ARG_PACC + (((i64)split * GD_BATCH + batch) * CL_M + m) * CL_N + n) = v;
 #else
       elem4 y;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[i][j][r]);
+      for (int r = 0; r < 4; ++r) y[r] = to_elem(v[r]);
       *reinterpret_cast<elem4*>(CL_ARG_OUT + ((i64)batch * CL_M + m) * CL_N + n) = y;
 #endif
     }
 #endif  // CL_SWIGLU
   }
+  };
+#if CL_TAIL
+  static_assert(!CL_ROWSUM && !CL_TRANS_A && GD_BATCH == 1 && CL_SPLITS == 1, "the tail split halves row-major A tiles of an unsplit, unbatched product");
+  if (half >= 0) {
+    body(GdInt<CL_BM / 2>{}, tile_m0 + half * (CL_BM / 2));
+    return;
+  }
+#endif
+  body(GdInt<CL_BM>{}, tile_m0);
 }
 #endif  // CL_EMIT_PARTIAL

@@ -185,12 +185,25 @@ class CompiledKernel:
         return tuple(s if isinstance(s, int) else eval_extent(s, dims) for s in p.shape)
 
     def _materialise(self, bound, dims, device):
+        import os
+
         import torch
+
+        # CLEAVE_POISON_BUFFERS=1: fresh outputs and scratch start as NaN instead of whatever the
+        # allocator hands back, so that a kernel which leaves part of a buffer unwritten (or reads
+        # scratch it has not written) fails its comparison every time instead of now and then.
+        poison = bool(os.environ.get("CLEAVE_POISON_BUFFERS"))
+
+        def fresh(shape, dtype):
+            t = torch.empty(shape, dtype=dtype, device=device)
+            if poison and t.is_floating_point():
+                t.fill_(float("nan"))
+            return t
 
         outs = []
         for p in self.params:
             if p.role == "output" and p.name not in bound:
-                t = torch.empty(self._shape(p, dims), dtype=getattr(torch, p.dtype), device=device)
+                t = fresh(self._shape(p, dims), getattr(torch, p.dtype))
                 bound[p.name] = t
                 outs.append(t)
             elif p.role == "output":
@@ -202,7 +215,7 @@ class CompiledKernel:
             shape = self._shape(p, dims)
             key = (owner, shape, str(device))
             if key not in self._scratch:
-                self._scratch[key] = torch.empty(shape, dtype=getattr(torch, p.dtype), device=device)
+                self._scratch[key] = fresh(shape, getattr(torch, p.dtype))
             bound[p.name] = self._scratch[key]
         return outs
 

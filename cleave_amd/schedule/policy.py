@@ -159,6 +159,14 @@ def gemm_dma_candidates(low, role, factor, arch: Arch):
         tiling = dict(BM=bm, BN=bn, BK=64, WM=wm, WN=wn)
         out.append(TileDict("gemm_dma", role, tiling, output_tile=[bm, bn], rstep_map={"k": 64}, n_threads=threads,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+        # A last round that fills at most half of the machine: its tiles as two half-height
+        # workgroups each (row-major A, one workgroup per compute unit, unsplit, unbatched).
+        tail = blocks % arch.compute_units
+        if (blocks > arch.compute_units and 0 < tail <= arch.compute_units // 2 and per_cu == 1 and splits == 1
+                and batch == 1 and not p["trans_A"] and tm >= 2 and M % bm == 0):
+            out.append(TileDict("gemm_dma", role, dict(tiling, TAIL=tail), output_tile=[bm, bn], rstep_map={"k": 64},
+                                n_threads=threads, split_factor=factor, score=(passes - 0.45) * pass_clk,
+                                lds_bytes=lds, est_vgprs=vgprs))
     return out
 
 

@@ -71,6 +71,30 @@ def test_matmul_gemm_dma(tiling, split):
     _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling, split=split)
 
 
+@pytest.mark.parametrize("tiling", [dict(BM=64, BN=64, BK=64, WM=2, WN=2, TAIL=24), dict(BM=64, BN=64, BK=64, WM=2, WN=2, TAIL=5),
+                                    dict(BM=256, BN=128, BK=64, WM=4, WN=2, TAIL=6),
+                                    dict(BM=256, BN=256, BK=64, WM=2, WN=2, TAIL=8),
+                                    dict(BM=128, BN=128, BK=64, WM=2, WN=2, TAIL=28, ASM_MFMA=1)],
+                         ids=lambda t: "x".join(str(v) for v in t.values()))
+def test_matmul_gemm_dma_split_tail(tiling):
+    """The last tiles of the launch run as two half-height workgroups each (both orders of the
+    tail workgroups: halves of a tile on one XCD when the tail is a multiple of eight, neighbours
+    otherwise); ragged columns; the matrix op as builtin and as assembly."""
+    fn, dt, mk = C.CASES["c1"]
+    shapes = dict(M=512, N=776, K=576)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling)
+    if tiling["BM"] == 64:
+        prog = matmul_nt.trace(cl.bf16, **shapes)
+        g = torch.Generator(device="cpu").manual_seed(5)
+        ins = [((torch.rand(*shp, generator=g) * 2 - 1) / 24).to(torch.bfloat16) for shp in ((512, 576), (776, 576))]
+        want = po.evaluate(prog, ins)[0]
+        for asm in (0, 1):
+            kernel = kernel_for(prog, template="gemm_dma", tiling=dict(tiling, ASM_MFMA=asm))
+            print(f"case matmul_nt bf16 gemm_dma {tiling} asm={asm}", flush=True)
+            got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+            np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
 def test_matmul_gemm_dma_bf16():
     shapes = dict(M=192, N=256, K=384)
     prog = C.matmul.trace(cl.bf16, **shapes)
