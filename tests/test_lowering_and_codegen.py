@@ -245,6 +245,27 @@ def test_paged_signature_matches_the_reference_operator():
     assert m["launches"][0]["grid"] == ["(batch * 8) * 1", "8", "1"]
 
 
+def test_split_tail_of_the_direct_to_lds_matmul():
+    """A launch whose last round fills at most half the compute units is also offered with that
+    round's tiles run as two half-height workgroups each: one-dimensional grid, whole tiles first;
+    refused where the row tiles are ragged or the A operand is stored K-major."""
+    g = stage_graph(C.matmul.trace(cl.f16, M=4096, N=14336, K=4096))
+    tails = [c for c in search_tiling(g, topk=10_000) if c.tiling.get("TAIL")]
+    assert tails and all(c.template == "gemm_dma" for c in tails)
+    big = next(c for c in tails if (c.tiling["BM"], c.tiling["BN"]) == (256, 256))
+    assert big.tiling["TAIL"] == (16 * 56) % 256 == 128
+    m = parse_manifest(HipCodeGen().gen(apply_tiling(big)))
+    assert m["launches"][0]["grid"] == [str(16 * 56 + 128), "1", "1"]
+    # 1024 tiles of 256 x 224 would be whole rounds; 896 + 0 tail tiles never carry the knob
+    even = stage_graph(C.matmul.trace(cl.f16, M=4096, N=16384, K=4096))
+    assert not [c for c in search_tiling(even, topk=10_000)
+                if c.tiling.get("TAIL") and (c.tiling["BM"], c.tiling["BN"]) == (256, 256)]
+    ragged = stage_graph(C.matmul.trace(cl.f16, M=4000, N=14336, K=4096))
+    with pytest.raises(CodegenError, match="tail split"):
+        HipCodeGen().gen(apply_tiling(TileDict("gemm_dma", "main", dict(BM=256, BN=256, BK=64, WM=4, WN=2, TAIL=8),
+                                               flat_graph=ragged)))
+
+
 def test_codegen_refuses_impossible_plans():
     g = stage_graph(C.matmul.trace(cl.f16, M=128, N=128, K=4096))
     with pytest.raises(CodegenError, match="multiple"):
