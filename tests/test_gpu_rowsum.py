@@ -31,7 +31,7 @@ def _check(fn, dtype, shapes, rows=None, seed=3):
 @pytest.mark.parametrize("rows", [1, 2, 4])
 @pytest.mark.parametrize("fn", [C.rowsum, C.rowsum_div], ids=["sum", "div"])
 def test_row_reductions(fn, rows):
-    for n in (8, 504, 512, 520, 2048, 2056, 4104):
+    for n in (8, 504, 512, 520, 2048, 2056, 4104, 8192, 8704):     # (whole 512-element pieces up to 8192 stay in registers)
         _check(fn, cl.f16, dict(M=37, N=n), rows)
 
 
