@@ -43,7 +43,7 @@ def log(*a):
 # ----------------------------------------------------------------------------- operator table
 def op_table():
     import cleave_amd.lang as cl
-    from tests import _cases as C
+    from cleave_amd import examples as C
 
     return {
         "c1": dict(title="matmul f16 128x128x4096", fn=C.matmul, dtype=cl.f16, shapes=C.FULL["c1"], inputs=C.inputs_c1,
@@ -52,7 +52,7 @@ def op_table():
                    shapes=C.FULL["c2"], inputs=C.inputs_c2, split=cl.Split("K", (2, 4, 8, 16)), bytes=90_669_056,
                    flops=1_442_840_576, bound="hbm", sets=6),
         "c3": dict(title="GQA decode f16 B=8 Hq=32 Hkv=8 D=128 SKV=8192 exact softmax", fn=C.gqa_decode_exact,
-                   dtype=cl.f16, shapes=C.FULL["c3"], inputs=C.inputs_c3, split=cl.Split("SKV", (4, 8, 16)),
+                   dtype=cl.f16, shapes=C.FULL["c3"], inputs=C.inputs_c3, split=cl.Split("SKV", (8, 16, 32)),
                    bytes=268_566_528, flops=1_073_741_824, bound="hbm", sets=3),
         "c4": dict(title="MLA decode bf16 B=16 H=128 512+64 SKV=4096", fn=C.mla_decode, dtype=cl.bf16,
                    shapes=C.FULL["c4"], inputs=C.inputs_c4, split=cl.Split("SKV", (2, 4, 8, 16)), bytes=79_953_920,
@@ -90,25 +90,44 @@ def op_table():
     }
 
 
+STREAM_GBPS = None     # read-only streaming rate measured on this box at start-up (run_stream_probe)
+
+
 def roofline(bound, nbytes, flops, us, traffic=None):
     if bound == "mfma":
         achieved = flops / us / 1e6
         return {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_TFLOPS, 4), "traffic": traffic}
     achieved = nbytes / us / 1e3
-    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_GBPS, 4), "traffic": traffic}
+    out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+           "frac": round(achieved / HBM_GBPS, 4), "traffic": traffic}
+    if STREAM_GBPS:
+        # second fraction: against what a plain read-only stream reaches on this box in this run
+        out["measured_stream_peak"] = round(STREAM_GBPS, 1)
+        out["frac_of_measured_stream"] = round(achieved / STREAM_GBPS, 4)
+    return out
 
 
-def measured_traffic(name):
+def _plan_key(plan):
+    """A plan label without the candidate's rank in its search (``#7``): ranks move between runs."""
+    import re
+
+    return re.sub(r"#\d+ ", "", plan or "")
+
+
+def measured_traffic(name, plan=None):
     """HBM bytes per launch of the op's dominant kernel as counted by the profiler's FETCH_SIZE and
-    WRITE_SIZE passes (scaled by the copy probe) and recorded in profiles/traffic.json, or None."""
+    WRITE_SIZE passes (scaled by the copy probe) and recorded in profiles/traffic.json; None when
+    there is no record, or when the record is of another plan than the one just selected."""
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get(name, {}).get("traffic_bytes")
+            rec = json.load(f).get(name, {})
     except (OSError, ValueError):
         return None
+    if plan is not None and _plan_key(rec.get("plan")) != _plan_key(plan):
+        return None
+    return rec.get("traffic_bytes")
 
 
 # ----------------------------------------------------------------------------- dense operators
@@ -151,7 +170,7 @@ def save_choice(kernels_dir, name, source, info):
         json.dump(info, g)
 
 
-def run_dense(name, op, steps, warmup, search_iters, kernels_dir=None):
+def run_dense(name, op, steps, warmup, search_iters, kernels_dir=None, ramp_s=0.0):
     import contextlib
 
     import torch
@@ -181,6 +200,11 @@ def run_dense(name, op, steps, warmup, search_iters, kernels_dir=None):
         log(f"[{name}] selected kernel read from {kernels_dir} (no search): {info['plan']}")
     fused = compiled(source)
     sets = [[t.cuda() for t in op["inputs"](op["shapes"], seed=100 + i)] for i in range(op["sets"])]
+    if ramp_s:
+        # matrix-bound kernels are timed at the clocks they settle to under load: the warm-up is as
+        # many launches as fill ramp_s seconds, whatever --warmup says
+        first = fused.time(*sets[0], warmup=2, iters=5, rotate=sets[1:])
+        warmup = max(warmup, int(math.ceil(ramp_s * 1e3 / max(first, 1e-3))))
     ms = fused.time(*sets[0], warmup=warmup, iters=steps, rotate=sets[1:])
     us = ms * 1e3
     dom_us = fused.time(*sets[0], warmup=warmup, iters=steps, rotate=sets[1:], only=[0]) * 1e3
@@ -191,7 +215,7 @@ def run_dense(name, op, steps, warmup, search_iters, kernels_dir=None):
            "graph_replay_us": round(graph_us, 3),
            **info,
            "hbm": roofline("hbm", op["bytes"], op["flops"], us), "mfma": roofline("mfma", op["bytes"], op["flops"], us)}
-    out["roofline"] = roofline(op["bound"], op["bytes"], op["flops"], dom_us, measured_traffic(name))
+    out["roofline"] = roofline(op["bound"], op["bytes"], op["flops"], dom_us, measured_traffic(name, info["plan"]))
     out["algorithmic_bytes"], out["algorithmic_flops"] = op["bytes"], op["flops"]
     return out, program
 
@@ -274,12 +298,13 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
     graph_us = k.time(*args, warmup=warmup, iters=max(steps, 20), graph_batch=20) * 1e3
     nbytes = sum(lens) * hkv * d * 2 * 2 + total_pages * 4 + 2 * 32 * hq * d * 2 + 32 * hq * 4 + 33 * 4 + 32 * 4
     flops = 4 * sum(lens) * hq * d
+    plan_label = " ".join(f"{a}={b}" for a, b in cfg.items())
     res = {"op": "c5", "workload": f"paged GQA decode f16, 32 requests ({sum(lens)} tokens), page 64, 300k-page pool",
            "best_us": round(us, 3), "dominant_kernel_us": round(dom, 3), "graph_replay_us": round(graph_us, 3),
            "variant": f"chunked items of {cfg['chunk_pages']} pages" if cfg.get("chunk_pages") else f"split-kv={cfg['split']}",
-           "plan": " ".join(f"{a}={b}" for a, b in cfg.items()), "candidates": tried, "validated": valid,
+           "plan": plan_label, "candidates": tried, "validated": valid,
            "hbm": roofline("hbm", nbytes, flops, us), "mfma": roofline("mfma", nbytes, flops, us),
-           "roofline": roofline("hbm", nbytes, flops, dom, measured_traffic("c5")), "algorithmic_bytes": nbytes,
+           "roofline": roofline("hbm", nbytes, flops, dom, measured_traffic("c5", plan_label)), "algorithmic_bytes": nbytes,
            "algorithmic_flops": flops}
     if with_cpu:
         from oracle import paged_oracle
@@ -300,7 +325,8 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
         dt = time.perf_counter() - t0
         tokens = sum(lens[b] for b in order)
         res["cpu_us"] = round(dt * 1e6 * sum(lens) / tokens, 1)
-        res["cpu_sample"] = f"2 shortest requests ({tokens} of {sum(lens)} tokens), scaled by token count"
+        res["cpu_sample"] = (f"extrapolated: the 2 shortest requests ({tokens} of {sum(lens)} tokens) timed, scaled "
+                             f"by token count")
     del args, want
     torch.cuda.empty_cache()
     return res
@@ -322,7 +348,7 @@ def run_dynamic(names=None):
     from cleave_amd.dynamic import OPERATORS
     from cleave_amd.dynamic import workloads as wl
     from cleave_amd.runtime.autotune import geomean
-    from tests import _cases as C
+    from cleave_amd import examples as C
 
     out = []
     for name, op in OPERATORS.items():
@@ -402,6 +428,47 @@ def run_copy(steps, warmup, mib=1024):
             "roofline": roofline("hbm", 2 * n, 0, us)}
 
 
+READ_SOURCE = r"""
+extern "C" __global__ __launch_bounds__(256) void read_probe(const uint4* __restrict__ src, uint4* __restrict__ sink,
+                                                             unsigned long long n16) {
+  unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
+  const unsigned long long stride = (unsigned long long)gridDim.x * 256;
+  uint4 acc = {0u, 0u, 0u, 0u};
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc.x ^= a.x ^ b.x ^ c.x ^ d.x; acc.y ^= a.y ^ b.y ^ c.y ^ d.y;
+    acc.z ^= a.z ^ b.z ^ c.z ^ d.z; acc.w ^= a.w ^ b.w ^ c.w ^ d.w;
+  }
+  for (; i < n16; i += stride) { const uint4 a = src[i]; acc.x ^= a.x; acc.y ^= a.y; acc.z ^= a.z; acc.w ^= a.w; }
+  if ((acc.x & acc.y & acc.z & acc.w) == 0x9e3779b9u) sink[threadIdx.x] = acc;   // (keeps the loads alive)
+}
+"""
+
+
+def run_stream_probe(mib=2048, steps=10, warmup=3):
+    """GB/s of a read-only stream over ``mib`` MiB (well beyond the 256 MB last-level cache): what
+    the memory system of this box returns to a kernel that does nothing else."""
+    import torch
+
+    from cleave_amd.runtime import shim
+
+    n = mib << 20
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    sink = torch.zeros(256 * 16, dtype=torch.uint8, device="cuda")
+    code, _ = shim.compile_source(READ_SOURCE, name="read_probe.hip")
+    mod = shim.Module(code)
+    args = shim.PackedArgs([("ptr", src.data_ptr()), ("ptr", sink.data_ptr()), ("u64", n // 16)])
+    best = 0.0
+    for blocks in (256 * 8, 256 * 16):
+        desc = shim.make_desc(mod.function("read_probe"), (blocks,), (256,), 0, args)
+        ms = shim.time_launches([desc], torch.cuda.current_stream().cuda_stream, warmup, steps)
+        best = max(best, n / ms / 1e6)
+    torch.cuda.synchronize()
+    del src
+    torch.cuda.empty_cache()
+    return best
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -424,6 +491,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
     torch.zeros(1, device="cuda")
+    global STREAM_GBPS
+    STREAM_GBPS = run_stream_probe()
+    log(f"[probe] read-only stream: {STREAM_GBPS:.0f} GB/s ({STREAM_GBPS / HBM_GBPS:.2f} of the published peak)")
     ops = op_table()
     wanted = [o.strip() for o in args.ops.split(",") if o.strip()]
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
@@ -440,8 +510,10 @@ def main():
         if name == "c5":
             results[name] = run_paged(max(10, args.steps // 4), max(2, args.warmup // 4), not args.no_cpu, args.kernels)
             continue
-        steps = args.steps if name not in ("mm", "swiglu", "attn", "qknorm", "mlapf") else max(10, args.steps // 10)
-        res, program = run_dense(name, ops[name], steps, args.warmup, args.search_iters, args.kernels)
+        heavy = ops[name]["bound"] == "mfma" and ops[name]["flops"] > 1e11
+        steps = max(50, args.steps // 4) if heavy else args.steps
+        res, program = run_dense(name, ops[name], steps, args.warmup, args.search_iters, args.kernels,
+                                 ramp_s=0.3 if heavy else 0.0)
         if not args.no_cpu and ops[name].get("cpu", True):     # (the large attention cases would take the oracle minutes)
             cpu_us, runs = cpu_dense(program, ops[name], budget_s=8.0 if name != "c4" else 15.0)
             res["cpu_us"] = round(cpu_us, 1)

@@ -525,7 +525,10 @@ class HipCodeGen:
         emit_lse = bool(p.get("emit_lse"))
         self._attn_common(unit, plan, params, partial, combine, fused, p["ckv"], total_rows, emit_lse)
         if int(t.get("XW", 0)):
-            return self._emit_mla_decode_xw(unit, plan, partial, combine, total_rows)
+            # The cross-wave form (64 heads per workgroup, weights exchanged through LDS) was
+            # withdrawn: it measured level with this kernel and its split form once returned a
+            # wrong result whose cause was never found.
+            raise CodegenError("tiling XW=1 (cross-wave MLA decode) is withdrawn; use WAVES/HG/VSPLIT/STAGES")
         waves, hg, stages = int(t.get("WAVES", 4)), int(t.get("HG", 1)), int(t.get("STAGES", 3))
         vsplit = int(t.get("VSPLIT", 1))
         if waves not in (1, 2, 4, 8):
@@ -603,34 +606,6 @@ class HipCodeGen:
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv(({batch_name} * {p['heads']}) * {p['ckv'] // 4}, 256)", 1, 1), 256, 0, args)
-
-    def _emit_mla_decode_xw(self, unit, plan, partial, combine, total_rows):
-        """The 64-heads-per-workgroup kernel: score product shared out by (token half, head half),
-        value product by feature quarter, softmax weights exchanged through LDS."""
-        p, t, op = plan.problem, plan.tiling, plan.operands
-        if p["heads"] % 64 or p["ckv"] % 256 or p["kpe"] % 64:
-            raise CodegenError(f"the cross-wave MLA template needs heads % 64 == 0, latent width % 256 == 0 and rope "
-                               f"width % 64 == 0, got {p['heads']} / {p['ckv']} / {p['kpe']}")
-        for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_SKV", p["skv"]),
-                     ("CL_BATCH", p["batch"])):
-            unit.define(k, v)
-        for k in t:
-            if k.startswith("DBG_"):
-                unit.define(f"CL_{k}", 1)
-        for knob in ("QA", "UNITS_AHEAD", "SG", "DMA_STAGGER"):
-            if knob in t:
-                unit.define(f"CL_{knob}", int(t[knob]))
-        unit.define("CL_PO_ELEM", 1)
-        unit.define("CL_SCALE_LOG2E", _f(float(p["scale"]) * LOG2E))
-        for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE")):
-            if role in op:
-                unit.define(macro, op[role])
-        unit.templates += ["mla_decode_xw.hip", "attn_combine.hip"]
-        if partial:
-            unit.launch(ENTRY, (p["batch"] * (p["heads"] // 64), plan.split_factor or 1, 1), 256, 0, self._partial_args)
-        if combine:
-            entry, args = self._combine_args
-            unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)
 
 
 def parse_manifest(source: str) -> dict:

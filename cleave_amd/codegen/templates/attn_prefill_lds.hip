@@ -99,12 +99,12 @@ CL_DEVICE int pl_clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? h
 template <int OFF>
 CL_DEVICE void pl_dma16(const void* gptr, unsigned lds_byte) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
-               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory");
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory", "m0");
 }
 // 4 bytes per lane, the same way
 CL_DEVICE void pl_dma4(const void* gptr, unsigned lds_byte) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
-               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)) : "memory");
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)) : "memory", "m0");
 }
 
 template <int I> struct PlC { static constexpr int value = I; };

@@ -143,7 +143,7 @@ struct GdOperand {
       const unsigned lds_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)(lds + u * 512);
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                    :: "v"(reinterpret_cast<const char*>(base) + goff[i]), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
-                   : "memory");
+                   : "memory", "m0");
 #else
       __builtin_amdgcn_global_load_lds((gd_gbl_void*)(reinterpret_cast<const char*>(base) + goff[i]),
                                        (gd_lds_void*)(lds + u * 512), 16, 0, 0);

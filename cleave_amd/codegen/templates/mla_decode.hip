@@ -96,7 +96,7 @@ template <int OFF>
 CL_DEVICE void ml_dma16(const void* gptr, unsigned lds_byte) {
   // (readfirstlane: the LDS address is uniform by construction, the operand must be scalar by type)
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
-               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory");
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory", "m0");
 }
 
 // A loading wave (the first four at most) takes, of every panel, the 8-token groups

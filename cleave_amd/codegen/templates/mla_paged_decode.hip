@@ -65,7 +65,7 @@ CL_DEVICE int mp_clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? h
 template <int OFF>
 CL_DEVICE void mp_dma16(const void* gptr, unsigned lds_byte) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
-               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory");
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory", "m0");
 }
 
 // panels P.. of row group RG (token rows 8 RG + lane / 8 of the step) from this lane's row

@@ -1,4 +1,4 @@
-"""Helpers that drive lower -> tiling -> codegen -> compile without the pipeline layer."""
+"""Helpers that drive lower -> tiling -> codegen -> compile without the search (explicit template and tiling in, callable kernel out)."""
 
 from __future__ import annotations
 

@@ -56,8 +56,13 @@ _LDS_MARKER = "LDS limit exceeded"
 _TRACEBACK_LINES = 20
 
 
+MAX_GPU_PROCESSES = 16     # processes that may hold the one GPU at once (parent included)
+
+
 def _effective_compile_and_run_parallelism(max_parallel, io_bytes):
-    """Cap workers so their inputs + outputs fit in 80 % of the free device memory."""
+    """Cap workers so their inputs + outputs fit in 80 % of the free device memory, and so that
+    workers plus this process stay within the number of processes one GPU is shared by."""
+    max_parallel = min(max_parallel, MAX_GPU_PROCESSES - 1)
     try:
         import torch
 

@@ -37,8 +37,6 @@ def _waves_time(blocks, per_cu, arch: Arch):
     return _ceil(blocks, max(1, per_cu * arch.compute_units))
 
 
-CROSS_WAVE_MLA = False     # whether the search includes the cross-wave MLA decode kernel
-
 # ----------------------------------------------------------------------------- GEMM
 def gemm_lds_bytes(bm, bn, bk, norm=False):
     return 2 * (bm + bn) * bk * 2 + (bm * 4 if norm else 0)
@@ -450,25 +448,6 @@ def mla_candidates(low, role, factor, arch: Arch):
         out.append(TileDict("mla_decode", role, dict(WAVES=waves, HG=hg, VSPLIT=vsplit, STAGES=stages),
                             output_tile=[heads_per_block, p["ckv"]], rstep_map={"kv": 32}, n_threads=waves * 64,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
-    # 64 heads per workgroup with the products shared out over four waves two ways (scores by
-    # token half x head half, values by feature quarter): about half the LDS operand traffic
-    # per matrix op of the kernels above, four images of the step in LDS
-    # Not searched by default (CROSS_WAVE_MLA): it measures level with the kernels above, and its split
-    # form has once given a wrong result in a long test session (never alone, never reproduced; cause
-    # not found).  An explicit tiling XW=1 still builds it.
-    if CROSS_WAVE_MLA and p["heads"] % 64 == 0 and p["ckv"] % 256 == 0:
-        lds = mla_lds_bytes(p["ckv"], p["kpe"], 4) + 2 * 64 * 32 * 2 + 4 * 64 * 4 + 8
-        if lds <= arch.lds_bytes:
-            blocks = p["batch"] * (p["heads"] // 64) * splits
-            passes = _waves_time(blocks, 1, arch)
-            steps = _ceil(_ceil(p["skv"], 32), splits)
-            mfma_clk = (2 * (d // 32) + 4 * (p["ckv"] // 64) + 1) * 18
-            util = min(1.0, blocks / arch.compute_units)
-            partial_clk = (4 * splits * p["batch"] * p["heads"] * p["ckv"]) / (arch.hbm_gbps * 1e3 * 0.6) * 2400 \
-                if splits > 1 else 0.0
-            score = passes * (steps + 1) * (mfma_clk + 400) * (1.0 + 0.3 * (1 - util)) + 8000 + partial_clk
-            out.append(TileDict("mla_decode", role, dict(XW=1), output_tile=[64, p["ckv"]], rstep_map={"kv": 32},
-                                n_threads=256, split_factor=factor, score=score, lds_bytes=lds, est_vgprs=400))
     return out
 
 

@@ -15,8 +15,8 @@ import cleave_amd
 import cleave_amd.lang as cl
 from cleave_amd.core.errors import CompileError, SpecError
 from cleave_amd.runtime import shim
-from tests import _cases as C
-from tests._lowlevel import source_for, stage_graph
+from cleave_amd import examples as C
+from cleave_amd.pipeline.direct import source_for, stage_graph
 
 ROOT = Path(__file__).resolve().parents[1]
 

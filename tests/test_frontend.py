@@ -9,7 +9,7 @@ import cleave_amd
 import cleave_amd.lang as cl
 from cleave_amd.core.errors import CleaveError, SpecError
 from cleave_amd.frontend import Program, trace
-from tests import _cases as C
+from cleave_amd import examples as C
 
 
 def softmax(x: cl.Tensor["R", "C"]):

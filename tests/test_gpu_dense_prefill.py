@@ -11,8 +11,8 @@ import torch
 import cleave_amd.lang as cl
 from cleave_amd import pipeline as P
 from oracle import program_oracle
-from tests import _cases as C
-from tests._lowlevel import kernel_for, stage_graph
+from cleave_amd import examples as C
+from cleave_amd.pipeline.direct import kernel_for, stage_graph
 
 pytestmark = pytest.mark.gpu
 

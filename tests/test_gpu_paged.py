@@ -11,7 +11,7 @@ from cleave_amd.dynamic.paging import (PAGED_DECODE_SLAB, CombineTiling, DenseAt
 from cleave_amd.dynamic.paging.apply import _paged_outputs, _paged_params, _plan
 from cleave_amd.runtime.compile import _compile, _load_main_kernel_from_code
 from oracle import paged_oracle
-from tests import _cases as C
+from cleave_amd import examples as C
 
 pytestmark = pytest.mark.gpu
 

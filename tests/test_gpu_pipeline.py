@@ -12,7 +12,7 @@ import cleave_amd
 import cleave_amd.lang as cl
 from cleave_amd import pipeline as P
 from oracle import paged_oracle, program_oracle
-from tests import _cases as C
+from cleave_amd import examples as C
 
 pytestmark = pytest.mark.gpu
 SHAPES = dict(M=128, N=128, K=512)   # K / 8 splits is still a whole 64-wide step

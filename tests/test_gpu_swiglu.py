@@ -12,8 +12,8 @@ import cleave_amd
 import cleave_amd.lang as cl
 from cleave_amd import pipeline as P
 from oracle import program_oracle
-from tests import _cases as C
-from tests._lowlevel import kernel_for
+from cleave_amd import examples as C
+from cleave_amd.pipeline.direct import kernel_for
 
 pytestmark = pytest.mark.gpu
 

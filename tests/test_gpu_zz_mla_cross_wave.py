@@ -1,17 +1,23 @@
-"""GPU parity of the cross-wave MLA decode kernel (tiling XW=1, built only on request) against the
-numpy oracle.  Collected last: its split form has once given a wrong result late in a long session
-(cause not found), and a failure here must not hide any other test."""
+"""GPU parity cases of the cross-wave MLA decode kernel (tiling XW=1) against the numpy oracle.
+
+The kernel is withdrawn: its split form once returned a wrong result (20 372 of 32 768 elements, late
+in a long session, never alone), reading the flag / candidate / reference handshake and the load
+accounting found no cause, and it measured no faster than the one-wave-per-head-set kernel.  The code
+generator now refuses XW=1, so these cases are skipped; they stay as the cases to run should the kernel
+ever come back with the cause known."""
 
 import numpy as np
 import pytest
 import torch
 
 from oracle import program_oracle as po
-from tests import _cases as C
-from tests._lowlevel import kernel_for
+from cleave_amd import examples as C
+from cleave_amd.pipeline.direct import kernel_for
 from tests.test_gpu_kernels import ATOL, RTOL, _check
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skip(reason="cross-wave MLA decode kernel withdrawn: one unexplained wrong result of its "
+                                      "split form; the code generator refuses tiling XW=1")]
 
 
 def test_mla_decode_cross_wave_small():

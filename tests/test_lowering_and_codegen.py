@@ -14,8 +14,8 @@ from cleave_amd.lower import to_bundles
 from cleave_amd.lower.stages import partial_buffers, split_stages
 from cleave_amd.schedule import apply_tiling, search_tiling
 from cleave_amd.schedule.hint import TileDict
-from tests import _cases as C
-from tests._lowlevel import source_for, stage_graph
+from cleave_amd import examples as C
+from cleave_amd.pipeline.direct import source_for, stage_graph
 
 STRUCT = Path(__file__).parent / "golden" / "graph_structures"
 

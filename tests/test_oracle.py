@@ -11,7 +11,7 @@ import torch
 import cleave_amd.lang as cl
 from cleave_amd.frontend import Program
 from oracle import paged_oracle, program_oracle as po
-from tests import _cases as C
+from cleave_amd import examples as C
 
 GOLD = Path(__file__).parent / "golden"
 
