@@ -1,5 +1,6 @@
 // libcleave_hip.so: hiprtc compile, module load, launch and event timing behind a C ABI.
-// Host code only; the kernels themselves are generated source text compiled at run time.
+// The operators' kernels are generated source text compiled at run time; the only device code in
+// this file is the fixed scratch array of chip_launch_seq_fixed_scratch and its fill kernel.
 #include "cleave_hip.h"
 
 #include <hip/hip_runtime.h>
@@ -93,6 +94,45 @@ int launch_one(const chip_launch_desc& d, void** args, hipStream_t stream) {
   }
   HIP_TRY(hipModuleLaunchKernel(f, d.grid[0], d.grid[1], d.grid[2], d.block[0], d.block[1], d.block[2],
                                 d.lds_bytes, stream, args, nullptr));
+  return CHIP_OK;
+}
+
+}  // namespace
+
+// ---- fixed scratch: device memory for callers that cannot allocate ---------------------------
+// One array per GPU, part of this library's code object, held until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress: the device address it resolves
+// to (one per GPU) is what kernels, and the fill below, are given.
+static __device__ __align__(256) unsigned char scratch[CHIP_FIXED_SCRATCH_BYTES];
+
+static __global__ void __launch_bounds__(256) chip_scratch_fill_zero(uint4* p, unsigned long long n16) {
+  unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x;
+  const unsigned long long stride = (unsigned long long)gridDim.x * 256;
+  for (; i < n16; i += stride) p[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+constexpr int kMaxSeq = 8;          // launches per call of the fixed-scratch entry point
+constexpr int kMaxArgs = 64;        // arguments per launch there
+
+// Device address of `scratch` on the current device, resolved once per device with that device
+// current (every GPU holds its own copy of the array at its own address).
+int fixed_scratch_ptr(unsigned char** out) {
+  static std::mutex mu;
+  static unsigned char* ptrs[kMaxDevices];
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(CHIP_ERR_INVALID, "fixed scratch: device index out of range");
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    unsigned char* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)));
+    if (!p) return fail(CHIP_ERR_RUNTIME, "fixed scratch: hipGetSymbolAddress returned a null address");
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
   return CHIP_OK;
 }
 
@@ -214,6 +254,15 @@ int chip_module_load(const void* code, size_t size, void** module) {
     return hip_fail("hipModuleLoadData", e);
   }
   *module = m;
+  // Set-up of the fixed scratch array for this device happens here, with the device current: every
+  // function handle a caller can launch comes out of a module loaded on its device, so the
+  // fixed-scratch entry point finds the address resolved.  (It resolves it itself otherwise.)
+  unsigned char* unused = nullptr;
+  std::string kept = g_error;
+  if (fixed_scratch_ptr(&unused) != CHIP_OK) {
+    (void)hipGetLastError();
+    g_error = kept;
+  }
   return CHIP_OK;
 }
 
@@ -271,6 +320,59 @@ int chip_launch_seq(const chip_launch_desc* seq, int n, void* stream) {
   if (!seq || n <= 0) return fail(CHIP_ERR_INVALID, "chip_launch_seq: empty sequence");
   for (int i = 0; i < n; ++i) {
     int rc = launch_one(seq[i], seq[i].args, static_cast<hipStream_t>(stream));
+    if (rc) return rc;
+  }
+  return CHIP_OK;
+}
+
+int chip_launch_seq_fixed_scratch(const chip_launch_desc* seq, int n, void* stream, const chip_scratch_arg* refs,
+                                  int nrefs, uint64_t scratch_bytes, int clear) {
+  if (!seq || n <= 0) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: empty sequence");
+  if (n > kMaxSeq) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: more than 8 launches in one call");
+  if (nrefs < 0 || (nrefs > 0 && !refs)) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: bad scratch argument list");
+  if (scratch_bytes > CHIP_FIXED_SCRATCH_BYTES) {
+    char buf[200];
+    snprintf(buf, sizeof buf, "chip_launch_seq_fixed_scratch: %llu bytes of scratch asked for, the fixed array holds %llu",
+             (unsigned long long)scratch_bytes, (unsigned long long)CHIP_FIXED_SCRATCH_BYTES);
+    return fail(CHIP_ERR_INVALID, buf);
+  }
+  for (int i = 0; i < n; ++i)
+    if (seq[i].nargs < 0 || seq[i].nargs > kMaxArgs || (seq[i].nargs > 0 && !seq[i].args))
+      return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: a launch has no argument array or more than 64 arguments");
+  for (int r = 0; r < nrefs; ++r) {
+    const chip_scratch_arg& a = refs[r];
+    if (a.launch < 0 || a.launch >= n || a.arg < 0 || a.arg >= seq[a.launch].nargs)
+      return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: scratch argument names no argument of the sequence");
+    if (a.offset % 256 || a.offset >= scratch_bytes)
+      return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: scratch offset not a multiple of 256 or outside scratch_bytes");
+  }
+  unsigned char* base = nullptr;
+  int rc = fixed_scratch_ptr(&base);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (clear && scratch_bytes) {
+    // a fill kernel, not hipMemsetAsync: callers may be recording this stream into a graph
+    const unsigned long long n16 = (scratch_bytes + 15) / 16;
+    unsigned blocks = (unsigned)((n16 + 255) / 256);
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(chip_scratch_fill_zero, dim3(blocks), dim3(256), 0, s, reinterpret_cast<uint4*>(base), n16);
+    HIP_TRY(hipGetLastError());
+  }
+  // the caller's argument arrays are left as they are: each launch gets a copy of its pointer
+  // array (on this stack) whose scratch slots point at addresses inside the fixed array
+  void* values[kMaxSeq * 4 + 32];
+  int used = 0;
+  for (int i = 0; i < n; ++i) {
+    void* args[kMaxArgs];
+    for (int j = 0; j < seq[i].nargs; ++j) args[j] = seq[i].args[j];
+    for (int r = 0; r < nrefs; ++r) {
+      if (refs[r].launch != i) continue;
+      if (used >= (int)(sizeof values / sizeof values[0]))
+        return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: more than 64 scratch arguments");
+      values[used] = base + refs[r].offset;
+      args[refs[r].arg] = &values[used++];
+    }
+    rc = launch_one(seq[i], args, s);
     if (rc) return rc;
   }
   return CHIP_OK;

@@ -24,6 +24,7 @@ from . import shim
 from .validate import DEFAULT_TOLERANCE, BenchOptions, Tolerance, _check_kernel, _stage
 
 _TORCH_DTYPES = {"float16": "float16", "bfloat16": "bfloat16", "float32": "float32", "int32": "int32"}
+_DTYPE_BYTES = {"float16": 2, "bfloat16": 2, "float32": 4, "int32": 4}
 
 
 @dataclass(frozen=True)
@@ -219,13 +220,20 @@ class CompiledKernel:
             bound[p.name] = self._scratch[key]
         return outs
 
-    def _descs(self, bound, dims):
+    def _descs(self, bound, dims, fixed=None, refs=None):
+        """Launch descriptors.  ``fixed``: ``{scratch parameter: byte offset}``; those arguments are
+        left null here and listed in ``refs`` as (launch, argument, offset) for the library to point
+        into its fixed scratch array."""
         keep, descs = [], []
         for l in self.manifest["launches"]:
             values = []
             for name in l["args"]:
                 if name in dims and name not in bound:
                     values.append(("i32", dims[name]))
+                    continue
+                if fixed is not None and name in fixed:
+                    refs.append((len(descs), len(values), fixed[name]))
+                    values.append(("ptr", 0))
                     continue
                 v = bound[name]
                 if isinstance(v, float):
@@ -258,6 +266,42 @@ class CompiledKernel:
         if self.out_idx is None:
             return None
         return outs[0] if len(outs) == 1 else outs
+
+    def fixed_scratch_layout(self, dims) -> tuple:
+        """``({scratch parameter: byte offset}, bytes)``: the kernel's scratch buffers laid out
+        one after the other at multiples of 256 bytes (two names of one buffer share an offset)."""
+        offsets, owners, end = {}, {}, 0
+        for p in self.params:
+            if p.role != "scratch":
+                continue
+            owner = p.alias or p.name
+            if owner not in owners:
+                owners[owner] = end
+                n = _DTYPE_BYTES[p.dtype]
+                for extent in self._shape(p, dims):
+                    n *= extent
+                end += -(-n // 256) * 256
+            offsets[p.name] = owners[owner]
+        return offsets, end
+
+    def call_fixed_scratch(self, *args, clear: bool = False) -> None:
+        """Run with caller-owned outputs and no allocation of device memory: the scratch buffers
+        (split partials) live in the native library's fixed per-GPU array instead of tensors.  The
+        kernel must have been made with ``out_idx=None``; ``args`` are the inputs, scalars and
+        outputs in parameter order.  A layout beyond the array's size is refused by the library.
+        Calls that overlap on one GPU share the array and race."""
+        import torch
+
+        if self.out_idx is not None:
+            raise TypeError("call_fixed_scratch needs caller-owned outputs: compile with out_idx=None")
+        bound, dims, device = self._bind(args)
+        fixed, nbytes = self.fixed_scratch_layout(dims)
+        refs = []
+        with torch.cuda.device(device):
+            descs, keep = self._descs(bound, dims, fixed, refs)
+            if descs:
+                shim.launch_seq_fixed_scratch(descs, torch.cuda.current_stream(device).cuda_stream, refs, nbytes, clear)
+        del keep
 
     def time(self, *args, warmup: int = 4, iters: int = 100, rotate=None, only=None, graph_batch: int = 0) -> float:
         """Milliseconds per call measured with HIP events inside the native library.  ``rotate``:

@@ -24,9 +24,10 @@ CHIP_OK, CHIP_ERR_INVALID, CHIP_ERR_COMPILE, CHIP_ERR_RUNTIME, CHIP_ERR_LDS = ra
 EXPORTS = (
     "chip_abi_version", "chip_last_error", "chip_device_count", "chip_device_info_get",
     "chip_compile", "chip_free", "chip_module_load", "chip_module_unload", "chip_get_function",
-    "chip_function_attributes", "chip_launch", "chip_launch_seq", "chip_time_launches",
-    "chip_time_graph",
+    "chip_function_attributes", "chip_launch", "chip_launch_seq", "chip_launch_seq_fixed_scratch",
+    "chip_time_launches", "chip_time_graph",
 )
+FIXED_SCRATCH_BYTES = 64 << 20      # CHIP_FIXED_SCRATCH_BYTES of the header
 
 # Options every kernel is compiled with.  Packed-fp32 instruction selection is switched off:
 # some of its forms have produced silently wrong results on this hardware generation.
@@ -56,6 +57,10 @@ class LaunchDesc(ctypes.Structure):
     _fields_ = [("fn", ctypes.c_void_p), ("grid", ctypes.c_uint32 * 3), ("block", ctypes.c_uint32 * 3),
                 ("lds_bytes", ctypes.c_uint32), ("nargs", ctypes.c_int32),
                 ("args", ctypes.POINTER(ctypes.c_void_p))]
+
+
+class ScratchArg(ctypes.Structure):
+    _fields_ = [("launch", ctypes.c_int32), ("arg", ctypes.c_int32), ("offset", ctypes.c_uint64)]
 
 
 _lock = threading.Lock()
@@ -123,6 +128,8 @@ def _declare(lib):
     lib.chip_launch.argtypes = [c.c_void_p, c.POINTER(c.c_uint32), c.POINTER(c.c_uint32), c.c_uint32,
                                 c.c_void_p, c.POINTER(c.c_void_p), c.c_int]
     lib.chip_launch_seq.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p]
+    lib.chip_launch_seq_fixed_scratch.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p, c.POINTER(ScratchArg),
+                                                  c.c_int, c.c_uint64, c.c_int]
     lib.chip_time_launches.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p, c.c_int, c.c_int, c.c_int,
                                        c.POINTER(c.POINTER(c.c_void_p)), c.POINTER(c.c_float)]
     lib.chip_time_graph.argtypes = [c.POINTER(LaunchDesc), c.c_int, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int,
@@ -271,6 +278,16 @@ def launch(fn: int, grid, block, lds_bytes: int, stream: int, args: PackedArgs):
 def launch_seq(descs, stream: int):
     arr = (LaunchDesc * len(descs))(*descs)
     _check(load().chip_launch_seq(arr, len(descs), ctypes.c_void_p(stream or 0)), "chip_launch_seq")
+
+
+def launch_seq_fixed_scratch(descs, stream: int, refs, scratch_bytes: int, clear: bool = False):
+    """``launch_seq`` with the sequence's scratch buffers inside the library's fixed per-GPU array:
+    ``refs`` is ``[(launch index, argument index, byte offset)]``.  Allocates no device memory."""
+    arr = (LaunchDesc * len(descs))(*descs)
+    ref_arr = (ScratchArg * max(1, len(refs)))(*[ScratchArg(int(l), int(a), int(o)) for l, a, o in refs])
+    _check(load().chip_launch_seq_fixed_scratch(arr, len(descs), ctypes.c_void_p(stream or 0), ref_arr, len(refs),
+                                                int(scratch_bytes), int(bool(clear))),
+           "chip_launch_seq_fixed_scratch")
 
 
 def time_launches(descs, stream: int, warmup: int, iters: int, arg_sets=None, graph_batch: int = 0) -> float:

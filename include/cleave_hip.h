@@ -148,6 +148,42 @@ typedef struct chip_launch_desc {
  * python/cleave/runtime/timer.py:66-73. */
 int chip_launch_seq(const chip_launch_desc* seq, int n, void* stream);
 
+/* Bytes of the fixed scratch array each GPU holds for chip_launch_seq_fixed_scratch. */
+#define CHIP_FIXED_SCRATCH_BYTES (64ull << 20)
+
+/* Names one pointer argument of a launch sequence that is to point into the
+ * fixed scratch array: argument `arg` of launch `launch`, at byte `offset`
+ * (a multiple of 256) from the array's start. */
+typedef struct chip_scratch_arg {
+  int32_t launch;
+  int32_t arg;
+  uint64_t offset;
+} chip_scratch_arg;
+
+/* chip_launch_seq for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * Has no counterpart in the reference, whose callers always allocate the
+ * split partials (python/cleave/runtime/autotune.py:164-227).  The scratch
+ * buffers of the sequence -- the split partials a partial kernel writes and
+ * its combine reads -- live in a fixed array of CHIP_FIXED_SCRATCH_BYTES that
+ * is part of the library and is held by every GPU the library runs on until
+ * the process ends; inputs and outputs are still the caller's.  For each of
+ * the `nrefs` entries of `refs` the named argument is launched with the
+ * address `array + offset` (whatever the caller's slot holds is ignored and
+ * left untouched); `scratch_bytes` is the extent the caller's layout uses.
+ *   - scratch_bytes above CHIP_FIXED_SCRATCH_BYTES, an offset that is not a
+ *     multiple of 256 or lies outside scratch_bytes, more than 8 launches or
+ *     64 arguments per launch: CHIP_ERR_INVALID, nothing is launched;
+ *   - the call makes no hipMalloc / hipFree and no other allocating call;
+ *   - all calls on one GPU share that GPU's array and it keeps the previous
+ *     call's contents: `clear` != 0 zeroes the first scratch_bytes with a fill
+ *     kernel on `stream` before the first launch (for kernels that accumulate
+ *     into scratch; kernels that write every element they later read need no
+ *     clear); calls that overlap in time on one GPU race on the array. */
+int chip_launch_seq_fixed_scratch(const chip_launch_desc* seq, int n, void* stream,
+                                  const chip_scratch_arg* refs, int nrefs,
+                                  uint64_t scratch_bytes, int clear);
+
 /* Time the sequence: `warmup` untimed passes, then `iters` passes between two
  * hipEvents recorded on `stream`; *ms_per_iter = elapsed / iters.  When
  * `nsets` > 1, `arg_sets` holds nsets*n alternative `args` arrays (set-major)
