@@ -1,40 +1,49 @@
-"""Content-addressed cache paths under ``current_session().cache_root / "persistent"``
-(``python/cleave/pipeline/cache.py:13-50``)."""
+"""Where finished work is kept between runs, addressed by what produced it.
+
+Everything lives under ``<session cache root>/persistent``: graph-search checkpoints under
+``superopt/<k0k1>/<key>/checkpoint.json`` and saved kernels under ``kernels/<name>-<key16>/``
+(the reference lays its cache out the same way, ``python/cleave/pipeline/cache.py:13-50``).  A
+key is a SHA-256 over the inputs that determine the result *and* over this build of the back
+end, so a kernel saved by other templates or another native library is never picked up.
+"""
 
 from __future__ import annotations
 
-import functools
 import hashlib
 import json
 from pathlib import Path
 
-SCHEMA = 1
+LAYOUT_VERSION = 1
+_build_id = None
 
 
-@functools.lru_cache(maxsize=None)
 def build_id() -> str:
-    """Package version plus a digest of the kernel templates and the native library source:
-    a cached kernel is only reused by the code that produced it."""
-    from .. import __version__
-    from ..codegen import TEMPLATE_DIR
-    from ..runtime.shim import CSRC_DIR
+    """``<package version>+<12 hex>``: the hex digests every kernel template and the native
+    library's source, name by name."""
+    global _build_id
+    if _build_id is None:
+        from .. import __version__
+        from ..codegen import TEMPLATE_DIR
+        from ..runtime.shim import CSRC_DIR
 
-    h = hashlib.sha256()
-    for path in sorted([*TEMPLATE_DIR.glob("*.hip"), *CSRC_DIR.glob("*.cpp")]):
-        h.update(path.name.encode())
-        h.update(path.read_bytes())
-    return f"{__version__}+{h.hexdigest()[:12]}"
+        sha = hashlib.sha256()
+        for source in sorted(list(TEMPLATE_DIR.glob("*.hip")) + list(CSRC_DIR.glob("*.cpp"))):
+            sha.update(source.name.encode() + b"\0" + source.read_bytes())
+        _build_id = __version__ + "+" + sha.hexdigest()[:12]
+    return _build_id
 
 
 def digest(*parts) -> str:
-    blob = json.dumps([SCHEMA, build_id(), *parts], sort_keys=True, default=str, separators=(",", ":"))
-    return hashlib.sha256(blob.encode()).hexdigest()
+    """Key of ``parts`` (anything JSON can write; other objects by their ``str``)."""
+    canonical = json.dumps([LAYOUT_VERSION, build_id(), list(parts)], sort_keys=True, default=str,
+                           separators=(",", ":"))
+    return hashlib.sha256(canonical.encode()).hexdigest()
 
 
 def root() -> Path:
     from ..core.session import current_session
 
-    return current_session().cache_root / "persistent"
+    return Path(current_session().cache_root) / "persistent"
 
 
 def superopt_key(program, max_ops: int, split: tuple, concat_matmul: bool) -> str:
@@ -42,9 +51,10 @@ def superopt_key(program, max_ops: int, split: tuple, concat_matmul: bool) -> st
 
 
 def checkpoint_path(key: str) -> Path:
-    d = root() / "superopt" / key[:2] / key
-    d.mkdir(parents=True, exist_ok=True)
-    return d / "checkpoint.json"
+    """The checkpoint file for ``key``; its directory is created."""
+    folder = root() / "superopt" / key[:2] / key
+    folder.mkdir(parents=True, exist_ok=True)
+    return folder / "checkpoint.json"
 
 
 def kernel_dir(name: str, key: str) -> Path:
