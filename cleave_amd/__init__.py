@@ -1,57 +1,45 @@
 """cleave_amd: an MI355X (gfx950) code-generation and runtime back end behind the Cleave API.
 
-``cleave_amd.compile(fn, shapes=..., dtype=..., preset=...)`` on a ``@cleave_amd.jit`` program
-follows the same staged pipeline as the reference (trace -> superoptimize -> schedule ->
-build -> evaluate), but plans are instantiated into hand-written HIP kernel templates,
-compiled with hiprtc for gfx950 and launched through ``libcleave_hip.so``.
+``cleave_amd.compile(fn, shapes=..., dtype=..., preset=...)`` on a ``@cleave_amd.jit`` program runs the
+staged pipeline trace -> superoptimize -> schedule -> build -> evaluate; plans are instantiated
+into hand-written HIP kernel templates, compiled with hiprtc for gfx950 and launched through
+``libcleave_hip.so``.
+
+Nothing heavy is imported until it is asked for: the public names below are resolved on first
+attribute access (the top-level names are those of ``python/cleave/__init__.py``, so user code
+only changes its import line).
 """
 
-from importlib import import_module
+import importlib
 
 __version__ = "0.1.0"
 
-_LAZY = {
-    "HipCodeGen": ".codegen",
-    "search_tiling": ".schedule",
-    "apply_tiling": ".schedule",
-    "Program": ".frontend",
-    "trace": ".frontend",
-    "jit": ".frontend",
-    "JitFunction": ".frontend",
-    "InputSpec": ".frontend",
-    "OutputSpec": ".frontend",
-    "compile": ".pipeline",
-    "superoptimize": ".pipeline",
-    "schedule_plans": ".pipeline",
-    "build": ".pipeline",
-    "evaluate": ".pipeline",
-    "load": ".pipeline",
-    "list_presets": ".pipeline",
-    "SuperoptConfig": ".pipeline",
-    "ScheduleConfig": ".pipeline",
-    "EvalConfig": ".pipeline",
-    "GraphSet": ".pipeline",
-    "SearchedGraph": ".pipeline",
-    "Plan": ".pipeline",
-    "PlanSet": ".pipeline",
-    "BuildSet": ".pipeline",
-    "Report": ".pipeline",
-    "Kernel": ".pipeline",
-    "CleaveError": ".core.errors",
-    "Session": ".core.session",
+# home module (relative) -> the public names it provides
+_PROVIDERS = {
+    ".frontend": "Program trace jit JitFunction InputSpec OutputSpec",
+    ".pipeline": ("compile superoptimize schedule_plans build evaluate load list_presets "
+                  "SuperoptConfig ScheduleConfig EvalConfig GraphSet SearchedGraph Plan PlanSet BuildSet Report Kernel"),
+    ".schedule": "search_tiling apply_tiling",
+    ".codegen": "HipCodeGen",
+    ".core.errors": "CleaveError",
+    ".core.session": "Session",
 }
-_SUBMODULES = {"core", "arch", "ir", "schedule", "codegen", "runtime", "dynamic", "frontend", "pipeline", "lang"}
+_PACKAGES = "arch codegen core dynamic frontend ir lang pipeline runtime schedule".split()
 
-__all__ = sorted([*_LAZY, *_SUBMODULES])
+_HOME = {name: module for module, names in _PROVIDERS.items() for name in names.split()}
+__all__ = sorted(set(_HOME) | set(_PACKAGES))
 
 
-def __getattr__(name: str):
-    if name in _SUBMODULES:
-        return import_module(f".{name}", __name__)
-    if name in _LAZY:
-        return getattr(import_module(_LAZY[name], __name__), name)
-    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+def __getattr__(name):
+    if name in _PACKAGES:
+        value = importlib.import_module("." + name, __name__)
+    elif name in _HOME:
+        value = getattr(importlib.import_module(_HOME[name], __name__), name)
+    else:
+        raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+    globals()[name] = value          # the next access does not come back here
+    return value
 
 
 def __dir__():
-    return __all__
+    return list(__all__)

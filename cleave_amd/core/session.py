@@ -1,9 +1,12 @@
-"""``Session``: target, cache root and parallelism scoped by a ``with`` block
-(``python/cleave/core/session.py:22-64``)."""
+"""``Session``: a ``with`` block that scopes the target, the cache root and the search width.
+
+Stands in for ``python/cleave/core/session.py:22-64`` (same constructor arguments and attributes).
+Sessions nest; each is a link in a chain held by one context variable, so threads and asyncio
+tasks each see their own innermost session.
+"""
 
 from __future__ import annotations
 
-import dataclasses
 from contextvars import ContextVar
 from pathlib import Path
 from typing import Optional
@@ -11,48 +14,63 @@ from typing import Optional
 from .settings import Settings
 from .target import Target, default_target
 
-_STACK: ContextVar[tuple] = ContextVar("cleave_amd_sessions", default=())
+# innermost entered session of the current context (None outside every ``with Session(...)``)
+_INNERMOST: ContextVar[Optional["Session"]] = ContextVar("cleave_amd_session", default=None)
+
+
+def _as_target(value):
+    return Target(value) if isinstance(value, str) else value
+
+
+def _as_width(value):
+    if value is None:
+        return None
+    width = int(value)
+    if width < 1:
+        raise ValueError(f"max_parallel must be >= 1, got {value}")
+    return width
 
 
 class Session:
+    """``target``: a ``Target`` or its name (default: detected); ``cache_root``: overrides the
+    environment's; ``max_parallel``: candidates compiled / validated side by side (default: the
+    evaluation config's); ``settings``: a ready ``Settings`` instead of the environment's."""
+
     def __init__(self, target=None, cache_root=None, max_parallel: Optional[int] = None,
                  settings: Optional[Settings] = None):
-        settings = settings or Settings.from_env()
-        if cache_root is not None:
-            settings = dataclasses.replace(settings, cache_root=Path(cache_root).expanduser())
-        if max_parallel is not None and int(max_parallel) < 1:
-            raise ValueError(f"max_parallel must be >= 1, got {max_parallel}")
-        self.settings = settings
-        self.explicit_target = Target(target) if isinstance(target, str) else target
-        self.max_parallel = None if max_parallel is None else int(max_parallel)
+        self.max_parallel = _as_width(max_parallel)
+        self.explicit_target = _as_target(target)
+        base = Settings.from_env() if settings is None else settings
+        self.settings = base if cache_root is None else base.replace(cache_root=Path(cache_root).expanduser())
+        self._outer = None
+        self._entered = False
 
-    @property
-    def target(self) -> Target:
-        return self.explicit_target or default_target()
-
-    @property
-    def cache_root(self) -> Path:
-        return Path(self.settings.cache_root)
+    target = property(lambda self: self.explicit_target or default_target())
+    cache_root = property(lambda self: Path(self.settings.cache_root))
 
     def __enter__(self):
-        _STACK.set(_STACK.get() + (self,))
+        if self._entered:
+            raise RuntimeError("this Session is already entered")
+        self._outer, self._entered = _INNERMOST.get(), True
+        _INNERMOST.set(self)
         return self
 
     def __exit__(self, *exc):
-        stack = _STACK.get()
-        if not stack or stack[-1] is not self:
+        if _INNERMOST.get() is not self:
             raise RuntimeError("Session exited out of order")
-        _STACK.set(stack[:-1])
+        _INNERMOST.set(self._outer)
+        self._outer, self._entered = None, False
 
     def __repr__(self):
-        return (f"Session(target={self.target!r}, cache_root={str(self.cache_root)!r}, "
-                f"max_parallel={self.max_parallel})")
+        fields = {"target": self.target, "cache_root": str(self.cache_root), "max_parallel": self.max_parallel}
+        return "Session(" + ", ".join(f"{k}={v!r}" for k, v in fields.items()) + ")"
 
 
 def active_session() -> Optional[Session]:
-    stack = _STACK.get()
-    return stack[-1] if stack else None
+    """The innermost entered session, or ``None``."""
+    return _INNERMOST.get()
 
 
 def current_session() -> Session:
-    return active_session() or Session()
+    """The innermost entered session, or a fresh one built from the environment."""
+    return _INNERMOST.get() or Session()

@@ -1,54 +1,67 @@
-"""The ``cl.*`` functions.  Given traced ``cl.Tensor`` handles they record ops; given torch
-tensors they compute eagerly, so the body of a ``@cleave.jit`` function doubles as its own
-eager definition (``python/cleave/frontend/composites.py:10-63``)."""
+"""The ``cl.*`` functions (``python/cleave/frontend/composites.py:10-63`` names and arguments).
+
+Each works on two kinds of operand: on a traced ``cl.Tensor`` it records ops, on a torch tensor
+it computes at once, so the body of a ``@jit`` function is also its own eager definition.  The
+choice is made in one place (``_DUAL``: per function, the handle's method and torch's spelling);
+what is built from other functions of this module (``rsqrt``, ``rms_norm``, ``softmax``) needs
+no choice of its own.
+"""
 
 from __future__ import annotations
+
+from typing import Optional
 
 from .program import grouped_matmul
 from .tensor import Tensor
 
+# name -> (what to call on a traced handle, what to call on a torch tensor)
+_DUAL = {
+    "exp": (lambda x: x.exp(), lambda torch, x: torch.exp(x)),
+    "sqrt": (lambda x: x.sqrt(), lambda torch, x: torch.sqrt(x)),
+    "silu": (lambda x: x.silu(), lambda torch, x: torch.nn.functional.silu(x)),
+    "max": (lambda x, dim, keepdim: x.max(dim, keepdim=keepdim),
+            lambda torch, x, dim, keepdim: x.amax(dim, keepdim=keepdim)),       # values only, no indices
+    "matmul": (lambda a, b: a @ b, lambda torch, a, b: grouped_matmul(a, b)),
+}
 
-def _torch():
+
+def _dual(name, *operands):
+    traced, eager = _DUAL[name]
+    if any(isinstance(x, Tensor) for x in operands):
+        return traced(*operands)
     import torch
 
-    return torch
-
-
-def _is_traced(*xs) -> bool:
-    return any(isinstance(x, Tensor) for x in xs)
+    return eager(torch, *operands)
 
 
 def exp(x):
-    return x.exp() if _is_traced(x) else _torch().exp(x)
+    return _dual("exp", x)
 
 
 def sqrt(x):
-    return x.sqrt() if _is_traced(x) else _torch().sqrt(x)
+    return _dual("sqrt", x)
 
 
 def silu(x):
-    return x.silu() if _is_traced(x) else _torch().nn.functional.silu(x)
+    return _dual("silu", x)
 
 
 def rsqrt(x):
-    """``1 / sqrt(x)``; the op vocabulary has no rsqrt of its own."""
+    """Reciprocal square root, spelled with the two ops the vocabulary has."""
     return 1.0 / sqrt(x)
 
 
 def matmul(a, b):
-    """``a @ b`` with grouped broadcast of the leading (batch) dims."""
-    return a @ b if _is_traced(a, b) else grouped_matmul(a, b)
-
-
-def sum(x, dim: int = -1, keepdim: bool = False):  # noqa: A001
-    return x.sum(dim, keepdim=keepdim)
+    """``a @ b``; leading (batch) extents may differ by a whole factor (grouped heads)."""
+    return _dual("matmul", a, b)
 
 
 def max(x, dim: int = -1, keepdim: bool = False):  # noqa: A001
-    """Values of the max over ``dim`` (no indices)."""
-    if _is_traced(x):
-        return x.max(dim, keepdim=keepdim)
-    return x.amax(dim, keepdim=keepdim)
+    return _dual("max", x, dim, keepdim)
+
+
+def sum(x, dim: int = -1, keepdim: bool = False):  # noqa: A001
+    return x.sum(dim, keepdim=keepdim)          # both kinds of operand spell it alike
 
 
 def mean(x, dim: int = -1, keepdim: bool = False):
@@ -56,20 +69,17 @@ def mean(x, dim: int = -1, keepdim: bool = False):
 
 
 def rms_norm(x, dim: int = -1, eps: float = 0.0):
-    """``x * rsqrt(mean(x * x) + eps)``, no learned weight."""
-    ms = mean(x * x, dim, keepdim=True)
-    if eps:
-        ms = ms + eps
-    return x * rsqrt(ms)
+    """``x / sqrt(mean(x^2) [+ eps])`` along ``dim``; no learned weight."""
+    power = mean(x * x, dim, keepdim=True)
+    return x * rsqrt(power + eps if eps else power)
 
 
-def softmax(x, dim: int = -1, shift: float | None = None):
-    """``shift=None``: exact ``exp(x - max x) / sum``.  A number: ``exp(x + shift) / sum`` with
-    no max op (the same function mathematically; it overflows where the exact form cannot)."""
+def softmax(x, dim: int = -1, shift: Optional[float] = None):
+    """Without ``shift``: the exact form, ``exp(x - max x) / sum``.  With a number: ``exp(x +
+    shift) / sum`` and no max op: mathematically the same function, but it can overflow."""
     if shift is None:
-        e = exp(x - max(x, dim, keepdim=True))
+        x = x - max(x, dim, keepdim=True)
     elif shift:
-        e = exp(x + shift)
-    else:
-        e = exp(x)
-    return e / sum(e, dim, keepdim=True)
+        x = x + shift
+    weights = exp(x)
+    return weights / sum(weights, dim, keepdim=True)

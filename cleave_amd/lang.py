@@ -1,24 +1,33 @@
-"""``import cleave_amd.lang as cl``: dims, dtypes, annotations and ops of the frontend
-(the names of ``python/cleave/lang.py``)."""
+"""The program-writing vocabulary, meant to be imported as ``import cleave_amd.lang as cl``.
 
-from .frontend.composites import exp, matmul, max, mean, rms_norm, rsqrt, silu, sqrt, sum  # noqa: A004,F401
-from .frontend.paged import PageTable, ScheduleHints, paged_gather, softmax  # noqa: F401
-from .frontend.tensor import DType, Dim, Scalar, Split, Tensor, bf16, dims, f16, f32, i32  # noqa: F401
+It gathers, under the short names programs are written with (those of ``python/cleave/lang.py``):
+element types and dimensions, argument annotations, the op functions, the paged-attention
+declarations, plus two names that are looked up late because their homes import torch
+(``Tolerance``) or the operator registry (``workloads``).
+"""
 
-__all__ = [
-    "DType", "Dim", "PageTable", "Scalar", "ScheduleHints", "Split", "Tensor", "Tolerance", "bf16",
-    "dims", "exp", "f16", "f32", "i32", "matmul", "max", "mean", "paged_gather", "rms_norm", "rsqrt",
-    "silu", "softmax", "sqrt", "sum", "workloads",
-]
+import importlib
+
+from .frontend import composites as _ops
+from .frontend import paged as _paged
+from .frontend import tensor as _tensor
+
+_EAGER = {
+    _tensor: "DType Dim Scalar Split Tensor bf16 dims f16 f32 i32",
+    _ops: "exp matmul max mean rms_norm rsqrt silu sqrt sum",
+    _paged: "PageTable ScheduleHints paged_gather softmax",
+}
+_LATE = {"Tolerance": (".runtime.validate", "Tolerance"), "workloads": (".frontend.paged", "workloads")}
+
+for _module, _names in _EAGER.items():
+    for _name in _names.split():
+        globals()[_name] = getattr(_module, _name)
+
+__all__ = sorted([name for names in _EAGER.values() for name in names.split()] + list(_LATE))
 
 
 def __getattr__(name):
-    if name == "Tolerance":
-        from .runtime.validate import Tolerance
-
-        return Tolerance
-    if name == "workloads":
-        from .frontend import paged
-
-        return paged.workloads
-    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+    if name not in _LATE:
+        raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+    module, attribute = _LATE[name]
+    return getattr(importlib.import_module(module, __package__), attribute)

@@ -67,7 +67,7 @@ def evaluate(program, inputs, round_outputs=True) -> list:
     ``round_outputs`` is False)."""
     feed = iter([to_f32(x) for x in inputs])
     env = {}
-    records = list(program._records)
+    records = list(program.ops)
 
     def val(a):
         return env[a] if isinstance(a, int) else np.float32(a)

@@ -152,7 +152,7 @@ def test_paged_program_refusals():
     from cleave_amd.frontend.paged import PagedProgram, trace_paged
 
     with pytest.raises(SpecError, match="dense program"):
-        PagedProgram.__new__(PagedProgram)._binary("sub", None, None)
+        PagedProgram("p").apply("sub", (None, None))
 
     @cleave_amd.jit(dtype=cl.bf16)
     def unscaled(q: cl.Tensor[batch, 8, 64], kc: cl.Tensor[num_pages, 1, 2, 64], vc: cl.Tensor[num_pages, 1, 2, 64],
@@ -172,3 +172,47 @@ def test_paged_decode_workloads_are_deterministic():
     assert wl.axes() == [(1, 16), (1, 128), (1, 1024), (7, 16), (7, 128), (7, 1024)]
     lens = wl.lengths(7, 1024)
     assert lens == wl.lengths(7, 1024) and lens[0] == 1024 and all(512 <= n <= 1024 for n in lens)
+
+
+def test_paged_program_survives_its_plain_data_form():
+    """A compiled paged operator is saved as JSON, not as a pickle: the program must come back
+    from ``to_doc()`` recognisable as the same operator."""
+    import json
+
+    from cleave_amd.frontend.paged import PagedProgram, trace_paged
+
+    op = paged_op(PAGE=64)
+    program = trace_paged(op)
+    program.split = (cl.Split("kv_len", (4, 8)),)
+    back = PagedProgram.from_doc(json.loads(json.dumps(program.to_doc())))
+    assert repr(back) == repr(program) and back.split == program.split
+    a, b = program.attention(), back.attention()
+    assert a.paging_spec() == b.paging_spec() and a.kind == b.kind
+    assert [p.name for p in a.inputs] == [p.name for p in b.inputs]
+    assert a.output_dims() == b.output_dims() and a.dense_body().fingerprint() == b.dense_body().fingerprint()
+    with pytest.raises(SpecError, match="format"):
+        PagedProgram.from_doc({"format": 7})
+
+
+def test_settings_and_sessions(monkeypatch, tmp_path):
+    from cleave_amd.core import Session, Settings, active_session, current_session
+
+    env = {"CLEAVE_COMPILE_AND_RUN_TIMEOUT_SECS": "0", "CLEAVE_COMPILE_PROGRESS_HEARTBEAT_SECS": "junk",
+           "COMPILATION_PROGRESS_LOG": " Yes ", "CLEAVE_TEST_SEED": str(2 ** 32 + 5), "SCRATCH": str(tmp_path)}
+    s = Settings.from_env(env)
+    assert s.compile_timeout_secs is None and s.heartbeat_secs == 15.0 and s.progress_log and s.test_seed == 5
+    assert s.cache_root == tmp_path / "cleave_cache" and s.runtime_root == s.cache_root / "runtime"
+    assert Settings.from_env({"CLEAVE_CACHE_ROOT": str(tmp_path / "x"), "SCRATCH": "/nowhere"}).cache_root == tmp_path / "x"
+    assert s.replace(progress_log=False) != s and s.replace() == s
+    with pytest.raises(AttributeError):
+        s.progress_log = False
+    assert active_session() is None
+    with Session(cache_root=tmp_path / "a", max_parallel=3) as outer:
+        with Session(settings=s) as inner:
+            assert current_session() is inner and inner.cache_root == s.cache_root
+            with pytest.raises(RuntimeError):
+                outer.__exit__(None, None, None)
+        assert active_session() is outer and outer.max_parallel == 3
+    assert active_session() is None
+    with pytest.raises(ValueError):
+        Session(max_parallel=0)
