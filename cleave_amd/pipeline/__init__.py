@@ -1,17 +1,29 @@
-"""Staged compile pipeline: superoptimize -> schedule -> build -> evaluate -> Kernel."""
+"""The staged compile pipeline: superoptimize -> schedule -> build -> evaluate -> ``Kernel``.
 
-from .build import BuildSet, BuiltKernel, build, evaluate
-from .compile import compile, resolve_configs  # noqa: A004
-from .config import (PRESETS, EvalConfig, Preset, ScheduleConfig, SuperoptConfig, auto_max_ops, get_preset,
-                     list_presets)
-from .kernel import Kernel, load
-from .plans import Plan, PlanSet, Refusal, lower, schedule
-from .report import Failures, Report, Result, VariantResult
-from .superopt import GraphSet, SearchedGraph, superoptimize
+One stage per module; this file only gathers their public names (those a Cleave user imports
+from ``cleave.pipeline``) into one namespace.
+"""
 
-schedule_plans = schedule
+from . import build as _build
+from . import compile as _compile
+from . import config as _config
+from . import kernel as _kernel
+from . import plans as _plans
+from . import report as _report
+from . import superopt as _superopt
 
-__all__ = ["BuildSet", "BuiltKernel", "EvalConfig", "Failures", "GraphSet", "Kernel", "PRESETS", "Plan", "PlanSet",
-           "Preset", "Refusal", "Report", "Result", "ScheduleConfig", "SearchedGraph", "SuperoptConfig",
-           "VariantResult", "auto_max_ops", "build", "compile", "evaluate", "get_preset", "list_presets", "load",
-           "lower", "resolve_configs", "schedule", "schedule_plans", "superoptimize"]
+_PUBLIC = {
+    _superopt: ("GraphSet", "SearchedGraph", "superoptimize"),
+    _plans: ("Plan", "PlanSet", "Refusal", "lower", "schedule"),
+    _build: ("BuildSet", "BuiltKernel", "build", "evaluate"),
+    _report: ("Failures", "Report", "Result", "VariantResult"),
+    _kernel: ("Kernel", "load"),
+    _compile: ("compile", "resolve_configs"),
+    _config: ("PRESETS", "Preset", "SuperoptConfig", "ScheduleConfig", "EvalConfig", "auto_max_ops", "get_preset",
+              "list_presets"),
+}
+for _module, _names in _PUBLIC.items():
+    globals().update({_name: getattr(_module, _name) for _name in _names})
+schedule_plans = _plans.schedule          # the name the top-level package exports the stage under
+
+__all__ = sorted([name for names in _PUBLIC.values() for name in names] + ["schedule_plans"])

@@ -268,3 +268,33 @@ def test_validation_evaluator_agrees_with_the_numpy_oracle(case):
     want = program_oracle.evaluate(prog, inputs)[0]
     got = execute(stage_graph(prog), inputs)[0].float().numpy().reshape(want.shape)
     np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2)
+
+
+def test_saved_paged_kernel_holds_its_program_as_json(tmp_path):
+    """A paged operator's directory is plain data: program.json + sources + dispatch.json.  It
+    loads back to the same operator, and a directory that names a pickle is refused unread."""
+    import json
+
+    import cleave_amd.lang as cl
+    from cleave_amd import examples
+    from cleave_amd.frontend.paged import trace_paged
+    from cleave_amd.pipeline import load
+    from cleave_amd.pipeline.dynamic import PagedKernel
+
+    attention = trace_paged(examples.paged_decode_op(32, 8, 128, 64, dtype=cl.bf16, name="op")).attention()
+    kernel = PagedKernel(attention, attention.paging_spec(), "// main", label="L", variant="solo", latency_us=1.5,
+                         dispatch={"min_tiles": 3, "geomean_us": {"hybrid": 1.0}},
+                         dispatch_sources={"split": "// pair", "single": "// one"})
+    folder = kernel.save(tmp_path / "k")
+    assert {"program.json", "kernel.json", "kernel.hip", "dispatch.json", "dispatch.split.hip"} <= {p.name for p in folder.iterdir()}
+    assert not list(folder.glob("*.pkl"))
+    back = load(folder)
+    assert isinstance(back, PagedKernel) and back.spec == kernel.spec and back.source == "// main"
+    assert back.dispatch["min_tiles"] == 3 and back.dispatch_sources == kernel.dispatch_sources
+    assert [p.name for p in back.attention.inputs] == [p.name for p in attention.inputs]
+    document = json.loads((folder / "kernel.json").read_text())
+    document["paged"] = "program.pkl"
+    (folder / "kernel.json").write_text(json.dumps(document))
+    (folder / "program.pkl").write_bytes(b"not read")
+    with pytest.raises(ValueError, match="pickle"):
+        load(folder)
