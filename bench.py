@@ -84,6 +84,13 @@ def op_table():
         "rsdiv": dict(title="rows divided by their sums f16 4096x4096 (the reference's rowsum_div case)", fn=C.rowsum_div,
                       dtype=cl.f16, shapes=dict(M=4096, N=4096), inputs=C.inputs_rows, split=False,
                       bytes=2 * 2 * 4096 * 4096, flops=2 * 4096 * 4096, bound="hbm", sets=6),
+        "rmsmm": dict(title="rmsnorm(x) @ w f16 4096x6144x4096 (the reference's rmsnorm_matmul case)",
+                      fn=C.rmsnorm_matmul_plain, dtype=cl.f16, shapes=dict(M=4096, N=6144, K=4096), inputs=C.inputs_plain_norm,
+                      split=False, bytes=2 * (4096 * 4096 + 4096 * 6144 + 4096 * 6144), flops=2 * 4096 * 6144 * 4096,
+                      bound="mfma", sets=2),
+        "mm2d": dict(title="chained matmul f16 (a@b)@c 4096x4096x64, b given (K, N) (the reference's matmul_matmul_small_k case)",
+                     fn=C.matmul_matmul_2d, dtype=cl.f16, shapes=dict(M=4096, N=4096, K=64), inputs=C.inputs_chain2d,
+                     split=False, bytes=2 * (4096 * 64 * 4), flops=2 * 2 * 4096 * 4096 * 64, bound="mfma", sets=4, cpu=False),
         "mmrs": dict(title="matmul + row sum f16 (x@w).sum(-1) 4096x4096x64", fn=C.matmul_rowsum, dtype=cl.f16,
                      shapes=C.FULL["matmul_rowsum"], inputs=C.inputs_c1, split=False,
                      bytes=2 * (4096 * 64 + 64 * 4096 + 4096), flops=2 * 4096 * 4096 * 64, bound="mfma", sets=4),
@@ -474,7 +481,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,lora,mmrs,rsdiv,attn,qknorm,mlapf")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,rmsmm,lora,mmrs,mm2d,rsdiv,attn,qknorm,mlapf")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")

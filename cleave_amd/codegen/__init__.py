@@ -467,6 +467,9 @@ class HipCodeGen:
         unit.define("CL_SCALE", _f(float(p.get("scale", 1.0))))
         norm = p.get("norm_eps") or {}
         unit.define("CL_LINEAR", bool(p.get("linear")))
+        if p.get("k_major") and p["skv"] % 32:
+            raise CodegenError("feature-major keys need a key count in whole 32-key steps")
+        unit.define("CL_KT", bool(p.get("k_major")))
         unit.define("CL_QNORM", "q" in norm)
         unit.define("CL_KNORM", "k" in norm)
         unit.define("CL_QNORM_EPS", _f(float(norm.get("q", 0.0))))

@@ -29,6 +29,13 @@
 // CL_LINEAR (dense mode): no softmax -- out = (q k^T) v, the raw scores times CL_SCALE, rounded to the
 // element type, are the weights; no maxima, no reference, no normalisation.
 //
+// CL_KT (dense mode): the keys are given feature-major, K (units, d, keys) -- the middle operand of a
+// chained product (a b) c with b stored (K, N).  A step's K image is then [D/64][64 features][32 keys]
+// (64-byte feature rows; the 32-byte halves of a row trade places on rows with feature bit 3 set,
+// which spreads the four lane groups of an operand read over the banks), wave w loads features
+// 16 w .. 16 w + 15 of every panel, and the score operand (key row, 8 consecutive features) comes
+// out of a pair of transposing reads like the value operand does.  CL_SKV must be a multiple of 32.
+//
 // CL_QNORM / CL_KNORM (QK-norm attention): query / key rows enter the scores RMS-normalised over
 // their features, x * rsqrt(mean(x^2) + eps).  Query rows are normalised once when they are loaded.
 // Key rows cannot be touched on their way into LDS, so their factors multiply the scores instead:
@@ -54,6 +61,12 @@
 #endif
 #ifndef CL_LINEAR
 #define CL_LINEAR 0
+#endif
+#ifndef CL_KT
+#define CL_KT 0
+#endif
+#if CL_KT && (!CL_DENSE || CL_SKV % 32 != 0)
+#error "feature-major keys: dense operands, a key count in whole 32-key steps"
 #endif
 #ifndef CL_QNORM
 #define CL_QNORM 0
@@ -265,9 +278,20 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     constexpr int PART = decltype(part_c)::value;
     constexpr bool IS_K = PART < PL_KPANELS;
     constexpr int P = IS_K ? PART : PART - PL_KPANELS;
+    const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024) + (IS_K ? 0 : PL_KIMG * 2);
+#if CL_KT
+    if constexpr (IS_K) {
+      // feature row 64 P + 16 wave + lane / 4 of the (d, keys) matrix, the step's 32 keys as four
+      // 16-byte chunks; `row` is the lane's key row of the step, so the step starts at row - my_r
+      const int feat = 64 * P + 16 * wave + (lane >> 2);
+      const int piece = (lane & 3) ^ ((lane >> 4) & 2);            // halves swapped where feature bit 3 is set
+      const char* src = kbase + ((i64)feat * CL_SKV + (row - my_r)) * 2 + 16 * piece;
+      pl_dma16<0>(src, group_byte + (unsigned)(P * PL_PANEL * 2));
+      return;
+    }
+#endif
     const int chunk = (lane & 7) ^ pl_swz(my_r);
     const char* src = (IS_K ? kbase + (i64)row * krow_bytes : vbase + (i64)row * vrow_bytes) + 16 * chunk;
-    const unsigned group_byte = tiles_byte + (unsigned)(slot * PL_STAGE * 2 + wave * 1024) + (IS_K ? 0 : PL_KIMG * 2);
     pl_dma16<128 * P>(src, group_byte + (unsigned)(P * PL_PANEL * 2) - 128 * P);
   };
   // the quarter `place` (0..3) of a step's loads: the body spreads them between its matrix work,
@@ -354,8 +378,18 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // 32-feature block, each feeding the wave's two row tiles
   auto k_frag = [&](auto slot_c, int j, int h) __attribute__((always_inline)) {
     constexpr int SLOT = decltype(slot_c)::value;
+#if CL_KT
+    // sixteen lanes address a 4 (feature) x 16 (key) patch, lane c: feature row c / 4, keys 4 (c % 4) .. + 3,
+    // and lane c receives the four features of key c; two reads give features 8 g .. 8 g + 7 of block j
+    const elem_t* p = pl_tiles + SLOT * PL_STAGE + (j >> 1) * PL_PANEL + (32 * (j & 1) + 8 * g + (c >> 2)) * 32 +
+                      16 * (h ^ (g & 1)) + 4 * (c & 3);
+    const pl_s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p));
+    const pl_s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p + 4 * 32));
+    return __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+#else
     return *reinterpret_cast<const elem8*>(pl_tiles + SLOT * PL_STAGE + (j >> 1) * PL_PANEL + 16 * h * 64 +
                                            (a_lo ^ ((4 * (j & 1)) << 3)));
+#endif
   };
   // value operand for feature block fb out of the V image in stage SLOT: rows = features
   // 16 fb + (0..15), slots = keys 4 g + (0..3), 16 + 4 g + (0..3)

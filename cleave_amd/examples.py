@@ -20,6 +20,14 @@ def matmul(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
 
 
 @cleave_amd.jit
+def batched_matmul(x: cl.Tensor["BX", "M", "K"], w: cl.Tensor["BW", "K", "N"]):
+    """``x @ w`` per batch entry; ``BX`` may be a whole multiple of ``BW`` (entries of ``w`` shared by
+    groups of ``x``).  Split over K it is the reference's ``batched_matmul_splitk_partial`` /
+    ``_combine`` pair, (2, 4, 128, 128, 1024) (``tests/_graphs.py:365-402``)."""
+    return x @ w
+
+
+@cleave_amd.jit
 def rmsnorm_matmul(x: cl.Tensor["M", "K"], gamma: cl.Tensor[1, "K"], w: cl.Tensor["K", "N"]):
     return (cl.rms_norm(x, dim=-1, eps=1e-6) * gamma) @ w
 
@@ -87,6 +95,13 @@ def matmul_matmul(q: cl.Tensor["H", "SQ", "D"], k: cl.Tensor["H", "SKV", "D"], v
 
 
 @cleave_amd.jit
+def matmul_matmul_2d(a: cl.Tensor["M", "K"], b: cl.Tensor["K", "N"], c: cl.Tensor["N", "K"]):
+    """``(a @ b) @ c`` with the middle operand given (K, N) (the reference's ``matmul_matmul_small_k``
+    (4096, 4096, 64) and ``matmul_matmul_small_n`` (4096, 64, 64) cases, ``tests/_graphs.py:65-76``)."""
+    return (a @ b) @ c
+
+
+@cleave_amd.jit
 def gqa_decode_shift(q: cl.Tensor["HQ", "SQ", "D"], k: cl.Tensor["HKV", "SKV", "D"], v: cl.Tensor["HKV", "SKV", "D"]):
     n = q.shape[-1] ** 0.5
     return cl.softmax((q @ k.mT) / n, dim=-1, shift=-50 / n) @ v
@@ -126,6 +141,30 @@ def inputs_c1(shapes, seed=1, device="cpu"):
     x = (torch.rand(M, K, generator=g) * 2 - 1) / math.sqrt(K)
     w = (torch.rand(K, N, generator=g) * 2 - 1) / math.sqrt(K)
     return [x.to(torch.float16).to(device), w.to(torch.float16).to(device)]
+
+
+def inputs_batched(shapes, seed=14, device="cpu"):
+    g = _gen(seed)
+    bx, bw, M, N, K = (shapes[k] for k in ("BX", "BW", "M", "N", "K"))
+    x = (torch.rand(bx, M, K, generator=g) * 2 - 1) / math.sqrt(K)
+    w = (torch.rand(bw, K, N, generator=g) * 2 - 1) / math.sqrt(K)
+    return [x.to(torch.float16).to(device), w.to(torch.float16).to(device)]
+
+
+def inputs_plain_norm(shapes, seed=15, device="cpu"):
+    g = _gen(seed)
+    M, N, K = shapes["M"], shapes["N"], shapes["K"]
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(K, N, generator=g) / math.sqrt(K)
+    return [x.to(torch.float16).to(device), w.to(torch.float16).to(device)]
+
+
+def inputs_chain2d(shapes, seed=16, device="cpu"):
+    """a (M, K) scaled so that sums of thousands of products stay inside f16, b (K, N), c (N, K)."""
+    g = _gen(seed)
+    M, N, K = shapes["M"], shapes["N"], shapes["K"]
+    a, b, c = torch.randn(M, K, generator=g) / 8, torch.randn(K, N, generator=g), torch.randn(N, K, generator=g)
+    return [t.to(torch.float16).to(device) for t in (a, b, c)]
 
 
 def inputs_swiglu(shapes, seed=6, device="cpu"):

@@ -418,30 +418,35 @@ def _try_rowsum(view, out):
 
 
 def _try_chained_matmul(view, out):
-    """``(q @ k^T) @ v`` with nothing between the products (the reference's ``matmul_matmul_bhsd``
-    case, ``tests/_graphs.py:78-101``): attention without a softmax.  It is the attention family
-    with ``linear`` set: the scores themselves, rounded to the element type, weigh the values."""
+    """``(q @ k^T) @ v`` with nothing between the products: attention without a softmax.  It is the
+    attention family with ``linear`` set: the scores themselves, rounded to the element type, weigh
+    the values.  Two spellings: keys given row-major and transposed by the product (the reference's
+    ``matmul_matmul_bhsd`` case, ``tests/_graphs.py:78-101``), or the middle operand given
+    feature-major, ``(a @ b) @ c`` with ``b`` stored (K, N) (its ``matmul_matmul_small_k`` /
+    ``_small_n`` cases, ``tests/_graphs.py:65-76``): then ``k_major`` is set as well."""
     n = view.skip(out)
     if not (_is(n, "matmul") and not n.attrs["trans_A"] and not n.attrs["trans_B"]):
         return None
     scores, v = view.ins(n)
-    if not (_is(scores, "matmul") and not scores.attrs["trans_A"] and scores.attrs["trans_B"]):
+    if not (_is(scores, "matmul") and not scores.attrs["trans_A"]):
         return None
+    k_major = not scores.attrs["trans_B"]
     q, k = view.ins(scores)
     if not all(isinstance(t, PlaceHolderNode) for t in (q, k, v)):
         return None
     if view.is_split:
         raise LoweringRejected("a chained matmul has no split form here")
-    sq_, sk_ = tuple(q.shape), tuple(k.shape)
-    if len(sq_) != len(sk_) or len(sq_) < 2 or tuple(v.shape[:-1]) != sk_[:-1] or sq_[-1] != sk_[-1]:
-        raise LoweringRejected(f"chained matmul operands do not line up: {sq_}, {sk_}, {tuple(v.shape)}")
+    sq_, sv_ = tuple(q.shape), tuple(v.shape)
+    sk_ = tuple(k.shape[:-2]) + (k.shape[-1], k.shape[-2]) if k_major else tuple(k.shape)   # as (.., keys, d)
+    if len(sq_) != len(sk_) or len(sq_) < 2 or sv_[:-1] != sk_[:-1] or sq_[-1] != sk_[-1]:
+        raise LoweringRejected(f"chained matmul operands do not line up: {sq_}, {tuple(k.shape)}, {sv_}")
     bq, bk = sq_[:-2], sk_[:-2]
     for i, (x, y) in enumerate(zip(bq, bk)):
         if x != y and (i != len(bq) - 1 or x % y):
             raise LoweringRejected("leading extents of a chained matmul must agree (or group on the innermost one)")
     units = math.prod(bk)
     prob = {"units": units, "group": math.prod(bq) // units, "sq": sq_[-2], "skv": sk_[-2], "head_dim": sq_[-1],
-            "vdim": v.shape[-1], "scale": 1.0, "exact": False, "shift": 0.0, "linear": True}
+            "vdim": sv_[-1], "scale": 1.0, "exact": False, "shift": 0.0, "linear": True, "k_major": k_major}
     return "attention", prob, {"Q": q, "K": k, "V": v}
 
 

@@ -162,7 +162,7 @@ def _attn_scores(low, feed):
         k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + norm["k"])
     units, rows = p["units"], p["group"] * p["sq"]
     q = q.reshape(units, rows, p["head_dim"])
-    k = k.reshape(units, p["skv"], p["head_dim"])
+    k = k.reshape(units, p["head_dim"], p["skv"]).mT if p.get("k_major") else k.reshape(units, p["skv"], p["head_dim"])
     v = v.reshape(units, p["skv"], p["vdim"])
     return (q @ k.mT) * (p["scale"] * LOG2E), v
 

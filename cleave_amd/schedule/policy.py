@@ -379,6 +379,8 @@ def attn_many_rows_candidates(low, role, factor, arch: Arch):
     vd = p["vdim"]
     if (factor or 1) > 1 or rows < 64 or d % 64 or d > 256 or vd % 64 or vd > 256 or p["skv"] < 1:
         return []
+    if p.get("k_major") and p["skv"] % 32:       # feature-major keys are loaded in whole 32-key steps
+        return []
     items = p["units"] * _ceil(rows, 128)
     steps = _ceil(p["skv"], 32)
     # a workgroup-step is 32 matrix ops per wave beside as many vector ops; two workgroups per CU

@@ -135,6 +135,30 @@ def test_chained_matmul_is_attention_without_softmax():
         np.testing.assert_allclose(out[h, s].float().cpu().numpy(), want, rtol=1e-2, atol=1e-2 * max(1.0, np.abs(want).max() / 16))
 
 
+def test_chained_matmul_with_a_feature_major_middle_operand():
+    """``(a @ b) @ c`` with ``b`` stored (K, N): the reference's ``matmul_matmul_small_n`` (4096, 64, 64)
+    and ``matmul_matmul_small_k`` (4096, 4096, 64) cases plus a small ragged-row one, each against
+    the oracle (which keeps the intermediate in fp32; the kernel rounds it to the element type, so
+    the absolute tolerance follows the magnitude of the outputs)."""
+    for dtype, shapes, seed in ((cl.f16, dict(M=200, N=96, K=64), 41), (cl.bf16, dict(M=128, N=32, K=128), 42),
+                                (cl.f16, dict(M=4096, N=64, K=64), 43), (cl.f16, dict(M=4096, N=4096, K=64), 44)):
+        prog = C.matmul_matmul_2d.trace(dtype, **shapes)
+        a, b, c = prog.random_inputs(seed=seed)
+        a = (a.float() / 8).to(a.dtype)                       # keeps sums of thousands of products inside f16
+        print(f"feature-major chained matmul case {dtype} {shapes}", flush=True)
+        out = kernel_for(prog)(a, b, c)
+        torch.cuda.synchronize()
+        want = program_oracle.evaluate(prog, [a, b, c])[0]
+        atol = 1e-2 + np.abs(want).max() * (2.0 ** -6 if dtype is cl.bf16 else 2.0 ** -9)
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=atol)
+        # independent of the oracle: a sample of rows in float64 with the intermediate rounded as the kernel rounds it
+        gen = np.random.default_rng(seed)
+        for m in gen.integers(0, shapes["M"], 8):
+            w = (a[m].float() @ b.float()).to(a.dtype).double()
+            row = (w @ c.double()).float().cpu().numpy()
+            np.testing.assert_allclose(out[m].float().cpu().numpy(), row, rtol=1e-2, atol=1e-2 * max(1.0, np.abs(row).max() / 16))
+
+
 def test_search_prefers_the_shared_kernel_for_many_rows_and_keeps_decode_for_few():
     from cleave_amd.schedule import search_tiling
 

@@ -173,6 +173,43 @@ def test_rmsnorm_matmul_gemm_path():
     _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=dict(BM=64, BN=64, BK=64, WM=2, WN=2), split=4)
 
 
+@pytest.mark.parametrize("template,tiling", [("gemm", dict(BM=64, BN=64, BK=64, WM=2, WN=2)),
+                                             ("gemm_dma", dict(BM=64, BN=64, BK=64, WM=2, WN=2)),
+                                             ("gemm_dma", dict(BM=32, BN=64, BK=64, WM=1, WN=2))])
+@pytest.mark.parametrize("split", [None, 4])
+def test_batched_matmul_split_k(template, tiling, split):
+    """A batch of products, unsplit and split over K into four partial products summed by the
+    combine kernel: the reference's ``batched_matmul_splitk_partial`` / ``_combine`` pair at its
+    size (2 entries of 128 x 128 x 4096, ``tests/schedule/end2end/test_end2end.py:15-16``), a ragged
+    one, and one whose second operand is shared by pairs of entries of the first."""
+    for shapes in (dict(BX=2, BW=2, M=128, N=128, K=4096), dict(BX=3, BW=3, M=72, N=136, K=512),
+                   dict(BX=4, BW=2, M=64, N=128, K=1024)):
+        _check(C.batched_matmul.trace(cl.f16, **shapes), C.inputs_batched, shapes, template=template, tiling=tiling,
+               split=split)
+
+
+def test_rmsnorm_matmul_at_the_large_fused_shape():
+    """RMSNorm -> matmul with many rows, 4096 x 6144 x 4096 (the reference's ``rmsnorm_matmul`` case,
+    ``tests/schedule/end2end/test_end2end.py:37``: no weight, no epsilon), through the register-staged
+    matmul that applies the norm to the A tile on its way into LDS; whole output against the oracle,
+    then a sample of rows recomputed in float64 independently of it."""
+    shapes = dict(M=4096, N=6144, K=4096)
+    prog = C.rmsnorm_matmul_plain.trace(cl.f16, **shapes)
+    x, w = C.inputs_plain_norm(shapes)
+    want = po.evaluate(prog, [x, w])[0]
+    for tiling in (dict(BM=128, BN=128, BK=64, WM=2, WN=2), dict(BM=256, BN=128, BK=64, WM=4, WN=2)):
+        print(f"case rmsnorm_matmul_plain {shapes} {tiling}", flush=True)
+        got = kernel_for(prog, template="gemm", tiling=tiling)(x.cuda(), w.cuda())
+        torch.cuda.synchronize()
+        got = got.float().cpu().numpy()
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+        gen = np.random.default_rng(7)
+        for m in gen.integers(0, shapes["M"], 6):
+            row = x[m].double()
+            ref = ((row / torch.sqrt((row * row).mean())) @ w.double()).numpy()
+            np.testing.assert_allclose(got[m], ref, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("waves", [1, 2, 4])
 @pytest.mark.parametrize("split", [None, 2, 8])
 def test_gqa_decode_small(waves, split):

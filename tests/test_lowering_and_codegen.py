@@ -163,6 +163,22 @@ def test_chained_matmul_is_attention_marked_linear():
     assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}
 
 
+def test_chained_matmul_with_a_feature_major_middle_operand_is_the_same_family():
+    """``(a @ b) @ c`` with ``b`` stored (K, N): the keys of the linear attention are then given
+    feature-major, which the many-row kernel reads through transposing LDS reads."""
+    for shapes in (dict(M=4096, N=4096, K=64), dict(M=4096, N=64, K=64)):
+        prog = C.matmul_matmul_2d.trace(cl.f16, **shapes)
+        g = stage_graph(prog)
+        p = g.lowered.problem
+        assert g.lowered.family == "attention" and p["linear"] and p["k_major"]
+        assert (p["units"], p["sq"], p["skv"], p["head_dim"], p["vdim"]) == (1, 4096, shapes["N"], 64, 64)
+        assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}
+        assert "#define CL_KT 1" in source_for(prog)
+    assert not stage_graph(C.matmul_matmul.trace(cl.f16, H=2, SQ=64, SKV=64, D=64)).lowered.problem["k_major"]
+    with pytest.raises(Exception, match="32-key steps|many-row"):       # 48 keys: no whole steps
+        source_for(C.matmul_matmul_2d.trace(cl.f16, M=256, N=48, K=64))
+
+
 def test_row_reductions_are_a_family():
     for fn, div, out_shape in ((C.rowsum, False, (4096, 1)), (C.rowsum_div, True, (4096, 4096))):
         g = stage_graph(fn.trace(cl.f16, M=4096, N=4096))
