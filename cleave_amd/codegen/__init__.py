@@ -263,8 +263,13 @@ class HipCodeGen:
 
     def _emit_gemm_dma(self, unit, plan, params, partial, combine, fused):
         p, t = plan.problem, plan.tiling
-        if plan.family not in ("matmul", "swiglu", "matmul_rowsum"):
-            raise CodegenError("the direct-to-LDS matmul template has no fused RMSNorm form")
+        if plan.family == "rmsnorm_matmul":
+            # the norm is applied to the product's rows, which needs a norm without a learned weight
+            if p.get("gamma") or p["trans_A"] or (plan.split_factor or 1) > 1 or combine:
+                raise CodegenError("the direct-to-LDS matmul fuses an RMSNorm only without a learned weight, for "
+                                   "row-major A, unsplit")
+        elif plan.family not in ("matmul", "swiglu", "matmul_rowsum"):
+            raise CodegenError(f"the direct-to-LDS matmul template has no {plan.family} form")
         self._matmul_common(unit, plan, params, partial, combine, fused)
         tile = dict(BM=128, BN=128, BK=64, WM=2, WN=2)
         tile.update(t)

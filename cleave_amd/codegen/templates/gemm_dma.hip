@@ -28,6 +28,12 @@
 // workgroup covers BN/2 columns of C; every wave owns the same columns in both halves (half of its
 // column fragments each) and multiplies the two accumulators in its epilogue.
 
+// CL_NORM (fused RMSNorm of the rows of A, no learned weight): C = (A * B) scaled per row by
+// rsqrt(mean(a^2) + eps).  The scale commutes with the product, so the tile pipeline is untouched:
+// every A fragment a wave reads for the matrix cores (each element of its rows exactly once) is also
+// squared and summed on the vector unit, in the shadow of the matrix ops, and the epilogue
+// multiplies.  Unsplit, A given (M, K).
+
 #define GD_WAVES (CL_WM * CL_WN)
 #define GD_THREADS (GD_WAVES * 64)
 #define GD_TM (CL_BM / CL_WM / 16)
@@ -53,6 +59,12 @@
 #endif
 #ifndef CL_TAIL
 #define CL_TAIL 0
+#endif
+#ifndef CL_NORM
+#define CL_NORM 0
+#endif
+#if CL_NORM && (CL_TRANS_A || CL_GAMMA || CL_SPLITS != 1 || CL_SWIGLU || CL_ROWSUM)
+#error "the fused norm of the direct-to-LDS matmul: row-major A, no learned weight, unsplit"
 #endif
 #ifndef CL_ASM_MFMA
 #define CL_ASM_MFMA (GD_TM * GD_TN * 4 > 128)   // wave tiles whose accumulators fill a register half
@@ -175,6 +187,23 @@ CL_DEVICE elem8 gd_read_kmaj(const elem_t* tile, int off0, int j, int s) {
   return __builtin_bit_cast(elem8, v);
 }
 
+// sum of the squares of a fragment's eight elements onto `sum`
+CL_DEVICE float gd_sumsq(elem8 f, float sum) {
+#if CL_BF16
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sum = __builtin_fmaf(to_f32(f[e]), to_f32(f[e]), sum);
+#else
+  typedef _Float16 gd_h2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const gd_h2 pair = {f[2 * q], f[2 * q + 1]};
+    sum = __builtin_amdgcn_fdot2(pair, pair, sum, false);
+  }
+#endif
+  return sum;
+}
+#define GD_SUMSQ_VALU (CL_NORM ? (CL_BF16 ? 24 : 4) : 0)   // vector instructions per fragment
+
 // The matrix op.  Through the compiler's builtin, a wave tile whose accumulators fill a whole
 // register half (8 x 8 fragments = 256 registers) comes out with the accumulators renamed from op
 // to op and copied back inside the loop (three copies per matrix op), and with the load addresses
@@ -223,6 +252,7 @@ constexpr int gd_reads_after(int TM, int s, int i) {
 template <int TM, int S, int I>
 CL_DEVICE void gd_sched_rows() {
   __builtin_amdgcn_sched_group_barrier(0x008, GD_TN, 0);
+  if constexpr (GD_SUMSQ_VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, GD_SUMSQ_VALU, 0);
   constexpr int n = gd_reads_after(TM, S, I);
   if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);
   if constexpr (I + 1 < TM) gd_sched_rows<TM, S, I + 1>();
@@ -347,6 +377,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < GD_TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#if CL_NORM
+  float ss[TM];        // this lane's share of the sum of squares of row am + 16 i + c (k chunks g, g + 4 of every step)
+#pragma unroll
+  for (int i = 0; i < TM; ++i) ss[i] = 0.f;
+#define GD_SUMSQ(i, frag) ss[i] = gd_sumsq(frag, ss[i]);
+#else
+#define GD_SUMSQ(i, frag)
+#endif
 
   // Matrix-core work of one step on one stage, software-pipelined: the B fragments of a 32-wide
   // k block stay in registers, the A fragments stream two ahead of their use, and the next k
@@ -364,6 +402,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                          \
         NEXT(s * TM + i)                                                                         \
         _Pragma("unroll") for (int j = 0; j < GD_TN; ++j) GD_MFMA(acc[i][j], bf[s][j], af[s][i]);              \
+        GD_SUMSQ(i, af[s][i])                                                                       \
         if (s * TM + i + 2 < 2 * TM)                                                          \
           af[(s * TM + i + 2) / TM][(i + 2) % TM] =                                        \
               GD_AFRAG(a_tile, (i + 2) % TM, (s * TM + i + 2) / TM);                       \
@@ -487,6 +526,16 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     return;
   }
 #endif
+#if CL_NORM
+  float row_scale[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    float t = ss[i];
+    t += lane_xor(t, lane, 16);
+    t += lane_xor(t, lane, 32);
+    row_scale[i] = fast_rsqrt(t * (1.0f / CL_K) + CL_EPS);
+  }
+#endif
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = m0 + am + 16 * i + c;
@@ -516,7 +565,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #else
       elem4 y;
 #pragma unroll
+#if CL_NORM
+      for (int r = 0; r < 4; ++r) y[r] = to_elem(v[r] * row_scale[i]);
+#else
       for (int r = 0; r < 4; ++r) y[r] = to_elem(v[r]);
+#endif
       *reinterpret_cast<elem4*>(CL_ARG_OUT + ((i64)batch * CL_M + m) * CL_N + n) = y;
 #endif
     }

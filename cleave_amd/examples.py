@@ -38,6 +38,11 @@ def rmsnorm_matmul_plain(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
 
 
 @cleave_amd.jit
+def rmsnorm_matmul_eps(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
+    return cl.rms_norm(x, dim=-1, eps=1e-2) @ w
+
+
+@cleave_amd.jit
 def swiglu(x: cl.Tensor["M", "K"], w_up: cl.Tensor["K", "N"], w_gate: cl.Tensor["K", "N"]):
     """``(x @ w_up) * silu(x @ w_gate)`` (the reference's ``demo/swiglu.py`` / ``tests/_graphs.py:403-436``)."""
     return (x @ w_up) * cl.silu(x @ w_gate)

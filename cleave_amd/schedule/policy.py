@@ -107,14 +107,17 @@ def gemm_candidates(low, role, factor, arch: Arch):
 
 
 def gemm_dma_candidates(low, role, factor, arch: Arch):
-    """Tilings of the direct-to-LDS matmul (plain matmul only: a fused norm needs the operand in
-    registers on its way to LDS).  No staging registers, so the budget is accumulators plus two
+    """Tilings of the direct-to-LDS matmul: the plain matmul, and the RMSNorm -> matmul without a
+    learned weight, unsplit (the norm then scales the product's rows; with a weight the operand
+    would have to pass through registers on its way to LDS).  No staging registers, so the budget is accumulators plus two
     k blocks of operand fragments; tiles whose accumulators would fill a whole register class
     (256) are left out: the compiler then shuffles them on every step."""
     p = low.problem
-    if low.family != "matmul":
-        return []
     splits = factor or 1
+    post_norm = low.family == "rmsnorm_matmul" and not p.get("gamma") and not p["trans_A"] and splits == 1 \
+        and role == "main"
+    if low.family != "matmul" and not post_norm:
+        return []
     M, N, K = p["M"], p["N"], p["K"]
     if K % (splits * 64) or (not p["trans_B"] and N % 8) or (p["trans_A"] and M % 8):
         return []
@@ -132,6 +135,8 @@ def gemm_dma_candidates(low, role, factor, arch: Arch):
         tm, tn = bm // wm // 16, bn // wn // 16
         if tm & (tm - 1) or tn & (tn - 1) or tm * tn * 4 > 128:
             continue
+        if post_norm and tm * tn * 4 > 64:
+            continue      # the row sums of squares need registers a 128-register accumulator tile does not leave (spills)
         # every wave must own whole 1 KiB load units of both tiles or none
         units_a, units_b = bm // 8, bn // 8
         vgprs = tm * tn * 4 + (tm + tn) * 6 + -(-units_a // (wm * wn)) + -(-units_b // (wm * wn)) + 24

@@ -188,6 +188,25 @@ def test_batched_matmul_split_k(template, tiling, split):
                split=split)
 
 
+@pytest.mark.parametrize("dtype", [cl.f16, cl.bf16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("tiling", [dict(BM=64, BN=64, BK=64, WM=2, WN=2), dict(BM=128, BN=64, BK=64, WM=4, WN=1),
+                                    dict(BM=16, BN=32, BK=64, WM=1, WN=2), dict(BM=256, BN=128, BK=64, WM=4, WN=2)],
+                         ids=lambda t: "x".join(str(v) for v in t.values()))
+def test_rmsnorm_matmul_without_weight_on_the_direct_to_lds_matmul(dtype, tiling):
+    """RMSNorm (no learned weight; with and without an epsilon) fused into the direct-to-LDS matmul
+    as a scale of the product's rows: ragged tile counts on both axes, an odd number of K steps."""
+    shapes = dict(M=200, N=136, K=320)
+    for fn in (C.rmsnorm_matmul_plain, C.rmsnorm_matmul_eps):
+        prog = fn.trace(dtype, **shapes)
+        ins = [t.to(dtype.torch) for t in C.inputs_plain_norm(shapes)]
+        want = po.evaluate(prog, ins)[0]
+        print(f"case {prog.name} {dtype} {shapes} {tiling}", flush=True)
+        got = kernel_for(prog, template="gemm_dma", tiling=tiling)(*[t.cuda() for t in ins])
+        torch.cuda.synchronize()
+        tol = 2e-2 if dtype is cl.bf16 else ATOL          # bf16 outputs of magnitude ~1 carry 8 bits
+        np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=tol, atol=tol)
+
+
 def test_rmsnorm_matmul_at_the_large_fused_shape():
     """RMSNorm -> matmul with many rows, 4096 x 6144 x 4096 (the reference's ``rmsnorm_matmul`` case,
     ``tests/schedule/end2end/test_end2end.py:37``: no weight, no epsilon), through the register-staged
@@ -197,9 +216,11 @@ def test_rmsnorm_matmul_at_the_large_fused_shape():
     prog = C.rmsnorm_matmul_plain.trace(cl.f16, **shapes)
     x, w = C.inputs_plain_norm(shapes)
     want = po.evaluate(prog, [x, w])[0]
-    for tiling in (dict(BM=128, BN=128, BK=64, WM=2, WN=2), dict(BM=256, BN=128, BK=64, WM=4, WN=2)):
-        print(f"case rmsnorm_matmul_plain {shapes} {tiling}", flush=True)
-        got = kernel_for(prog, template="gemm", tiling=tiling)(x.cuda(), w.cuda())
+    for template, tiling in (("gemm", dict(BM=128, BN=128, BK=64, WM=2, WN=2)), ("gemm", dict(BM=256, BN=128, BK=64, WM=4, WN=2)),
+                             ("gemm_dma", dict(BM=256, BN=256, BK=64, WM=4, WN=2)),
+                             ("gemm_dma", dict(BM=256, BN=256, BK=64, WM=4, WN=2, TAIL=128))):
+        print(f"case rmsnorm_matmul_plain {shapes} {template} {tiling}", flush=True)
+        got = kernel_for(prog, template=template, tiling=tiling)(x.cuda(), w.cuda())
         torch.cuda.synchronize()
         got = got.float().cpu().numpy()
         np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
