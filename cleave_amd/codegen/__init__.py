@@ -537,6 +537,8 @@ class HipCodeGen:
             # withdrawn: it measured level with this kernel and its split form once returned a
             # wrong result whose cause was never found.
             raise CodegenError("tiling XW=1 (cross-wave MLA decode) is withdrawn; use WAVES/HG/VSPLIT/STAGES")
+        if int(t.get("DUO", 0)):
+            return self._emit_mla_duo(unit, plan, partial, combine, total_rows)
         waves, hg, stages = int(t.get("WAVES", 4)), int(t.get("HG", 1)), int(t.get("STAGES", 3))
         vsplit = int(t.get("VSPLIT", 1))
         if waves not in (1, 2, 4, 8):
@@ -573,6 +575,36 @@ class HipCodeGen:
             entry, args = self._combine_args
             unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)
 
+
+    def _emit_mla_duo(self, unit, plan, partial, combine, total_rows):
+        """The score-wave / value-wave form of MLA decode: six waves own 64 heads, two making the
+        scores of 32 heads each, four the value products of 32 heads x half the latent features."""
+        p, t, op = plan.problem, plan.tiling, plan.operands
+        if p["heads"] % 64 or p["ckv"] % 128 or p["kpe"] % 64:
+            raise CodegenError("the score-wave / value-wave MLA kernel needs heads % 64 == 0, a latent width in "
+                               "multiples of 128 and a rope width in multiples of 64")
+        from ..schedule.policy import mla_lds_bytes
+
+        if mla_lds_bytes(p["ckv"], p["kpe"], 4) + 11 * 1024 > 160 * 1024:
+            raise CodegenError("four images of the paired-wave MLA kernel do not fit LDS at these widths")
+        for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_SKV", p["skv"]),
+                     ("CL_BATCH", p["batch"]), ("CL_PO_ELEM", 1)):
+            unit.define(k, v)
+        if "LDS_AHEAD" in t:
+            unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
+        for k in t:
+            if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
+                unit.define(f"CL_{k}", 1)
+        unit.define("CL_SCALE_LOG2E", _f(float(p["scale"]) * LOG2E))
+        for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE")):
+            if role in op:
+                unit.define(macro, op[role])
+        unit.templates += ["mla_decode_duo.hip", "attn_combine.hip"]
+        if partial:
+            unit.launch(ENTRY, (p["batch"] * (p["heads"] // 64), plan.split_factor or 1, 1), 384, 0, self._partial_args)
+        if combine:
+            entry, args = self._combine_args
+            unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)
 
     def _emit_mla_paged(self, unit, plan, params, partial, combine, fused):
         """Paged MLA decode (token table, page size 1): one wave per (work item, 16 heads); work

@@ -297,6 +297,40 @@ def test_mla_decode_c4_full(tiling, split):
     _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=tiling, split=split)
 
 
+@pytest.mark.parametrize("split", [None, 2, 3, 8])
+def test_mla_decode_paired_waves_small(split):
+    """The score-wave / value-wave form: 64 and 128 heads, key counts that leave a ragged last step,
+    a single step, more splits than steps (empty splits), unsplit."""
+    fn, dt, mk = C.CASES["c4"]
+    for shapes in (dict(B=2, H=64, D=512, PE=64, SKV=192), dict(B=1, H=128, D=512, PE=64, SKV=120),
+                   dict(B=3, H=64, D=512, PE=64, SKV=48), dict(B=1, H=64, D=256, PE=64, SKV=456)):
+        _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(DUO=1), split=split)
+
+
+def test_mla_decode_paired_waves_rising_maximum():
+    """Scores that keep growing along the KV axis: the score waves raise their reference points
+    several times per split and the value waves must rescale at exactly those steps."""
+    fn, dt, mk = C.CASES["c4"]
+    shapes = dict(B=1, H=64, D=512, PE=64, SKV=512)
+    prog = fn.trace(dt, **shapes)
+    q, kv, q_pe, k_pe = mk(shapes, device="cpu")
+    ramp = torch.linspace(0.2, 6.0, shapes["SKV"]).reshape(1, -1, 1)
+    kv = (kv.float() * 0.2 + ramp * torch.sign(q.float().mean(dim=(1,), keepdim=True))).to(kv.dtype)
+    ins = [q, kv, q_pe, k_pe]
+    want = po.evaluate(prog, ins)[0]
+    for split in (None, 2, 4):
+        kernel = kernel_for(prog, template="mla_decode", tiling=dict(DUO=1), split=split)
+        print(f"case mla paired waves rising maximum split={split}", flush=True)
+        got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("split", [4, 8, 16])
+def test_mla_decode_paired_waves_c4_full(split):
+    fn, dt, mk = C.CASES["c4"]
+    _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=dict(DUO=1), split=split)
+
+
 def test_graph_replay_timer_matches_eager_results_and_time():
     """The graph-replay timer (a fused partial + combine pair captured ``graph_batch`` times):
     every replayed batch must leave the eager result in the output, with the program's own eager
