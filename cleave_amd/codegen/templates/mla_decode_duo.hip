@@ -124,18 +124,19 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int set = scores ? wave - 2 : (wave & 1);
   const int fhalf = wave >> 2;
   const int loader = 2 * (wave & 1) + fhalf;              // value waves: which 8-token group of every panel they load
-  // Workgroups go to the eight XCDs (one L2 each) round-robin in launch order.  The head blocks
-  // that read the same rows (one batch entry, one split) get launch ids 8 apart: they run on one
-  // XCD at about the same time and all but the first find the rows in its L2.
+  // Workgroups go to the eight XCDs (one L2 each) round-robin in launch order.  Every workgroup
+  // of a batch entry is given to one XCD (batch entry b to XCD b % 8): the head blocks of a split
+  // read the same kv rows and the splits of a head block the same Q rows, so each row comes out of
+  // HBM once and every other reader finds it in that L2.
   int b, split, hg_block;
   {
-    constexpr int units = CL_BATCH * CL_SPLITS;
+    constexpr int per_entry = CL_SPLITS * MD_HEAD_GROUPS;
     const int launch = blockIdx.y * gridDim.x + blockIdx.x;
-    if (units % 8 == 0) {
-      hg_block = (launch / 8) % MD_HEAD_GROUPS;
-      const int unit = (launch % 8) + 8 * (launch / (8 * MD_HEAD_GROUPS));
-      b = unit / CL_SPLITS;
-      split = unit % CL_SPLITS;
+    if (CL_BATCH % 8 == 0) {
+      const int k = launch / 8;                              // the k-th workgroup of XCD launch % 8
+      b = launch % 8 + 8 * (k / per_entry);
+      split = (k % per_entry) / MD_HEAD_GROUPS;
+      hg_block = k % MD_HEAD_GROUPS;
     } else {
       split = blockIdx.y;
       b = blockIdx.x / MD_HEAD_GROUPS;
