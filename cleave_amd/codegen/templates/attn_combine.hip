@@ -23,34 +23,33 @@ CL_COMBINE_NAME(CL_COMBINE_PARAMS) {
   p1 = p1 < 0 ? 0 : (p1 > n_idx ? n_idx : p1);
   const int first = req + p0 / chunk_pages;
   const int count = p1 > p0 ? (p1 - 1) / chunk_pages - p0 / chunk_pages + 1 : 0;
-  // items are walked four at a time with every load of a group issued before the first use (the
-  // trip count is a run-time value: left alone, each item's loads wait for the previous item's);
-  // slots past the end repeat the last item with weight zero
-  float m = CL_NEG_BIG;
-  for (int s = 0; s < count; s += 4) {
-    float pm[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int it = s + u < count ? s + u : count - 1;
-      pm[u] = CL_CARG_PM[(i64)(first + it) * CL_Q_HEADS + qh];
-    }
-    m = fmaxf(fmaxf(m, fmaxf(pm[0], pm[1])), fmaxf(pm[2], pm[3]));
-  }
-  float l = 0.f;
+  // One pass, eight items at a time, every load of a group issued before the first use (the trip
+  // count is a run-time value: left alone, each item's loads wait for the previous item's).  The
+  // running maximum is carried along and the sums rescaled when a group raises it, so a request of
+  // up to eight items costs one round trip to memory; slots past the end repeat the last item with
+  // weight zero.
+  float m = CL_NEG_BIG, l = 0.f;
   f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < count; s += 4) {
-    float pm[4], pl[4];
-    f32x4 po[4];
+  for (int s = 0; s < count; s += 8) {
+    float pm[8], pl[8];
+    f32x4 po[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 8; ++u) {
       const int it = s + u < count ? s + u : count - 1;
       const i64 prow = (i64)(first + it) * CL_Q_HEADS + qh;
       pm[u] = CL_CARG_PM[prow];
       pl[u] = CL_CARG_PL[prow];
       po[u] = *reinterpret_cast<const f32x4*>(CL_CARG_PO + prow * CL_VDIM + d);
     }
+    float m_new = m;
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 8; ++u) m_new = fmaxf(m_new, pm[u]);   // (a repeated item's maximum is one the group has anyway)
+    const float keep = fast_exp2(m - m_new);
+    m = m_new;
+    l *= keep;
+    o *= keep;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
       const float f = s + u < count ? fast_exp2(pm[u] - m) : 0.f;
       l += pl[u] * f;
       o += po[u] * f;
