@@ -455,6 +455,24 @@ extern "C" __global__ __launch_bounds__(256) void read_probe(const uint4* __rest
   for (; i < n16; i += stride) { const uint4 a = src[i]; acc.x ^= a.x; acc.y ^= a.y; acc.z ^= a.z; acc.w ^= a.w; }
   if ((acc.x & acc.y & acc.z & acc.w) == 0x9e3779b9u) sink[threadIdx.x] = acc;   // (keeps the loads alive)
 }
+
+// The same bytes as private streams: wave w reads its own contiguous n16 / waves share front to back,
+// eight 1 KiB loads in flight (a decode kernel's pattern: every wave walks its own rows).
+extern "C" __global__ __launch_bounds__(256) void stream_probe(const uint4* __restrict__ src, uint4* __restrict__ sink,
+                                                               unsigned long long n16) {
+  const unsigned long long waves = (unsigned long long)gridDim.x * 4, wave = ((unsigned long long)blockIdx.x * 256 + threadIdx.x) >> 6;
+  const unsigned long long per = n16 / waves / 512 * 512;        // whole groups of eight 64-lane loads
+  const uint4* p = src + wave * per + (threadIdx.x & 63);
+  uint4 acc = {0u, 0u, 0u, 0u};
+  for (unsigned long long i = 0; i < per; i += 512) {
+    uint4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = p[i + 64 * k];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { acc.x ^= v[k].x; acc.y ^= v[k].y; acc.z ^= v[k].z; acc.w ^= v[k].w; }
+  }
+  if ((acc.x & acc.y & acc.z & acc.w) == 0x9e3779b9u) sink[threadIdx.x] = acc;
+}
 """
 
 
@@ -472,10 +490,12 @@ def run_stream_probe(mib=2048, steps=10, warmup=3):
     mod = shim.Module(code)
     args = shim.PackedArgs([("ptr", src.data_ptr()), ("ptr", sink.data_ptr()), ("u64", n // 16)])
     best = 0.0
-    for blocks in (256 * 8, 256 * 16):
-        desc = shim.make_desc(mod.function("read_probe"), (blocks,), (256,), 0, args)
+    for entry, blocks in (("read_probe", 256 * 8), ("read_probe", 256 * 16), ("stream_probe", 172), ("stream_probe", 688),
+                          ("stream_probe", 1376)):
+        desc = shim.make_desc(mod.function(entry), (blocks,), (256,), 0, args)
         ms = shim.time_launches([desc], torch.cuda.current_stream().cuda_stream, warmup, steps)
-        best = max(best, n / ms / 1e6)
+        moved = n if entry == "read_probe" else (n // 16 // (blocks * 4) // 512 * 512) * blocks * 4 * 16
+        best = max(best, moved / ms / 1e6)
     torch.cuda.synchronize()
     del src
     torch.cuda.empty_cache()

@@ -17,31 +17,53 @@ from .kinds import (CAUSAL_KINDS, FIELDS_READ, KINDS, MLA_FIELDS_READ, MLA_KINDS
                     RAGGED_PREFILL_CAUSAL, SLAB_KINDS)
 
 
-def _refuse_unread_fields(spec, optional, read):
-    """A field the chosen layer ignores must still be at its default."""
-    stray = []
-    for f in fields(spec):
-        if f.name not in optional or f.name in read:
+def _fail(message):
+    raise InvalidSpec(message)
+
+
+def _check(rules):
+    """``rules``: (holds, message) pairs in the order a reader would meet the problems; the first
+    one that does not hold is reported."""
+    for holds, message in rules:
+        if not holds:
+            _fail(message() if callable(message) else message)
+
+
+def _whole_numbers(spec, names):
+    for name in names:
+        value = getattr(spec, name)
+        if value is not None and (isinstance(value, bool) or not isinstance(value, int)):
+            _fail(f"{name} must be an int, got {value!r}")
+
+
+def _distinct(what, names):
+    if len(set(names)) != len(names):
+        _fail(f"{what} collide: {names}")
+
+
+def _only_read_fields_are_set(spec, optional, read):
+    """A field that the chosen access layer never looks at must be left at its default: a value
+    there would silently change nothing in the kernel."""
+    defaults = {f.name: f.default for f in fields(spec)}
+    changed = []
+    for name in optional:
+        if name in read:
             continue
-        assert f.default is not MISSING, f"{f.name} has a default_factory and cannot be optional"
-        value = getattr(spec, f.name)
-        if isinstance(f.default, tuple):
-            value = tuple(value)
-        if value != f.default:
-            stray.append(f"{f.name}={value!r}")
-    if stray:
-        raise InvalidSpec(f"the {spec.kind!r} layer does not read {', '.join(stray)}, so setting them "
-                          "would have no effect on the emitted kernel")
-
-
-def _need_ints(pairs):
-    for name, value in pairs:
-        if isinstance(value, bool) or not isinstance(value, int):
-            raise InvalidSpec(f"{name} must be an int, got {value!r}")
+        assert defaults[name] is not MISSING, f"{name} needs a plain default to be optional"
+        value = getattr(spec, name)
+        value = tuple(value) if isinstance(defaults[name], tuple) else value
+        if value != defaults[name]:
+            changed.append(f"{name}={value!r}")
+    if changed:
+        _fail(f"the {spec.kind!r} layer does not read {', '.join(changed)}, so setting them would have no effect "
+              "on the emitted kernel")
 
 
 def _default_pass_configs():
     return {"tl.disable_safe_memory_legalize": True}
+
+
+WARP_POLICIES = ("rows", "cols", "even")
 
 
 @dataclass(frozen=True)
@@ -76,50 +98,40 @@ class PagingSpec:
         return self.num_qo_heads // self.num_kv_heads
 
     def validate(self) -> None:
-        ints = [("num_qo_heads", self.num_qo_heads), ("num_kv_heads", self.num_kv_heads), ("page_size", self.page_size)]
-        if self.rasterization is not None:
-            ints.append(("rasterization", self.rasterization))
-        _need_ints(ints)
-        if self.num_qo_heads <= 0 or self.num_kv_heads <= 0:
-            raise InvalidSpec(f"head counts must be positive, got {self.num_qo_heads}/{self.num_kv_heads}")
-        if self.num_qo_heads % self.num_kv_heads:
-            raise InvalidSpec(f"{self.num_qo_heads} query heads do not divide into {self.num_kv_heads} kv heads, "
-                              "so a block's query tile would not be a whole head group")
-        if self.num_kv_heads <= 1:
-            raise InvalidSpec("a single kv head leaves the cache with no head axis; use the MLA layer instead")
-        if self.kind != RAGGED_PREFILL_CAUSAL and self.group <= 1:
-            raise InvalidSpec(f"{self.num_qo_heads} query heads over {self.num_kv_heads} kv heads leaves a group "
-                              "of 1; the decode layers tile a head group of at least two rows")
-        if self.kind in SLAB_KINDS:
-            if self.page_size <= 1:
-                raise InvalidSpec(f"page_size={self.page_size} makes the slab layer's address split degenerate; "
-                                  f"use kind={PAGED_DECODE!r} for one token per page")
-        elif self.page_size != 1:
-            raise InvalidSpec(f"page_size={self.page_size} needs the slab access layer (kind={PAGED_DECODE_SLAB!r}) "
-                              f"and its {self.last_page_len_input} input; only page_size=1 is expressible by the "
-                              f"{self.kind!r} layer")
-        if len(self.cache_inputs) != 2:
-            raise InvalidSpec(f"expected a (K, V) cache pair, got {self.cache_inputs}")
-        if self.kind not in KINDS:
-            raise InvalidSpec(f"unknown access layer {self.kind!r}; expected {KINDS}")
+        _whole_numbers(self, ("num_qo_heads", "num_kv_heads", "page_size", "rasterization"))
+        q, kv, page = self.num_qo_heads, self.num_kv_heads, self.page_size
+        slab = self.kind in SLAB_KINDS
+        _check([
+            (q > 0 and kv > 0, f"head counts must be positive, got {q}/{kv}"),
+            (kv <= 0 or q % kv == 0, f"{q} query heads do not divide into {kv} kv heads, so a block's query tile "
+                                     "would not be a whole head group"),
+            (kv > 1, "a single kv head leaves the cache with no head axis; use the MLA layer instead"),
+            (self.kind == RAGGED_PREFILL_CAUSAL or kv <= 1 or q // kv > 1,
+             f"{q} query heads over {kv} kv heads leaves a group of 1; the decode layers tile a head group of at "
+             "least two rows"),
+            (not slab or page > 1, f"page_size={page} makes the slab layer's address split degenerate; use "
+                                   f"kind={PAGED_DECODE!r} for one token per page"),
+            (slab or page == 1, f"page_size={page} needs the slab access layer (kind={PAGED_DECODE_SLAB!r}) and its "
+                                f"{self.last_page_len_input} input; only page_size=1 is expressible by the "
+                                f"{self.kind!r} layer"),
+            (len(self.cache_inputs) == 2, f"expected a (K, V) cache pair, got {self.cache_inputs}"),
+            (self.kind in KINDS, f"unknown access layer {self.kind!r}; expected {KINDS}"),
+        ])
         read = FIELDS_READ[self.kind]
-        _refuse_unread_fields(self, OPTIONAL_FIELDS, read)
-        names = [self.indptr_input, self.query_input, self.scale_input, *self.cache_inputs]
-        names += [getattr(self, n) for n in ("index_input", "last_page_len_input", "query_indptr_input") if n in read]
-        if len(set(names)) != len(names):
-            raise InvalidSpec(f"input names collide: {names}")
-        dims = [self.indptr_dim, self.scale_input]
-        dims += [getattr(self, n) for n in ("batch_dim", "tokens_dim", "kv_tokens_dim", "pages_dim", "index_dim")
-                 if n in read]
-        if len(set(dims)) != len(dims):
-            raise InvalidSpec(f"symbolic extent names collide: {dims}")
-        if self.warp_policy not in ("rows", "cols", "even"):
-            raise InvalidSpec(f"unsupported warp policy {self.warp_policy!r}")
-        if tuple(self.grid_order) not in (("batch", "head"), ("head", "batch")):
-            raise InvalidSpec(f"grid_order must permute ('batch', 'head'), got {self.grid_order}")
-        if self.causal != (self.kind in CAUSAL_KINDS):
-            raise InvalidSpec(f"causal={self.causal} does not match the {self.kind!r} layer; only the causal "
-                              "prefill layers mask against the diagonal")
+        _only_read_fields_are_set(self, OPTIONAL_FIELDS, read)
+        per_layer = [getattr(self, n) for n in ("index_input", "last_page_len_input", "query_indptr_input") if n in read]
+        _distinct("input names", [self.indptr_input, self.query_input, self.scale_input, *self.cache_inputs, *per_layer])
+        extents = [getattr(self, n) for n in ("batch_dim", "tokens_dim", "kv_tokens_dim", "pages_dim", "index_dim")
+                   if n in read]
+        _distinct("symbolic extent names", [self.indptr_dim, self.scale_input, *extents])
+        _check([
+            (self.warp_policy in WARP_POLICIES, f"unsupported warp policy {self.warp_policy!r}"),
+            (sorted(self.grid_order) == ["batch", "head"],
+             f"grid_order must permute ('batch', 'head'), got {self.grid_order}"),
+            (self.causal == (self.kind in CAUSAL_KINDS),
+             f"causal={self.causal} does not match the {self.kind!r} layer; only the causal prefill layers mask "
+             "against the diagonal"),
+        ])
 
 
 @dataclass(frozen=True)
@@ -150,44 +162,32 @@ class MLASpec:
     warp_policy: str = "cols"
 
     def validate(self) -> None:
-        ints = [("num_qo_heads", self.num_qo_heads), ("page_size", self.page_size),
-                ("index_window_tiles", self.index_window_tiles)]
-        if self.rasterization is not None:
-            ints.append(("rasterization", self.rasterization))
-        _need_ints(ints)
-        if self.num_qo_heads < 16 or self.num_qo_heads % 16:
-            raise InvalidSpec(f"{self.num_qo_heads} query heads is not a positive multiple of 16; MLA's query tile "
-                              "is the head block itself, so the head count is the matrix-core M extent")
-        if self.index_window_tiles < 1:
-            raise InvalidSpec(f"index_window_tiles={self.index_window_tiles} leaves no window to stage")
-        if self.index_window_tiles == 1 and self.prefetch:
-            raise InvalidSpec("index_window_tiles=1 leaves the prefetch no next tile to read inside the window; "
-                              "set prefetch=False or widen the window")
-        if self.page_size != 1:
-            raise InvalidSpec(f"page_size={self.page_size} would give the MLA cache a slot axis the gather does "
-                              "not index; only page_size=1 is expressible here")
-        if len(self.query_inputs) != 2:
-            raise InvalidSpec(f"expected a (nope, pe) query pair, got {self.query_inputs}")
-        if len(self.cache_inputs) != 2:
-            raise InvalidSpec(f"expected a (ckv, kpe) cache pair, got {self.cache_inputs}")
-        if self.warp_policy not in ("rows", "cols", "even"):
-            raise InvalidSpec(f"unsupported warp policy {self.warp_policy!r}")
-        if self.kind not in MLA_KINDS:
-            raise InvalidSpec(f"unknown MLA access layer {self.kind!r}; expected {MLA_KINDS}")
+        _whole_numbers(self, ("num_qo_heads", "page_size", "index_window_tiles", "rasterization"))
+        heads, window = self.num_qo_heads, self.index_window_tiles
+        _check([
+            (heads >= 16 and heads % 16 == 0,
+             f"{heads} query heads is not a positive multiple of 16; MLA's query tile is the head block itself, so "
+             "the head count is the matrix-core M extent"),
+            (window >= 1, f"index_window_tiles={window} leaves no window to stage"),
+            (window > 1 or not self.prefetch, "index_window_tiles=1 leaves the prefetch no next tile to read inside "
+                                              "the window; set prefetch=False or widen the window"),
+            (self.page_size == 1, f"page_size={self.page_size} would give the MLA cache a slot axis the gather does "
+                                  "not index; only page_size=1 is expressible here"),
+            (len(self.query_inputs) == 2, f"expected a (nope, pe) query pair, got {self.query_inputs}"),
+            (len(self.cache_inputs) == 2, f"expected a (ckv, kpe) cache pair, got {self.cache_inputs}"),
+            (self.warp_policy in WARP_POLICIES, f"unsupported warp policy {self.warp_policy!r}"),
+            (self.kind in MLA_KINDS, f"unknown MLA access layer {self.kind!r}; expected {MLA_KINDS}"),
+        ])
         read = MLA_FIELDS_READ[self.kind]
-        _refuse_unread_fields(self, MLA_OPTIONAL_FIELDS, read)
-        names = [*self.query_inputs, *self.cache_inputs, self.index_input, self.indptr_input, self.scale_input]
-        if "query_indptr_input" in read:
-            names.append(self.query_indptr_input)
-        if len(set(names)) != len(names):
-            raise InvalidSpec(f"input names collide: {names}")
-        dims = [self.pages_dim, self.indptr_dim, self.index_dim, self.scale_input,
-                self.tokens_dim if "tokens_dim" in read else self.batch_dim]
-        if len(set(dims)) != len(dims):
-            raise InvalidSpec(f"symbolic extent names collide: {dims}")
-        if self.causal != (self.kind == MLA_PAGED_PREFILL_CAUSAL):
-            raise InvalidSpec(f"causal={self.causal} does not match the {self.kind!r} layer; only the causal "
-                              "prefill layer masks against the diagonal")
+        _only_read_fields_are_set(self, MLA_OPTIONAL_FIELDS, read)
+        row_ptr = [self.query_indptr_input] if "query_indptr_input" in read else []
+        _distinct("input names", [*self.query_inputs, *self.cache_inputs, self.index_input, self.indptr_input,
+                                  self.scale_input, *row_ptr])
+        _distinct("symbolic extent names", [self.pages_dim, self.indptr_dim, self.index_dim, self.scale_input,
+                                            self.tokens_dim if "tokens_dim" in read else self.batch_dim])
+        _check([(self.causal == (self.kind == MLA_PAGED_PREFILL_CAUSAL),
+                 f"causal={self.causal} does not match the {self.kind!r} layer; only the causal prefill layer masks "
+                 "against the diagonal")])
 
 
 @dataclass(frozen=True)
@@ -205,13 +205,11 @@ class CombineTiling:
     input_scope: str = "g"
 
     def validate(self, head_dim: int) -> None:
-        if self.split <= 1:
-            raise InvalidSpec(f"a split factor of {self.split} is not a split")
-        if not (1 <= self.split_step <= self.split and self.split % self.split_step == 0):
-            raise InvalidSpec(f"split_step={self.split_step} does not divide split={self.split}")
-        if not (1 <= self.cols <= head_dim and head_dim % self.cols == 0):
-            raise InvalidSpec(f"cols={self.cols} does not divide the head dim {head_dim}")
-        if self.loop_kind not in ("serial", "pipelined"):
-            raise InvalidSpec(self.loop_kind)
-        if self.input_scope not in ("s", "g"):
-            raise InvalidSpec(self.input_scope)
+        step, cols = self.split_step, self.cols
+        _check([
+            (self.split > 1, f"a split factor of {self.split} is not a split"),
+            (1 <= step <= self.split and self.split % step == 0, f"split_step={step} does not divide split={self.split}"),
+            (1 <= cols <= head_dim and head_dim % cols == 0, f"cols={cols} does not divide the head dim {head_dim}"),
+            (self.loop_kind in ("serial", "pipelined"), f"unknown loop kind {self.loop_kind!r}"),
+            (self.input_scope in ("s", "g"), f"unknown input scope {self.input_scope!r}"),
+        ])
