@@ -102,13 +102,20 @@ def op_table():
 
 
 STREAM_GBPS = None     # read-only streaming rate measured on this box at start-up (run_stream_probe)
+MATRIX_TFLOPS = None   # rate of a loop of nothing but f16 matrix ops on this box (run_matrix_probe)
 
 
 def roofline(bound, nbytes, flops, us, traffic=None):
     if bound == "mfma":
         achieved = flops / us / 1e6
-        return {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / MFMA_TFLOPS, 4), "traffic": traffic}
+        out = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_TFLOPS, "unit": "TFLOP/s",
+               "frac": round(achieved / MFMA_TFLOPS, 4), "traffic": traffic}
+        if MATRIX_TFLOPS:
+            # second fraction: against a loop of nothing but matrix ops on operands held in registers (no
+            # memory, no LDS, no barrier) on this box in this run: what the clocks under matrix load leave
+            out["measured_matrix_peak"] = round(MATRIX_TFLOPS, 1)
+            out["frac_of_measured_matrix"] = round(achieved / MATRIX_TFLOPS, 4)
+        return out
     achieved = nbytes / us / 1e3
     out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
            "frac": round(achieved / HBM_GBPS, 4), "traffic": traffic}
@@ -476,6 +483,52 @@ extern "C" __global__ __launch_bounds__(256) void stream_probe(const uint4* __re
 """
 
 
+MATRIX_SOURCE = r"""
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+// eight waves per compute unit, each a chain of 16x16x32 f16 matrix ops on eight accumulators; the operands
+// are random values read once (the matrix cores' clock under load depends on how many bits toggle)
+extern "C" __global__ __launch_bounds__(512) void matrix_probe(const h8* __restrict__ src, float* __restrict__ sink, int trips) {
+  const int t = blockIdx.x * 512 + threadIdx.x;
+  h8 a[4], b[4];
+  for (int i = 0; i < 4; ++i) { a[i] = src[(t * 8 + i) & 65535]; b[i] = src[(t * 8 + 4 + i) & 65535]; }
+  f4 c[8];
+  for (int i = 0; i < 8; ++i) c[i] = (f4){0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < trips; ++n) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i & 3], b[(i >> 1) & 3], c[i], 0, 0, 0);
+  }
+  float total = 0.f;
+  for (int i = 0; i < 8; ++i) total += c[i][0] + c[i][1] + c[i][2] + c[i][3];
+  if (total == 12345.f) sink[t] = total;
+}
+"""
+
+
+def run_matrix_probe(trips=20000):
+    """TFLOP/s of a loop of nothing but f16 16x16x32 matrix ops (eight waves per compute unit, operands in
+    registers): the matrix rate this box sustains once its clocks have settled under that load."""
+    import torch
+
+    from cleave_amd.runtime import shim
+
+    code, log_text = shim.compile_source(MATRIX_SOURCE, name="matrix_probe.hip")
+    if not code:
+        raise RuntimeError(log_text)
+    mod = shim.Module(code)
+    src = (torch.randn(65536 * 8, device="cuda") * 0.5).to(torch.float16)
+    sink = torch.zeros(2048 * 512, dtype=torch.float32, device="cuda")
+    blocks = 256 * 4
+    args = shim.PackedArgs([("ptr", src.data_ptr()), ("ptr", sink.data_ptr()), ("i32", trips)])
+    desc = shim.make_desc(mod.function("matrix_probe"), (blocks,), (512,), 0, args)
+    stream = torch.cuda.current_stream().cuda_stream
+    shim.time_launches([desc], stream, 2, 2)                     # ~0.3 s of matrix work before the reading
+    ms = shim.time_launches([desc], stream, 1, 3)
+    torch.cuda.synchronize()
+    flops = blocks * 8 * trips * 8 * 16 * 16 * 32 * 2
+    return flops / ms / 1e9
+
+
 def run_stream_probe(mib=2048, steps=10, warmup=3):
     """GB/s of a read-only stream over ``mib`` MiB (well beyond the 256 MB last-level cache): what
     the memory system of this box returns to a kernel that does nothing else."""
@@ -529,6 +582,10 @@ def main():
     log(f"[probe] read-only stream: {STREAM_GBPS:.0f} GB/s ({STREAM_GBPS / HBM_GBPS:.2f} of the published peak)")
     ops = op_table()
     wanted = [o.strip() for o in args.ops.split(",") if o.strip()]
+    if any(ops.get(n, {}).get("bound") == "mfma" for n in wanted):
+        global MATRIX_TFLOPS
+        MATRIX_TFLOPS = run_matrix_probe()
+        log(f"[probe] matrix ops only: {MATRIX_TFLOPS:.0f} TFLOP/s ({MATRIX_TFLOPS / MFMA_TFLOPS:.2f} of the published peak)")
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     threads = int(os.environ.get("OMP_NUM_THREADS", cores))
     results = {}
