@@ -56,15 +56,16 @@ _LAST_LEVEL_CACHE = 256 << 20      # bytes of memory-side cache in front of HBM 
 
 
 def rotation_sets(input_tensors) -> list | None:
-    """Copies of the inputs to rotate through while timing, or None.  Inputs between 1/16 of and the
-    whole memory-side cache (256 MB here) would be served from that cache by every launch after the
-    first, and candidates would be ranked by a speed no caller sees (a decode step streams weights or
-    a KV cache that other work has evicted since): enough copies are made that consecutive launches
-    read different memory, more than twice the cache in total.  Smaller inputs stay cached in real
-    use as well; larger ones stream anyway."""
+    """Copies of the inputs to rotate through while timing, or None.  Inputs between 1/16 of and
+    twice the memory-side cache (256 MB here) would be served from that cache, wholly or in part (a
+    269 MB working set still finds a good share of itself there), by every launch after the first,
+    and candidates would be ranked by a speed no caller sees (a decode step streams weights or a KV
+    cache that other work has evicted since): enough copies are made that consecutive launches read
+    different memory, at least twice the cache in total.  Smaller inputs stay cached in real use as
+    well; larger ones stream anyway."""
     tensors = [t for t in input_tensors if hasattr(t, "element_size")]
     live = _live_bytes(tensors)
-    if not (_LAST_LEVEL_CACHE // 16 <= live < _LAST_LEVEL_CACHE):
+    if not (_LAST_LEVEL_CACHE // 16 <= live < 2 * _LAST_LEVEL_CACHE):
         return None
     copies = min(8, -(-2 * _LAST_LEVEL_CACHE // live)) - 1
     return [[t.clone() if hasattr(t, "element_size") else t for t in input_tensors] for _ in range(copies)]
