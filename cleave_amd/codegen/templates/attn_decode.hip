@@ -26,6 +26,7 @@
 //                per kv head, so that the eight waves together stream whole contiguous token
 //                rows of the cache and a long request costs many items rather than long ones.
 
+#define ATT_RAISE_BY 8.0f
 #ifndef CL_CHUNK_PAGES
 #define CL_CHUNK_PAGES 0
 #endif
@@ -234,7 +235,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
   }
 
-  float m_run = CL_NEG_BIG;   // running max of the scaled scores (log2 domain), uniform over g
+  float m_run = CL_NEG_BIG;   // reference point of the row's scaled scores (log2 domain, within 8 of their running max), uniform over g
   float l_run = 0.f;          // this lane's share of the running sum
   f32x4 acc[ATT_VC][8];       // acc[vc][j][r] = O[row c][128 vc + 32 g + 8 r + j]
 #pragma unroll
@@ -291,14 +292,23 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           s[4 * h + q] = t < u.kv_len ? st[q] * scale2 : CL_NEG_BIG;
         }
       }
+      // The softmax reference point of a row is raised only when a score passes it by more than 8
+      // (a factor 2^8: weights stay below 256, softmax does not depend on the reference point), so
+      // after the first steps of a split the maxima are not even compared across the four lane
+      // groups and the accumulators are not rescaled: both happen only when some lane asks.
       float mx = s[0];
 #pragma unroll
       for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-      mx = fmaxf(mx, lane_xor(mx, lane, 16));
-      mx = fmaxf(mx, lane_xor(mx, lane, 32));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2(m_run - m_new);
-      m_run = m_new;
+      float alpha = 1.0f;
+      if (__builtin_amdgcn_ballot_w64(mx > m_run + ATT_RAISE_BY)) {     // wave-uniform, cold
+        mx = fmaxf(mx, lane_xor(mx, lane, 16));
+        mx = fmaxf(mx, lane_xor(mx, lane, 32));
+        if (mx > m_run + ATT_RAISE_BY) {
+          alpha = fast_exp2(m_run - mx);
+          m_run = mx;
+        }
+      }
+      const float m_new = m_run;
       elem8 pf;
       float psum = 0.f;
 #pragma unroll
