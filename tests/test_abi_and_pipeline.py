@@ -292,6 +292,9 @@ def test_saved_paged_kernel_holds_its_program_as_json(tmp_path):
     assert isinstance(back, PagedKernel) and back.spec == kernel.spec and back.source == "// main"
     assert back.dispatch["min_tiles"] == 3 and back.dispatch_sources == kernel.dispatch_sources
     assert [p.name for p in back.attention.inputs] == [p.name for p in attention.inputs]
+    # the host-side dispatch rule: kv tiles of the longest request against the calibrated threshold
+    back.dispatch.update(page_size=64, kv_tile=32)
+    assert back.dispatch_role(1) == "single" and back.dispatch_role(2) == "split"       # 64 tokens = 2 tiles < 3 <= 4 tiles
     document = json.loads((folder / "kernel.json").read_text())
     document["paged"] = "program.pkl"
     (folder / "kernel.json").write_text(json.dumps(document))

@@ -127,6 +127,18 @@ def test_compile_dynamic_paged_decode(cache_root):
     _close(out, want_o)
     live = np.isfinite(want_l)
     np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
+    # a caller that knows its longest request picks the split pair or the single kernel on the host:
+    # both sides of the calibrated threshold give the same answer as the plain call, also after a reload
+    assert rep.dispatch is not None
+    pages = max(-(-n // 64) for n in lens)
+    roles = {kernel.dispatch_role(1), kernel.dispatch_role(10 ** 6)}
+    assert roles == {"single", "split"}
+    reloaded = cleave_amd.pipeline.load(kernel.save(cache_root / "saved_paged"))
+    for k in (kernel, reloaded):
+        for longest in (1, pages, 10 ** 6):
+            o2, l2 = k(*args, longest=longest)
+            _close(o2, want_o)
+            np.testing.assert_allclose(l2.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
 
 
 @pytest.mark.parametrize("name", ["gqa_paged_decode_h32_kv4_d128_ps1", "gqa_paged_decode_h32_kv8_d128_ps1"])
