@@ -577,21 +577,26 @@ class HipCodeGen:
 
 
     def _emit_mla_duo(self, unit, plan, partial, combine, total_rows):
-        """The score-wave / value-wave form of MLA decode: six waves own 64 heads, two making the
-        scores of 32 heads each, four the value products of 32 heads x half the latent features."""
+        """The score-wave / value-wave form of MLA decode: eight waves own 64 heads, four making the
+        scores of 32 heads x half of each step's tokens, four the value products of 32 heads x half
+        the latent features."""
         p, t, op = plan.problem, plan.tiling, plan.operands
         if p["heads"] % 64 or p["ckv"] % 128 or p["kpe"] % 64:
             raise CodegenError("the score-wave / value-wave MLA kernel needs heads % 64 == 0, a latent width in "
                                "multiples of 128 and a rope width in multiples of 64")
         from ..schedule.policy import mla_lds_bytes
 
-        if mla_lds_bytes(p["ckv"], p["kpe"], 4) + 11 * 1024 > 160 * 1024:
+        if mla_lds_bytes(p["ckv"], p["kpe"], 4) + 9 * 1024 > 160 * 1024:
             raise CodegenError("four images of the paired-wave MLA kernel do not fit LDS at these widths")
         for k, v in (("CL_HEADS", p["heads"]), ("CL_CKV", p["ckv"]), ("CL_KPE", p["kpe"]), ("CL_SKV", p["skv"]),
                      ("CL_BATCH", p["batch"]), ("CL_PO_ELEM", 1)):
             unit.define(k, v)
         if "LDS_AHEAD" in t:
-            unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
+            ahead = int(t["LDS_AHEAD"])
+            if ahead < 2 or ahead % 2 or (p["ckv"] // 32) % (ahead // 2):
+                raise CodegenError("LDS_AHEAD of the score-wave / value-wave MLA kernel: an even number of reads whose "
+                                   "half divides the feature blocks of a value wave")
+            unit.define("CL_LDS_AHEAD", ahead)
         for k in t:
             if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
                 unit.define(f"CL_{k}", 1)
@@ -601,7 +606,7 @@ class HipCodeGen:
                 unit.define(macro, op[role])
         unit.templates += ["mla_decode_duo.hip", "attn_combine.hip"]
         if partial:
-            unit.launch(ENTRY, (p["batch"] * (p["heads"] // 64), plan.split_factor or 1, 1), 384, 0, self._partial_args)
+            unit.launch(ENTRY, (p["batch"] * (p["heads"] // 64), plan.split_factor or 1, 1), 512, 0, self._partial_args)
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (-(-(total_rows * (p["ckv"] // 8)) // 256), 1, 1), 256, 0, args)

@@ -10,36 +10,54 @@
 // LDS read: 272 KB out of LDS per step and 64 heads, at the ~128 bytes per clock a compute unit's
 // LDS delivers twice as long as the matrix ops take.  Sharing an operand between two head tiles
 // needs the registers of 32 heads (Q fragments 144, accumulators 256), which one wave does not
-// have.  Two kinds of wave do:
+// have.  Two kinds of wave do, eight waves for 64 heads:
 //
-//   score wave s (2 of them)    keeps the Q fragments of heads 32 s .. 32 s + 31; every key
+//   score wave (s, h) (4)       keeps the Q fragments of heads 32 s .. 32 s + 31 and makes their
+//                               scores against tokens 16 h .. 16 h + 15 of every step; every key
 //                               fragment it reads feeds two matrix ops (its two head tiles).  It
-//                               makes the scores of step t, the softmax weights against its
-//                               reference points, their row sums, and leaves the weights (as the
-//                               value product's B operand, 16 bytes per lane and head tile) and a
-//                               rescale factor per head in LDS;
+//                               turns them into weights against reference points of its own (one
+//                               per head) and leaves the weights (its half of the value product's
+//                               B operand, 8 bytes per lane and head tile) and the reference
+//                               points it used in LDS;
 //   value wave (s, f) (4)       keeps the accumulators of the same 32 heads for half of the
-//                               latent features (2 x 16 x 16 x 16 values); every value fragment it
-//                               reads feeds two matrix ops.  It picks the weights of step t - 1 up
-//                               and adds their value product.  The value waves also issue every
-//                               tile load.
+//                               latent features (2 x 16 x 16 x 16 values), the weight sums and the
+//                               reference points the accumulators stand against; every value
+//                               fragment it reads feeds two matrix ops.  It picks the weights of
+//                               step t - 1 up and adds their value product.  The value waves also
+//                               issue every tile load and write the result.
 //
-// Per step and 64 heads that is 72 + 72 KB out of LDS for the same 276 matrix ops, which brings
-// the two limits level.  The waves sit on the four SIMDs as {value, value}, {value, value},
-// {score}, {score} (wave w runs on SIMD w % 4): 66 to 72 matrix ops per SIMD and step.  The loop is
-// skewed by one step, one barrier per step: in iteration t the score waves read image t and the
-// value waves image t - 1, the loads of images t + 1 and t + 2 are in flight (four images).
+// Per step and 64 heads that is 72 + 72 KB out of LDS for 280 matrix ops.  Every SIMD holds one
+// score wave and one value wave (wave w runs on SIMD w % 4): 70 matrix ops per SIMD and step, and
+// what a score wave does outside the matrix unit -- wait for its first key fragments after the
+// barrier, then maxima, exponentials and the hand-over, a third of its step -- runs under the
+// value wave's matrix ops (measured: 0.90 us per step against 1.0 with the score waves paired on
+// two SIMDs and the value waves on the other two).  The loop is skewed by one step, one barrier
+// per step: in iteration t the score waves read image t and the value waves image t - 1, the
+// loads of images t + 1 and t + 2 are in flight (four images).  A value wave reads the operands
+// of its first feature blocks of image t at the end of iteration t, across the barrier, and asks
+// for the panels of image t + 2 between its matrix ops.
 //
-// Softmax reference: a head's reference point is raised only when a score passes it by 2^8; the
-// score wave then also publishes alpha = 2^(old - new) for that step (1 otherwise) and the value
-// waves multiply their accumulators by it before adding the step -- the factor travels with the
-// weights it belongs to, so there is no handshake.  At the end the score waves hand over (m, l).
+// Ends of the kernel.  The 64 heads' Q rows reach the score waves through LDS (whole 1 KiB runs
+// into the LDS of the two images loaded last; read straight from global memory a fragment is
+// sixteen 64-byte pieces per instruction and both token halves would fetch the same rows: 3 us
+// more before the first step at 16 x 128 heads), and the value waves' results leave through LDS
+// as whole half rows (2 us less than 8-byte pieces).
+//
+// Softmax reference points without a handshake.  A score wave raises a head's reference point
+// only when a score of its own tokens passes it by 2^8, so its weights never exceed 2^8; with
+// each step's weights it publishes the points it used, and one step later adopts the other token
+// half's points where those are higher (a maximum, nothing to rescale: score waves keep no
+// sums).  The value waves compare the two published points of a step with the point their
+// accumulators stand against: equal on ordinary steps; otherwise (cold) they take the highest
+// of the three, scale accumulators and sums by 2^(old - new) and the weights of a token half
+// that used a lower point by 2^(its - new), rounded to 16 bits again (the sums are taken over the
+// weights as used).
 //
 //   CL_HEADS (multiple of 64)  CL_CKV (multiple of 128)  CL_KPE (multiple of 64)  CL_SKV  CL_BATCH
-//   CL_SPLITS  CL_SCALE_LOG2E  CL_PO_ELEM (1: split partials normalised, in the element type)
+//   CL_SPLITS  CL_SCALE_LOG2E  CL_PO_ELEM (must be 1: split partials normalised, in the element type)
 
-#ifndef CL_PO_ELEM
-#define CL_PO_ELEM 0
+#if CL_SPLITS > 1 && !CL_PO_ELEM
+#error "the score-wave / value-wave kernel writes its split partials in the element type"
 #endif
 #define MD_STEP 32
 #define MD_D (CL_CKV + CL_KPE)
@@ -51,11 +69,14 @@
 #define MD_KJ (MD_D / 32)
 #define MD_FB (CL_CKV / 16)
 #define MD_FBW (MD_FB / 2)                       // feature blocks one value wave accumulates
-#define MD_THREADS 384
+#define MD_THREADS 512
 #define MD_HEADS_PER_BLOCK 64
 #define MD_HEAD_GROUPS (CL_HEADS / MD_HEADS_PER_BLOCK)
 #define MD_UNITS_PER MD_PANELS                  // 1 KiB loads per value wave and step: its 8-token group of every panel
 #define MD_RESCALE_STEP 8.0f
+#define MD_QCHUNKS (MD_D / 8)                    // 16-byte chunks of one head's Q row (latent + rope)
+#define MD_OROW (16 * MD_FBW * 2 + 16)           // bytes of a staged half row of results: its 16-bit values and a 16-byte gap
+#define MD_REF_FLOOR (-1.0e20f)                   // lowest reference point: a token half with every token masked stands here
 #ifndef CL_LDS_AHEAD
 #define CL_LDS_AHEAD 8
 #endif
@@ -63,12 +84,32 @@ static_assert(CL_CKV % 128 == 0 && CL_KPE % 64 == 0, "whole 64-feature panels, t
 static_assert(CL_HEADS % MD_HEADS_PER_BLOCK == 0, "64 heads per workgroup");
 static_assert(CL_SCALE_LOG2E > 0.f, "the largest raw score must be the largest scaled one");
 static_assert(MD_UNITS_PER < 32, "load counter range");
+static_assert(4 * 16 * MD_OROW <= MD_TILE * 2, "the four value waves' staged rows fit one image slot");
 constexpr bool MD_RAGGED = CL_SKV % MD_STEP != 0;
 
 __shared__ __attribute__((aligned(1024))) elem_t md_tiles[MD_STAGES * MD_TILE];
-__shared__ __attribute__((aligned(16))) u32x4 md_weights[2][2][2][64]; // [step parity][head set][head tile][lane]: the lane's eight weights
-__shared__ float md_alpha[2][2][2][64];                                // the same index: rescale factor of head lane % 16 of the tile
-__shared__ float md_final[2][2][2][16];                                // [head set][head tile][m, l][head]
+// [step parity][head set][head tile][lane][token half]: the lane's four weights of each token half
+__shared__ __attribute__((aligned(16))) u32x2 md_weights[2][2][2][64][2];
+// [step parity][head set][head tile][head][token half]: the reference point those weights stand against
+__shared__ __attribute__((aligned(8))) float md_ref[2][2][2][16][2];
+
+#ifdef CL_DBG_TIME
+// measurement switch (the result is wrong by design): every wave stamps the shader clock at the
+// marks below, and when a workgroup ends its stamps overwrite a piece of the Q operand
+__shared__ unsigned long long md_stamps[8][48];
+#define MD_MARK(k) do { md_last = __builtin_amdgcn_s_memtime(); if (lane == 0) md_stamps[wave][(k)] = md_last; } while (0)
+// time since the previous MD_MARK / MD_SUB of this wave, added up in slot 38 + k
+#define MD_SUB(k) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long now_ = __builtin_amdgcn_s_memtime(); \
+    md_sub[k] += now_ - md_last; md_last = now_; __builtin_amdgcn_sched_barrier(0); } while (0)
+#define MD_MARK_WALL(k) do { if (lane == 0) md_stamps[wave][(k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define MD_DUMP() do { if (lane < 4) md_stamps[wave][38 + lane] = md_sub[lane]; __builtin_amdgcn_s_waitcnt(0xC07F); if (lane < 48) \
+    ((unsigned long long*)CL_ARG_Q)[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 48 + lane] = md_stamps[wave][lane]; } while (0)
+#else
+#define MD_MARK(k)
+#define MD_SUB(k)
+#define MD_MARK_WALL(k)
+#define MD_DUMP()
+#endif
 
 typedef short md_s16x4 __attribute__((ext_vector_type(4)));
 typedef short md_s16x8 __attribute__((ext_vector_type(8)));
@@ -81,6 +122,14 @@ template <int OFF>
 CL_DEVICE void md_dma16(const void* gptr, unsigned lds_byte) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off offset:%2"
                :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)), "n"(OFF) : "memory", "m0");
+}
+
+// the same between the matrix ops of a loop body: without the compiler-level memory barrier (the
+// slot written is one no wave reads before the next workgroup barrier), so LDS reads may still be
+// scheduled across it
+CL_DEVICE void md_dma16_loose(const void* gptr, unsigned lds_byte) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_byte)) : "m0");
 }
 
 // every LDS access of this wave has completed, then the workgroup barrier
@@ -113,16 +162,36 @@ CL_DEVICE void md_issue_from(u32 lat_off, u32 pe_off, const elem_t* lat_rows, co
   }
 }
 
+// value wave `lw`: its load of panel `p` of one step (p constant after unrolling)
+CL_DEVICE void md_issue_panel(int p, u32 lat_off, u32 pe_off, const elem_t* lat_rows, const elem_t* pe_rows, int t0,
+                              unsigned stage_byte, int lw) {
+  const unsigned lds_byte = stage_byte + (unsigned)(p * MD_PANEL * 2 + lw * 1024);
+  const bool lat = p < MD_LAT_PANELS;
+  const int col = 64 * (lat ? p : p - MD_LAT_PANELS);
+  if (MD_RAGGED) {
+    const int lane = threadIdx.x & 63;
+    const int r = 8 * lw + (lane >> 3);
+    int t = t0 + r;
+    t = t < CL_SKV - 1 ? t : CL_SKV - 1;
+    const int chunk = (lane & 7) ^ md_swz(r);
+    md_dma16_loose(lat ? lat_rows + (i64)(t - t0) * CL_CKV + col + 8 * chunk : pe_rows + (i64)(t - t0) * CL_KPE + col + 8 * chunk,
+                   lds_byte);
+  } else {
+    md_dma16_loose(lat ? reinterpret_cast<const char*>(lat_rows + col) + lat_off
+                       : reinterpret_cast<const char*>(pe_rows + col) + pe_off, lds_byte);
+  }
+}
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(MD_THREADS)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
-  // waves 2, 3: score waves of head sets 0, 1; waves 0, 4 / 1, 5: value waves of head set 0 / 1,
-  // feature halves 0, 1
-  const bool scores = wave == 2 || wave == 3;
-  const int set = scores ? wave - 2 : (wave & 1);
-  const int fhalf = wave >> 2;
+  // waves 0..3: score waves, waves 4..7: value waves; of both, wave w has head set w % 2 and
+  // token half (score) or feature half (value) (w / 2) % 2.  Wave w runs on SIMD w % 4: one score
+  // wave and one value wave on every SIMD.
+  const bool scores = wave < 4;
+  const int set = wave & 1;
+  const int fhalf = (wave >> 1) & 1;                      // score waves: the token half
   const int loader = 2 * (wave & 1) + fhalf;              // value waves: which 8-token group of every panel they load
   // Workgroups go to the eight XCDs (one L2 each) round-robin in launch order.  Every workgroup
   // of a batch entry is given to one XCD (batch entry b to XCD b % 8): the head blocks of a split
@@ -155,76 +224,113 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   step_end = step_end < n_steps ? step_end : n_steps;
   const int n_own = step_end > step_begin ? step_end - step_begin : 0;       // steps of this split
   const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)md_tiles;
+#ifdef CL_DBG_TIME
+  if (lane < 48) md_stamps[wave][lane] = 0;
+  unsigned long long md_last = 0, md_sub[4] = {0, 0, 0, 0};
+#endif
+  MD_MARK(0);
+  MD_MARK_WALL(1);
 
+  // The Q rows of the 64 heads go through LDS: every wave asks for its share as whole 1 KiB runs
+  // (64 consecutive 16-byte slots each), into the two images' worth of LDS the loop fills last;
+  // slot n holds, for head n / MD_QCHUNKS, the 16-byte chunk (n % MD_QCHUNKS) with its low three
+  // bits XOR head % 8 (the score waves' fragment reads then spread over the banks).  Read straight
+  // from global memory, a fragment is sixteen 64-byte pieces per instruction, and both token
+  // halves would fetch the same rows.
+  if (n_own > 0) {
+    const i64 wg_row0 = (i64)b * CL_HEADS + hg_block * MD_HEADS_PER_BLOCK;
+    for (int k = wave; k < MD_QCHUNKS; k += MD_THREADS / 64) {       // 64 heads x MD_QCHUNKS slots = MD_QCHUNKS runs
+      const int n = 64 * k + lane;
+      const int h = n / MD_QCHUNKS, pos = n % MD_QCHUNKS;
+      const int q = (pos & ~7) | ((pos ^ h) & 7);
+      const elem_t* src = q < CL_CKV / 8 ? CL_ARG_Q + (wg_row0 + h) * CL_CKV + 8 * q
+                                         : CL_ARG_QPE + (wg_row0 + h) * CL_KPE + 8 * (q - CL_CKV / 8);
+      md_dma16<0>(src, tiles_byte + (unsigned)(2 * MD_TILE * 2 + 1024 * k));
+    }
+  }
   if (scores) {
     // =========================================================================== score wave
     // Q fragments (B operand): lane (c, g) holds q[head 16 t + c][32 j + 8 g .. + 8] for head tile t
     elem8 qf[2][MD_KJ];
+    if (n_own > 0) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);             // this wave's runs have landed
+      md_barrier();                                   // and everybody else's
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int j = 0; j < MD_KJ; ++j) {
-        const int col = 32 * j + 8 * g;
-        const i64 row = row0 + 16 * t + c;
-        const elem_t* src = col < CL_CKV ? CL_ARG_Q + row * CL_CKV + col : CL_ARG_QPE + row * CL_KPE + (col - CL_CKV);
-        qf[t][j] = as_elem8(ld16(src));
-      }
-    elem8 ones;
+        for (int j = 0; j < MD_KJ; ++j) {
+          const int h = 32 * set + 16 * t + c, q = 4 * j + g;
+          qf[t][j] = *reinterpret_cast<const elem8*>(md_tiles + 2 * MD_TILE + (h * MD_QCHUNKS + ((q & ~7) | ((q ^ c) & 7))) * 8);
+        }
+    } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) ones[i] = to_elem(1.0f);
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < MD_KJ; ++j) qf[t][j] = (elem8){};
+    }
     float m_run[2] = {CL_NEG_BIG, CL_NEG_BIG};      // reference point of head c of each tile (log2 domain), uniform over g
-    f32x4 l_acc[2];                                 // every component: sum of the weights of head c
-    l_acc[0] = l_acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int a_lo = c * 64 + ((g ^ md_swz(c)) << 3);
+    const int half = fhalf;
+    const int a_lo = (16 * half + c) * 64 + ((g ^ md_swz(c)) << 3);
 
+#ifdef CL_DBG_TIME
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
+    MD_MARK(2);
     for (int it = 0; it <= n_own; ++it) {
       md_barrier();                                 // image `it` has landed (the value waves waited for it)
+      MD_MARK(3 + 2 * it);
       if (it == n_own) break;
       const elem_t* tile = md_tiles + (it % MD_STAGES) * MD_TILE;
 #ifdef CL_DBG_NOS
       continue;
 #endif
-      // scores^T: rows = tokens 16 h + (0..15), columns = heads of tile t
-      f32x4 st[2][2];
+      // the points the other token half used one step ago: asked for first, so that the answer is
+      // there when the matrix ops are done
+      float other[2] = {CL_NEG_BIG, CL_NEG_BIG};
+      if (it > 0) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) st[t][0] = st[t][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < 2; ++t) other[t] = md_ref[(it - 1) & 1][set][t][c][half ^ 1];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // scores^T: rows = tokens 16 half + (0..15), columns = heads of tile t; even and odd
+      // 32-feature slices in accumulators of their own
+      f32x4 sp[2][2];
 #pragma unroll
-      for (int j = 0; j < MD_KJ; ++j)
+      for (int t = 0; t < 2; ++t) sp[t][0] = sp[t][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const elem8 a = *reinterpret_cast<const elem8*>(tile + (j >> 1) * MD_PANEL + 16 * h * 64 +
-                                                          (a_lo ^ ((4 * (j & 1)) << 3)));
+      for (int j = 0; j < MD_KJ; ++j) {
+        const elem8 a = *reinterpret_cast<const elem8*>(tile + (j >> 1) * MD_PANEL + (a_lo ^ ((4 * (j & 1)) << 3)));
 #pragma unroll
-          for (int t = 0; t < 2; ++t) st[t][h] = mfma16(a, qf[t][j], st[t][h]);
-        }
-      // the operand reads stay CL_LDS_AHEAD ahead of the matrix ops that consume them.  (Working the
-      // first token half's weights out between the second half's matrix ops was measured and is
-      // no faster: a wave alone on its SIMD issues its vector and matrix instructions one after
-      // the other either way.)
+        for (int t = 0; t < 2; ++t) sp[t][j & 1] = mfma16(a, qf[t][j], sp[t][j & 1]);
+      }
       __builtin_amdgcn_sched_group_barrier(0x100, CL_LDS_AHEAD, 0);
 #pragma unroll
-      for (int n = 0; n < 2 * MD_KJ - CL_LDS_AHEAD; ++n) {
+      for (int n = 0; n < MD_KJ - CL_LDS_AHEAD; ++n) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * CL_LDS_AHEAD, 0);
+      f32x4 st[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) st[t] = sp[t][0] + sp[t][1];
+#ifdef CL_DBG_TIME
+      asm volatile("" :: "v"(st[0]), "v"(st[1]));
+#endif
+      MD_SUB(0);
 
       if (MD_RAGGED) {
-        const int t0 = (step_begin + it) * MD_STEP;
+        const int t0 = (step_begin + it) * MD_STEP + 16 * half + 4 * g;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (t0 + 16 * h + 4 * g + r >= CL_SKV) st[t][h][r] = CL_NEG_BIG;      // weight exp2(-huge) = 0
+          for (int r = 0; r < 4; ++r)
+            if (t0 + r >= CL_SKV) st[t][r] = CL_NEG_BIG;      // weight exp2(-huge) = 0
       }
-      float mx[2], alpha[2] = {1.0f, 1.0f};
+      float mx[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const float lo = fmaxf(fmaxf(st[t][0][0], st[t][0][1]), fmaxf(st[t][0][2], st[t][0][3]));
-        const float hi = fmaxf(fmaxf(st[t][1][0], st[t][1][1]), fmaxf(st[t][1][2], st[t][1][3]));
-        mx[t] = fmaxf(lo, hi) * CL_SCALE_LOG2E;
+        mx[t] = fmaxf(fmaxf(st[t][0], st[t][1]), fmaxf(st[t][2], st[t][3])) * CL_SCALE_LOG2E;
+        m_run[t] = fmaxf(m_run[t], other[t]);         // adopted where higher
       }
       if (it == 0 || __builtin_amdgcn_ballot_w64(mx[0] > m_run[0] + MD_RESCALE_STEP || mx[1] > m_run[1] + MD_RESCALE_STEP)) {
         // cold after the first step: each head's largest score of this step over all four lane groups
@@ -233,36 +339,26 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           float v = mx[t];
           v = fmaxf(v, lane_xor(v, lane, 16));
           v = fmaxf(v, lane_xor(v, lane, 32));
-          if (it == 0) {
-            m_run[t] = v;                           // nothing accumulated yet: the step's own maximum
-          } else if (v > m_run[t] + MD_RESCALE_STEP) {
-            alpha[t] = fast_exp2(m_run[t] - v);
+          if (it == 0)
+            m_run[t] = fmaxf(v, MD_REF_FLOOR);      // nothing behind it yet: the step's own maximum
+          else if (v > m_run[t] + MD_RESCALE_STEP)
             m_run[t] = v;
-            l_acc[t] *= alpha[t];
-          }
         }
       }
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        elem8 pf;
+        elem4 pf;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            pf[4 * h + r] = to_elem(fast_exp2(__builtin_fmaf(st[t][h][r], CL_SCALE_LOG2E, -m_run[t])));
-        md_weights[it & 1][set][t][lane] = as_u32x4(pf);
-        md_alpha[it & 1][set][t][lane] = alpha[t];
-        l_acc[t] = mfma16(ones, pf, l_acc[t]);      // row sums of exactly the rounded weights
+        for (int r = 0; r < 4; ++r) pf[r] = to_elem(fast_exp2(__builtin_fmaf(st[t][r], CL_SCALE_LOG2E, -m_run[t])));
+        md_weights[it & 1][set][t][lane][half] = __builtin_bit_cast(u32x2, pf);
+        if (g == 0) md_ref[it & 1][set][t][c][half] = m_run[t];
       }
+      MD_SUB(1);
+      MD_MARK(4 + 2 * it);
     }
-    if (g == 0) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        md_final[set][t][0][c] = m_run[t];
-        md_final[set][t][1][c] = l_acc[t][0];
-      }
-    }
-    md_barrier();                                   // (m, l) are there for the value waves
+    MD_MARK(45);
+    MD_MARK_WALL(46);
+    MD_DUMP();
     return;
   }
 
@@ -291,86 +387,149 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int fb = 0; fb < MD_FBW; ++fb) acc[t][fb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  elem8 ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = to_elem(1.0f);
+  f32x4 l_acc[2];                                   // every component: sum of the weights of head c (both feature halves keep it)
+  l_acc[0] = l_acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m_acc[2] = {CL_NEG_BIG, CL_NEG_BIG};        // the reference point accumulators and sums stand against
   const int vtok = 4 * g + (c >> 2);
   const int v_lo = fhalf * (MD_FBW / 4) * MD_PANEL + vtok * 64 + (((((c & 3) >> 1)) ^ md_swz(vtok)) << 3) + 4 * (c & 1);
 
   if (n_own > 0) {
     issue(0);
     issue(1);
+    // this wave's Q runs (asked for before the two images) have landed, then everybody else's
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * MD_UNITS_PER) & 15) | (((2 * MD_UNITS_PER) >> 4) << 14));
+    md_barrier();
   }
+  MD_MARK(2);
+  // the value operands of the first MD_PRE feature blocks of the next image: read at the end of an
+  // iteration, they are on their way while the waves meet at the barrier
+  constexpr int MD_PRE = CL_LDS_AHEAD / 2;
+  static_assert(MD_PRE >= 1 && MD_FBW % MD_PRE == 0, "the read-ahead operands are a ring the feature blocks walk whole turns of");
+  md_s16x4 pre_lo[MD_PRE], pre_hi[MD_PRE];
+#pragma unroll
+  for (int fb = 0; fb < MD_PRE; ++fb) pre_lo[fb] = pre_hi[fb] = (md_s16x4){0, 0, 0, 0};
+  auto operand = [&](const elem_t* tile, int fb, md_s16x4& lo, md_s16x4& hi) __attribute__((always_inline)) {
+    const elem_t* p = tile + (fb >> 2) * MD_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
+    lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((md_lds_s16x4*)(p));
+    hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((md_lds_s16x4*)(p + 16 * 64));
+  };
   for (int it = 0; it <= n_own; ++it) {
     // image `it` must have landed before the barrier lets the score waves read it: at most the
     // loads of image it + 1 may be outstanding (none are issued for an empty split)
     if (n_own > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (MD_UNITS_PER & 15) | ((MD_UNITS_PER >> 4) << 14));
     md_barrier();
-    if (it < n_own) issue(it + 2);                  // into the slot image it - 2 has left
-    if (it == 0) continue;
+    MD_MARK(3 + 2 * it);
+    const elem_t* next_tile = md_tiles + (it % MD_STAGES) * MD_TILE;           // image `it`: there from here on
+    if (it == 0) {
+      if (it < n_own) issue(it + 2);
+#ifndef CL_DBG_NOV
+#pragma unroll
+      for (int fb = 0; fb < MD_PRE; ++fb) operand(next_tile, fb, pre_lo[fb], pre_hi[fb]);
+#endif
+      continue;
+    }
     const elem_t* tile = md_tiles + ((it - 1) % MD_STAGES) * MD_TILE;
 #ifdef CL_DBG_NOV
+    if (it < n_own) issue(it + 2);
     continue;
 #endif
     elem8 pf[2];
-    float alpha[2];
+    f32x2 ref[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      pf[t] = as_elem8(md_weights[(it - 1) & 1][set][t][lane]);
-      alpha[t] = md_alpha[(it - 1) & 1][set][t][lane];
+      pf[t] = as_elem8(*reinterpret_cast<const u32x4*>(&md_weights[(it - 1) & 1][set][t][lane][0]));
+      ref[t] = *reinterpret_cast<const f32x2*>(&md_ref[(it - 1) & 1][set][t][c][0]);
     }
-    if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
-      // cold: the score wave raised a reference point at this step
+    if (__builtin_amdgcn_ballot_w64(ref[0][0] != m_acc[0] || ref[0][1] != m_acc[0] || ref[1][0] != m_acc[1] ||
+                                    ref[1][1] != m_acc[1])) {
+      // cold: a score wave raised a reference point at this step (or this is the first step)
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t) {
+        const float m_new = fmaxf(ref[t][0], ref[t][1]);          // never below m_acc
+        const float alpha = fast_exp2(m_acc[t] - m_new);
+        const float f_lo = fast_exp2(ref[t][0] - m_new), f_hi = fast_exp2(ref[t][1] - m_new);
+        m_acc[t] = m_new;
 #pragma unroll
-        for (int fb = 0; fb < MD_FBW; ++fb) acc[t][fb] *= alpha[t];
+        for (int fb = 0; fb < MD_FBW; ++fb) acc[t][fb] *= alpha;
+        l_acc[t] *= alpha;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pf[t][i] = to_elem(to_f32(pf[t][i]) * (i < 4 ? f_lo : f_hi));
+      }
     }
+#ifdef CL_DBG_TIME
+    asm volatile("" :: "v"(pf[0]), "v"(pf[1]));
+#endif
+    MD_SUB(1);
+    // The loads of image it + 2 (into the slot image it - 2 has left) are asked for between the
+    // matrix ops, panel p after feature block p * MD_FBW / MD_PANELS.  Past the split's end the
+    // last image is asked for again, into the slot of image n_own + 1 (which holds or awaits the
+    // same rows): the load counter then holds the same number of loads at every wait.
+    const int ahead = it + 2 < n_own + 1 ? it + 2 : n_own + 1;
+    const int rel = ahead < n_own - 1 ? ahead : n_own - 1;
+    const int t0 = (step_begin + rel) * MD_STEP;
+    const elem_t* lat_rows = kv + (i64)t0 * CL_CKV;
+    const elem_t* pe_rows = kpe + (i64)t0 * CL_KPE;
+    const unsigned stage_byte = tiles_byte + (unsigned)((ahead % MD_STAGES) * MD_TILE * 2);
     // out^T block fb: rows = features 16 fb + (0..15), slots = tokens 4 g + (0..3), 16 + 4 g + (0..3)
 #pragma unroll
     for (int fb = 0; fb < MD_FBW; ++fb) {
-      const elem_t* p = tile + (fb >> 2) * MD_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
-      const md_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((md_lds_s16x4*)(p));
-      const md_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((md_lds_s16x4*)(p + 16 * 64));
+      md_s16x4 lo = pre_lo[fb % MD_PRE], hi = pre_hi[fb % MD_PRE];
       const elem8 a = __builtin_bit_cast(elem8, (md_s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
       for (int t = 0; t < 2; ++t) acc[t][fb] = mfma16(a, pf[t], acc[t][fb]);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x100, CL_LDS_AHEAD, 0);
+      // the operand MD_PRE blocks on: of this image, or (the last MD_PRE) of the next one
+      if (fb + MD_PRE < MD_FBW)
+        operand(tile, fb + MD_PRE, pre_lo[fb % MD_PRE], pre_hi[fb % MD_PRE]);
+      else
+        operand(next_tile, fb + MD_PRE - MD_FBW, pre_lo[fb % MD_PRE], pre_hi[fb % MD_PRE]);
+#ifndef CL_DBG_NODMA
 #pragma unroll
-    for (int n = 0; n < MD_FBW - CL_LDS_AHEAD / 2; ++n) {
+      for (int pn = 0; pn < MD_PANELS; ++pn)
+        if ((pn * MD_FBW) / MD_PANELS == fb) md_issue_panel(pn, lat_off, pe_off, lat_rows, pe_rows, t0, stage_byte, loader);
+#endif
+    }
+#pragma unroll
+    for (int n = 0; n < MD_FBW; ++n) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, CL_LDS_AHEAD, 0);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) l_acc[t] = mfma16(ones, pf[t], l_acc[t]);      // row sums of exactly the weights used
+    MD_SUB(2);
+    MD_MARK(4 + 2 * it);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);               // no load may still be on its way into LDS when the workgroup ends
-  md_barrier();                                     // the score waves have left (m, l)
+  MD_MARK(44);
 
   // ---- this wave writes its half of the features of its head set --------------------------------
+  // Through LDS, so that a store instruction covers whole half rows (two of 512 bytes at a latent
+  // width of 512) instead of sixteen 32-byte pieces: 16 head rows of MD_OROW bytes in a piece of
+  // LDS only this wave touches -- in the image slot (n_own + 2) % 4, which nothing reads any more
+  // (its image was used up one iteration ago) and no load still in flight writes (those go to the
+  // slots of images n_own and n_own + 1).
+  char* rows = reinterpret_cast<char*>(md_tiles) + ((n_own + 2) % MD_STAGES) * (MD_TILE * 2) + loader * (16 * MD_OROW);
+  constexpr int lanes_per_row = 16 * MD_FBW * 2 / 16;            // 16-byte pieces of a half row
+  constexpr int rows_per_store = 64 / lanes_per_row;
+  static_assert(lanes_per_row <= 64 && 64 % lanes_per_row == 0 && 16 % rows_per_store == 0, "a store covers whole half rows");
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    const float m = md_final[set][t][0][c], l = md_final[set][t][1][c];
-    const i64 orow = row0 + 16 * t + c;
-    const int f0 = 16 * MD_FBW * fhalf + 4 * g;
-#if CL_SPLITS > 1 && !CL_PO_ELEM
-    const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
-#pragma unroll
-    for (int fb = 0; fb < MD_FBW; ++fb) *reinterpret_cast<f32x4*>(CL_ARG_PO + prow * CL_CKV + f0 + 16 * fb) = acc[t][fb];
-    if (g == 0 && fhalf == 0) {
-      CL_ARG_PM[prow] = m;
-      CL_ARG_PL[prow] = l;
-    }
-#else
+    const float m = m_acc[t], l = l_acc[t][0];
+    const i64 orow = row0 + 16 * t;                                // first head row of this tile
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
 #if CL_SPLITS > 1
     const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
-    elem_t* dst_row = CL_ARG_PO + prow * CL_CKV;
+    char* dst = reinterpret_cast<char*>(CL_ARG_PO + prow * CL_CKV + 16 * MD_FBW * fhalf);
     if (g == 0 && fhalf == 0) {
-      CL_ARG_PM[prow] = l > 0.f ? m + fast_log2(l) : CL_NEG_BIG;
-      CL_ARG_PL[prow] = l > 0.f ? 1.0f : 0.f;
+      CL_ARG_PM[prow + c] = l > 0.f ? m + fast_log2(l) : CL_NEG_BIG;
+      CL_ARG_PL[prow + c] = l > 0.f ? 1.0f : 0.f;
     }
 #else
-    elem_t* dst_row = CL_ARG_OUT + orow * CL_CKV;
+    char* dst = reinterpret_cast<char*>(CL_ARG_OUT + orow * CL_CKV + 16 * MD_FBW * fhalf);
 #if CL_EMIT_LSE
-    if (g == 0 && fhalf == 0) CL_ARG_LSE[orow] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
+    if (g == 0 && fhalf == 0) CL_ARG_LSE[orow + c] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
 #endif
 #endif
 #pragma unroll
@@ -378,9 +537,19 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       elem4 y;
 #pragma unroll
       for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[t][fb][r] * inv);
-      *reinterpret_cast<elem4*>(dst_row + f0 + 16 * fb) = y;
+      *reinterpret_cast<elem4*>(rows + c * MD_OROW + (16 * fb + 4 * g) * 2) = y;
     }
-#endif
+#pragma unroll
+    for (int i = 0; i < 16 / rows_per_store; ++i) {
+      const int r = rows_per_store * i + lane / lanes_per_row, piece = lane % lanes_per_row;
+      *reinterpret_cast<u32x4*>(dst + (i64)r * (CL_CKV * 2) + 16 * piece) = *reinterpret_cast<const u32x4*>(rows + r * MD_OROW + 16 * piece);
+    }
   }
+#ifdef CL_DBG_TIME
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
+  MD_MARK(45);
+  MD_MARK_WALL(46);
+  MD_DUMP();
 }
 #endif  // CL_EMIT_PARTIAL

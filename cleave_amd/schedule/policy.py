@@ -455,13 +455,15 @@ def mla_candidates(low, role, factor, arch: Arch):
         out.append(TileDict("mla_decode", role, dict(WAVES=waves, HG=hg, VSPLIT=vsplit, STAGES=stages),
                             output_tile=[heads_per_block, p["ckv"]], rstep_map={"kv": 32}, n_threads=waves * 64,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
-    # The score-wave / value-wave form: six waves own 64 heads, every LDS operand feeds two matrix
-    # ops.  Measured 15-20 % ahead of the best form above wherever both run, so it is ranked first.
-    duo_lds = mla_lds_bytes(p["ckv"], p["kpe"], 4) + 11 * 1024
+    # The score-wave / value-wave form: eight waves own 64 heads, every LDS operand feeds two matrix
+    # ops.  Measured 25-30 % ahead of the best form above wherever both run, so it is ranked first
+    # (with the shorter read-ahead of its value operands as a second candidate).
+    duo_lds = mla_lds_bytes(p["ckv"], p["kpe"], 4) + 9 * 1024
     if out and p["heads"] % 64 == 0 and p["ckv"] % 128 == 0 and duo_lds <= arch.lds_bytes:
-        out.append(TileDict("mla_decode", role, dict(DUO=1), output_tile=[64, p["ckv"]], rstep_map={"kv": 32},
-                            n_threads=384, split_factor=factor, score=0.8 * min(c.score for c in out), lds_bytes=duo_lds,
-                            est_vgprs=224))
+        best = min(c.score for c in out)
+        for tiling, rel in ((dict(DUO=1), 0.75), (dict(DUO=1, LDS_AHEAD=4), 0.76)):
+            out.append(TileDict("mla_decode", role, tiling, output_tile=[64, p["ckv"]], rstep_map={"kv": 32},
+                                n_threads=512, split_factor=factor, score=rel * best, lds_bytes=duo_lds, est_vgprs=208))
     return out
 
 

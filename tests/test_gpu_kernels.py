@@ -299,8 +299,9 @@ def test_mla_decode_c4_full(tiling, split):
 
 @pytest.mark.parametrize("split", [None, 2, 3, 8])
 def test_mla_decode_paired_waves_small(split):
-    """The score-wave / value-wave form: 64 and 128 heads, key counts that leave a ragged last step,
-    a single step, more splits than steps (empty splits), unsplit."""
+    """The score-wave / value-wave form: 64 and 128 heads, key counts that leave a ragged last step
+    (a token half with every token masked among them), a single step, more splits than steps
+    (empty splits), unsplit."""
     fn, dt, mk = C.CASES["c4"]
     for shapes in (dict(B=2, H=64, D=512, PE=64, SKV=192), dict(B=1, H=128, D=512, PE=64, SKV=120),
                    dict(B=3, H=64, D=512, PE=64, SKV=48), dict(B=1, H=64, D=256, PE=64, SKV=456)):
@@ -309,7 +310,8 @@ def test_mla_decode_paired_waves_small(split):
 
 def test_mla_decode_paired_waves_rising_maximum():
     """Scores that keep growing along the KV axis: the score waves raise their reference points
-    several times per split and the value waves must rescale at exactly those steps."""
+    several times per split, each token half on its own, and the value waves must rescale
+    accumulators, sums and the lower half's weights at exactly those steps."""
     fn, dt, mk = C.CASES["c4"]
     shapes = dict(B=1, H=64, D=512, PE=64, SKV=512)
     prog = fn.trace(dt, **shapes)
@@ -323,6 +325,15 @@ def test_mla_decode_paired_waves_rising_maximum():
         print(f"case mla paired waves rising maximum split={split}", flush=True)
         got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
         np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+def test_mla_decode_paired_waves_read_ahead_depths():
+    """The value waves' operand ring at its other depths (2, 4 and 16 feature blocks read ahead, across
+    the barrier at the end of every step)."""
+    fn, dt, mk = C.CASES["c4"]
+    shapes = dict(B=2, H=64, D=512, PE=64, SKV=328)
+    for ahead in (4, 8, 32):
+        _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(DUO=1, LDS_AHEAD=ahead), split=2)
 
 
 @pytest.mark.parametrize("split", [4, 8, 16])

@@ -291,5 +291,11 @@ def test_codegen_refuses_impossible_plans():
                                                             flat_graph=g)).__dict__, "problem": {**g.lowered.problem, "K": 4100}}))
     with pytest.raises(CodegenError, match="no template"):
         HipCodeGen().gen(apply_tiling(TileDict("nonesuch", "main", {}, flat_graph=g)))
+    # the value waves of the score-wave / value-wave MLA kernel walk their read-ahead ring in whole turns
+    mla = stage_graph(C.mla_decode.trace(cl.bf16, B=2, H=64, D=512, PE=64, SKV=256))
+    with pytest.raises(CodegenError, match="LDS_AHEAD"):
+        HipCodeGen().gen(apply_tiling(TileDict("mla_decode", "main", dict(DUO=1, LDS_AHEAD=12), flat_graph=mla)))
+    m = parse_manifest(HipCodeGen().gen(apply_tiling(TileDict("mla_decode", "main", dict(DUO=1, LDS_AHEAD=4), flat_graph=mla))))
+    assert m["launches"][0]["block"] == [512, 1, 1] and m["launches"][0]["grid"][0] == "2"
     with pytest.raises(CodegenError, match="manifest"):
         parse_manifest("__global__ void k() {}")
