@@ -597,6 +597,10 @@ class HipCodeGen:
                 raise CodegenError("LDS_AHEAD of the score-wave / value-wave MLA kernel: an even number of reads whose "
                                    "half divides the feature blocks of a value wave")
             unit.define("CL_LDS_AHEAD", ahead)
+        if "S_AHEAD" in t:
+            if not 1 <= int(t["S_AHEAD"]) <= (p["ckv"] + p["kpe"]) // 32:
+                raise CodegenError("S_AHEAD: between 1 and the key fragments of a step")
+            unit.define("CL_S_AHEAD", int(t["S_AHEAD"]))
         for k in t:
             if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
                 unit.define(f"CL_{k}", 1)

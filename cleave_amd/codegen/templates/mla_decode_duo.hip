@@ -80,6 +80,9 @@
 #ifndef CL_LDS_AHEAD
 #define CL_LDS_AHEAD 8
 #endif
+#ifndef CL_S_AHEAD
+#define CL_S_AHEAD CL_LDS_AHEAD                 // key fragments a score wave asks for ahead of its matrix ops
+#endif
 static_assert(CL_CKV % 128 == 0 && CL_KPE % 64 == 0, "whole 64-feature panels, the latent ones halved between two value waves");
 static_assert(CL_HEADS % MD_HEADS_PER_BLOCK == 0, "64 heads per workgroup");
 static_assert(CL_SCALE_LOG2E > 0.f, "the largest raw score must be the largest scaled one");
@@ -303,13 +306,13 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) sp[t][j & 1] = mfma16(a, qf[t][j], sp[t][j & 1]);
       }
-      __builtin_amdgcn_sched_group_barrier(0x100, CL_LDS_AHEAD, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, CL_S_AHEAD, 0);
 #pragma unroll
-      for (int n = 0; n < MD_KJ - CL_LDS_AHEAD; ++n) {
+      for (int n = 0; n < MD_KJ - CL_S_AHEAD; ++n) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 2 * CL_LDS_AHEAD, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * CL_S_AHEAD, 0);
       f32x4 st[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) st[t] = sp[t][0] + sp[t][1];
