@@ -90,7 +90,8 @@ def op_table():
                       bound="mfma", sets=2),
         "mm2d": dict(title="chained matmul f16 (a@b)@c 4096x4096x64, b given (K, N) (the reference's matmul_matmul_small_k case)",
                      fn=C.matmul_matmul_2d, dtype=cl.f16, shapes=dict(M=4096, N=4096, K=64), inputs=C.inputs_chain2d,
-                     split=False, bytes=2 * (4096 * 64 * 4), flops=2 * 2 * 4096 * 4096 * 64, bound="mfma", sets=4, cpu=False,
+                     split=cl.Split("N", (4, 8, 16)), bytes=2 * (4096 * 64 * 4), flops=2 * 2 * 4096 * 4096 * 64, bound="mfma",
+                     sets=4, cpu=False,
                      # the intermediate a@b is rounded to f16 before the second product (as the reference rounds it):
                      # one flipped last bit of a score of magnitude 16..32 (ulp 2^-6) moves an output by up to 0.05,
                      # while outputs are sums of 4096 such terms with a spread of ~500; the absolute bound follows that

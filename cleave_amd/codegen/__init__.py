@@ -114,7 +114,8 @@ class HipCodeGen:
         """Partial and combine in one unit: the partial's outputs become scratch parameters."""
         if partial.role != "partial" or combine.role != "combine":
             raise CodegenError("a fused pair is [partial, combine]")
-        if partial.template != combine.template and not {partial.template, combine.template} <= {"gemm", "gemm_dma", "skinny"}:
+        pair = {partial.template, combine.template}
+        if len(pair) > 1 and not pair <= {"gemm", "gemm_dma", "skinny"} and pair != {"attn_prefill", "attn_decode"}:
             raise CodegenError(f"partial ({partial.template}) and combine ({combine.template}) templates differ")
         params = [p for p in partial.params if p.role in ("input", "scalar")]
         operands = dict(partial.operands)
@@ -406,7 +407,7 @@ class HipCodeGen:
 
     def _emit_attn_decode(self, unit, plan, params, partial, combine, fused):
         p, t, op = plan.problem, plan.tiling, plan.operands
-        if p.get("norm_eps") or p.get("linear"):
+        if partial and (p.get("norm_eps") or p.get("linear")):
             raise CodegenError("the streaming attention kernel has no QK-norm form and no softmax-free form")
         paged = bool(p.get("paged"))
         rows = p["group"] * p["sq"]
@@ -460,9 +461,10 @@ class HipCodeGen:
         """The LDS-shared prefill kernel over the dense attention family's operands: every unit
         (batch entry x kv head) has ``group * sq`` query rows that all see all keys."""
         p, op = plan.problem, plan.operands
-        if combine or (plan.split_factor or 1) > 1:
-            raise CodegenError("the many-row attention kernel has no split-KV form")
+        splits = plan.split_factor or 1
         d, rows = p["head_dim"], p["group"] * p["sq"]
+        if splits > 1 and p.get("emit_lse"):
+            raise CodegenError("the split form of the many-row attention kernel has no lse output")
         if d % 64 or d > 256 or p["vdim"] % 64 or p["vdim"] > 256:
             raise CodegenError("the many-row attention kernel needs key and value widths in whole 64-feature panels (<= 256)")
         self._attn_common(unit, plan, params, partial, combine, False, p["vdim"], p["units"] * rows, False)
@@ -484,9 +486,13 @@ class HipCodeGen:
         for k, v in plan.tiling.items():
             if k != "SHARED":
                 unit.define(f"CL_PF_{k}", int(v))
-        unit.templates.append("attn_prefill_lds.hip")
-        items = -(-(-(-rows // 128)) // 8) * 8                  # padded to a multiple of 8 (one eighth of the space per XCD)
-        unit.launch(ENTRY, (items, p["units"], 1), 256, 0, self._partial_args)
+        unit.templates += ["attn_prefill_lds.hip", "attn_combine.hip"]
+        if partial:
+            items = -(-(-(-rows // 128)) // 8) * 8              # padded to a multiple of 8 (one eighth of the space per XCD)
+            unit.launch(ENTRY, (items, p["units"], splits), 256, 0, self._partial_args)
+        if combine:
+            entry, args = self._combine_args
+            unit.launch(entry, (-(-(p["units"] * rows * (p["vdim"] // 4)) // 256), 1, 1), 256, 0, args)
 
     def _emit_attn_prefill(self, unit, plan, params, partial, combine, fused):
         if not plan.problem.get("paged"):

@@ -26,6 +26,14 @@
 // CL_SKV and CL_SCALE are constants, an item is 128 consecutive rows of one unit, there are no
 // row pointers and no lse.
 //
+// CL_SPLITS > 1 (dense mode): the 32-key steps are dealt out to CL_SPLITS ranges of
+// ceil(steps / CL_SPLITS) steps each (the split of attn_decode.hip; the last ranges may be short or
+// empty), grid.z = split; a workgroup walks its range only and writes f32 partials (split, row[,
+// feature]): the reference point m, the weight sum l against it and the unnormalised values, which
+// attn_combine.hip merges by the max-rescale rule (an empty range: m = -huge, l = 0, zeros).  In
+// linear mode the partials are plain sums: m = 0 and l = 1 / CL_SPLITS make the same combine add
+// them up.
+//
 // CL_LINEAR (dense mode): no softmax -- out = (q k^T) v, the raw scores times CL_SCALE, rounded to the
 // element type, are the weights; no maxima, no reference, no normalisation.
 //
@@ -76,6 +84,9 @@
 #endif
 #if CL_DENSE && !CL_RAGGED
 #error "dense operands have consecutive key rows (CL_RAGGED)"
+#endif
+#if CL_SPLITS > 1 && !CL_DENSE
+#error "split keys: dense operands only"
 #endif
 #define PL_STEP 32
 #define PL_GROUP (CL_Q_HEADS / CL_KV_HEADS)
@@ -167,11 +178,16 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lo = item * PL_ROWS;
   if (lo >= CL_ROWS) return;                            // (the item axis is padded)
   const int n_rows = CL_ROWS - lo < PL_ROWS ? CL_ROWS - lo : PL_ROWS;
-  const int q0 = 0, kv0 = 0, kv_len = CL_SKV, off = 0, ext = CL_SKV;
+  const int split = CL_SPLITS > 1 ? (int)blockIdx.z : 0;
+  constexpr int steps_per_split = ((CL_SKV + 31) / 32 + CL_SPLITS - 1) / CL_SPLITS;
+  const int key0 = split * steps_per_split * 32;                     // this split's first key
+  int n_keys = CL_SKV - key0 < steps_per_split * 32 ? CL_SKV - key0 : steps_per_split * 32;
+  n_keys = n_keys > 0 ? n_keys : 0;
+  const int q0 = 0, kv0 = 0, kv_len = n_keys, off = 0, ext = n_keys;
   const float sm_scale = CL_SCALE;
   (void)q0; (void)off;
   auto row_index = [&](int m) __attribute__((always_inline)) { return (i64)head * CL_ROWS + lo + m; };
-  auto row_limit = [&](int m) __attribute__((always_inline)) { (void)m; return CL_SKV - 1; };
+  auto row_limit = [&](int m) __attribute__((always_inline)) { (void)m; return n_keys - 1; };
 #else
   // The request whose items include `item`: the last b with b + qo_indptr[b] / PL_QT <= item, found by
   // all lanes at once (one round trip to memory, which also brings the key row pointers).
@@ -208,6 +224,24 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     limit[rt] = live[rt] ? row_limit(m) : -1;
   }
 
+#if CL_SPLITS > 1
+  if (ext == 0) {
+    // a range past the last key: the partial of nothing
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      if (!live[rt]) continue;
+      const i64 prow = (i64)split * CL_TOTAL_ROWS + orow[rt];
+      float* dstp = CL_ARG_PO + prow * CL_VDIM + 4 * g;
+#pragma unroll
+      for (int fb = 0; fb < PL_FB; ++fb) *reinterpret_cast<f32x4*>(dstp + 16 * fb) = (f32x4){0.f, 0.f, 0.f, 0.f};
+      if (g == 0) {
+        CL_ARG_PM[prow] = CL_LINEAR ? 0.f : CL_NEG_BIG;
+        CL_ARG_PL[prow] = CL_LINEAR ? 1.0f / CL_SPLITS : 0.f;
+      }
+    }
+    return;
+  }
+#else
   if (ext == 0) {
     // no row of the item sees a key: zeros and -inf, nothing to read
 #pragma unroll
@@ -222,14 +256,17 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
     return;
   }
+#endif
 
   // the softmax scale as a positive factor of the raw scores (its sign goes into the Q rows, exactly)
   const float scale2 = fmaxf(fabsf(sm_scale) * 1.4426950408889634f, 1.0e-30f);
   const unsigned q_sign = sm_scale < 0.f ? 0x80008000u : 0u;
 #if CL_DENSE
   const i64 krow_bytes = (i64)CL_HEAD_DIM * 2, vrow_bytes = (i64)CL_VDIM * 2;       // K, V: (unit, key, feature)
-  const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_SKV * CL_HEAD_DIM * 2;
-  const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_SKV * CL_VDIM * 2;
+  // (feature-major keys: a key is a column, the split's first key a byte offset along the rows)
+  const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_SKV * CL_HEAD_DIM * 2 +
+                      (i64)key0 * (CL_KT ? 2 : CL_HEAD_DIM * 2);
+  const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + ((i64)head * CL_SKV + key0) * CL_VDIM * 2;
 #else
   // K, V: (key row, kv head, feature)
   const i64 krow_bytes = (i64)CL_KV_HEADS * CL_HEAD_DIM * 2, vrow_bytes = (i64)CL_KV_HEADS * CL_VDIM * 2;
@@ -643,6 +680,25 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
 #endif
     const i64 orow = row_index(m);
+#if CL_SPLITS > 1
+    // split partials: unnormalised f32 values (16 bytes per lane and block), m and l by the g == 0 lanes
+    {
+      const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
+      float* dstp = CL_ARG_PO + prow * CL_VDIM + 4 * g_e;
+#pragma unroll
+      for (int fb = 0; fb < PL_FB; ++fb) *reinterpret_cast<f32x4*>(dstp + 16 * fb) = acc[rt][fb];
+      if (g_e == 0) {
+#if CL_LINEAR
+        CL_ARG_PM[prow] = 0.f;
+        CL_ARG_PL[prow] = 1.0f / CL_SPLITS;
+#else
+        CL_ARG_PM[prow] = m_run[rt];
+        CL_ARG_PL[prow] = l;
+#endif
+      }
+      (void)inv;
+    }
+#else
     // A lane holds features 16 fb + 4 g .. + 3 of its row for every block fb.  Lanes g and g ^ 1
     // trade halves of a pair of blocks (one row swap per register), so that each stores 16
     // contiguous bytes: even g the 8 features from 4 g of the even block, odd g those from
@@ -664,6 +720,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
 #if CL_EMIT_LSE
     if (g_e == 0) CL_ARG_LSE[orow] = l > 0.f ? m_run[rt] + fast_log2(l) : CL_NEG_INF;
+#endif
 #endif
   }
 }

@@ -4,7 +4,8 @@ Everything lives under ``<session cache root>/persistent``: graph-search checkpo
 ``superopt/<k0k1>/<key>/checkpoint.json`` and saved kernels under ``kernels/<name>-<key16>/``
 (the reference lays its cache out the same way, ``python/cleave/pipeline/cache.py:13-50``).  A
 key is a SHA-256 over the inputs that determine the result *and* over this build of the back
-end, so a kernel saved by other templates or another native library is never picked up.
+end (templates, native library and the package's own Python sources: the recogniser and the
+schedule policy decide what a checkpoint holds), so nothing saved by another build is picked up.
 """
 
 from __future__ import annotations
@@ -18,17 +19,20 @@ _build_id = None
 
 
 def build_id() -> str:
-    """``<package version>+<12 hex>``: the hex digests every kernel template and the native
-    library's source, name by name."""
+    """``<package version>+<12 hex>``: the hex digests every kernel template, the native
+    library's source and every Python source of the package, name by name."""
     global _build_id
     if _build_id is None:
         from .. import __version__
         from ..codegen import TEMPLATE_DIR
         from ..runtime.shim import CSRC_DIR
 
+        package = Path(__file__).resolve().parent.parent
         sha = hashlib.sha256()
         for source in sorted(list(TEMPLATE_DIR.glob("*.hip")) + list(CSRC_DIR.glob("*.cpp"))):
             sha.update(source.name.encode() + b"\0" + source.read_bytes())
+        for source in sorted(package.rglob("*.py")):
+            sha.update(str(source.relative_to(package)).encode() + b"\0" + source.read_bytes())
         _build_id = __version__ + "+" + sha.hexdigest()[:12]
     return _build_id
 

@@ -120,7 +120,7 @@ def _split_dim_of(program, lowered) -> str | None:
     if lowered.family in ("matmul", "rmsnorm_matmul", "lora"):
         node, axis = lowered.operands["A"], (-2 if lowered.problem["trans_A"] else -1)
     elif lowered.family == "attention":
-        node, axis = lowered.operands["K"], -2
+        node, axis = lowered.operands["K"], (-1 if lowered.problem.get("k_major") else -2)    # feature-major keys: (d, keys)
     elif lowered.family == "mla":
         node, axis = lowered.operands["KV"], -2
     else:

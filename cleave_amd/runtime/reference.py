@@ -171,7 +171,8 @@ def _eval_attention(low, feed, role, factor, out_dtype, out_shapes):
     import torch
 
     s, v = _attn_scores(low, feed)
-    if low.problem.get("linear"):     # (q k^T) v: the scores themselves, in the storage type, weigh the values
+    linear = bool(low.problem.get("linear"))    # (q k^T) v: the scores themselves, in the storage type, weigh the values
+    if linear and role != "partial":
         return [((s / LOG2E).to(out_dtype).float() @ v).to(out_dtype).reshape(out_shapes[0])]
     if role == "partial":
         n = s.shape[-1]
@@ -181,11 +182,16 @@ def _eval_attention(low, feed, role, factor, out_dtype, out_shapes):
         for i in range(factor):
             lo, hi = min(n, i * per * 32), min(n, (i + 1) * per * 32)
             if hi <= lo:
-                pm.append(torch.full(s.shape[:-1], -1.0e30, device=s.device))
-                pl.append(torch.zeros(s.shape[:-1], device=s.device))
+                pm.append(torch.full(s.shape[:-1], 0.0 if linear else -1.0e30, device=s.device))
+                pl.append(torch.full(s.shape[:-1], 1.0 / factor if linear else 0.0, device=s.device))
                 po.append(torch.zeros(*s.shape[:-1], v.shape[-1], device=s.device))
                 continue
             blk = s[..., lo:hi]
+            if linear:       # plain partial sums: m = 0 and l = 1 / factor make the softmax combine add them up
+                pm.append(torch.zeros(s.shape[:-1], device=s.device))
+                pl.append(torch.full(s.shape[:-1], 1.0 / factor, device=s.device))
+                po.append((blk / LOG2E).to(out_dtype).float() @ v[..., lo:hi, :])
+                continue
             m = blk.amax(-1)
             w = torch.exp2(blk - m.unsqueeze(-1)).to(out_dtype).float()
             pm.append(m)

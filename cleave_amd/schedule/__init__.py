@@ -48,7 +48,8 @@ def _candidates(graph, arch):
         if low.problem.get("norm_eps") or low.problem.get("linear"):
             if not many:
                 raise ScheduleRejected("QK-norm attention and chained matmuls run on the many-row kernel only: at least "
-                                       "64 query rows per unit, widths in 64-feature panels, unsplit")
+                                       "64 query rows per unit, widths in 64-feature panels, keys split into equal ranges "
+                                       "(whole 32-key steps when feature-major)")
             return many
         return policy.attn_candidates(low, role, factor, arch) + many
     if fam == "mla":

@@ -378,16 +378,20 @@ def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
 def attn_many_rows_candidates(low, role, factor, arch: Arch):
     """Units with many query rows (prefill-shaped dense attention): the kernel whose four waves
     share every key tile through LDS, 128 query rows per workgroup, instead of one 16-row tile per
-    workgroup streaming all keys.  Unsplit, key and value widths in 64-feature panels."""
+    workgroup streaming all keys.  Key and value widths in 64-feature panels; split over the keys
+    (ranges of whole 32-key steps, f32 partials) when there are too few units and rows to fill the chip."""
     p = low.problem
     rows, d = p["group"] * p["sq"], p["head_dim"]
     vd = p["vdim"]
-    if (factor or 1) > 1 or rows < 64 or d % 64 or d > 256 or vd % 64 or vd > 256 or p["skv"] < 1:
+    splits = factor or 1
+    if rows < 64 or d % 64 or d > 256 or vd % 64 or vd > 256 or p["skv"] < 1:
+        return []
+    if splits > 1 and p.get("emit_lse"):
         return []
     if p.get("k_major") and p["skv"] % 32:       # feature-major keys are loaded in whole 32-key steps
         return []
-    items = p["units"] * _ceil(rows, 128)
-    steps = _ceil(p["skv"], 32)
+    items = p["units"] * _ceil(rows, 128) * splits
+    steps = _ceil(_ceil(p["skv"], 32), splits)
     # a workgroup-step is 32 matrix ops per wave beside as many vector ops; two workgroups per CU
     score = _waves_time(items, 2, arch) * (steps * 2200 + 9000)
     return [TileDict("attn_prefill", role, dict(SHARED=1), output_tile=[128, vd], rstep_map={"kv": 32}, n_threads=256,

@@ -159,6 +159,42 @@ def test_chained_matmul_with_a_feature_major_middle_operand():
             np.testing.assert_allclose(out[m].float().cpu().numpy(), row, rtol=1e-2, atol=1e-2 * max(1.0, np.abs(row).max() / 16))
 
 
+@pytest.mark.parametrize("split", [2, 4, 8])
+def test_many_row_attention_split_over_the_keys(split):
+    """Keys cut into equal ranges, one workgroup per (128 rows, range), f32 partials merged by the
+    decode kernels' combine: softmax attention (reference points differ per range), key ranges
+    that end inside a 32-key step, and the shifted form."""
+    for fn, dtype, shapes in ((C.gqa_decode_exact, cl.f16, dict(HQ=8, HKV=2, SQ=100, SKV=320, D=64)),
+                              (C.gqa_decode_exact, cl.bf16, dict(HQ=4, HKV=4, SQ=130, SKV=1000, D=128)),
+                              (C.gqa_decode_shift, cl.f16, dict(HQ=8, HKV=4, SQ=64, SKV=200, D=64)),
+                              (C.mla_prefill, cl.f16, dict(H=4, SQ=100, SKV=152, DK=192, DV=128))):
+        prog = fn.trace(dtype, **shapes)
+        args = prog.random_inputs(seed=51 + split)
+        print(f"split-key many-row attention case {prog.name} {dtype} {shapes} split={split}", flush=True)
+        out = kernel_for(prog, template="attn_prefill", tiling=dict(SHARED=1), split=split)(*args)
+        torch.cuda.synchronize()
+        want = program_oracle.evaluate(prog, list(args))[0]
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("split", [2, 8])
+def test_chained_matmul_split_over_the_middle_dimension(split):
+    """``(a @ b) @ c`` with the N walk cut into ranges (plain sums of f32 partials), ``b`` given
+    (K, N) or as its transpose: the reference's (4096, 4096, 64) size and a small one."""
+    for fn, dtype, shapes, seed in ((C.matmul_matmul_2d, cl.f16, dict(M=200, N=256, K=64), 61),
+                                    (C.matmul_matmul_2d, cl.f16, dict(M=4096, N=4096, K=64), 62),
+                                    (C.matmul_matmul, cl.bf16, dict(H=2, SQ=100, SKV=144, D=128), 63)):
+        prog = fn.trace(dtype, **shapes)
+        args = list(prog.random_inputs(seed=seed))
+        args[0] = (args[0].float() / 8).to(args[0].dtype)      # keeps sums of thousands of products inside f16
+        print(f"split chained matmul case {prog.name} {dtype} {shapes} split={split}", flush=True)
+        out = kernel_for(prog, split=split)(*args)
+        torch.cuda.synchronize()
+        want = program_oracle.evaluate(prog, args)[0]
+        atol = 1e-2 + np.abs(want).max() * (2.0 ** -6 if dtype is cl.bf16 else 2.0 ** -9)
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=atol)
+
+
 def test_search_prefers_the_shared_kernel_for_many_rows_and_keeps_decode_for_few():
     from cleave_amd.schedule import search_tiling
 
