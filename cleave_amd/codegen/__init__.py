@@ -427,6 +427,9 @@ class HipCodeGen:
         unit.define("CL_ROWS", rows)
         unit.define("CL_WAVES", waves)
         unit.define("CL_PREFETCH", int(t.get("PREFETCH", 1)))
+        for k in t:
+            if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
+                unit.define(f"CL_{k}", 1)
         chunk_pages = bool(t.get("CHUNK_PAGES", 0)) and paged and (plan.split_factor or 1) > 1
         unit.define("CL_CHUNK_PAGES", chunk_pages)
         unit.define("CL_PAGED", paged)
