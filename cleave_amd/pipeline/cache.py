@@ -18,22 +18,28 @@ LAYOUT_VERSION = 1
 _build_id = None
 
 
+def _fed(hasher, label: str, path: Path) -> None:
+    hasher.update(label.encode() + b"\0" + path.read_bytes())
+
+
 def build_id() -> str:
     """``<package version>+<12 hex>``: the hex digests every kernel template, the native
     library's source and every Python source of the package, name by name."""
     global _build_id
-    if _build_id is None:
-        from .. import __version__
-        from ..codegen import TEMPLATE_DIR
-        from ..runtime.shim import CSRC_DIR
+    if _build_id is not None:
+        return _build_id
+    from .. import __version__
+    from ..codegen import TEMPLATE_DIR
+    from ..runtime.shim import CSRC_DIR
 
-        package = Path(__file__).resolve().parent.parent
-        sha = hashlib.sha256()
-        for source in sorted(list(TEMPLATE_DIR.glob("*.hip")) + list(CSRC_DIR.glob("*.cpp"))):
-            sha.update(source.name.encode() + b"\0" + source.read_bytes())
-        for source in sorted(package.rglob("*.py")):
-            sha.update(str(source.relative_to(package)).encode() + b"\0" + source.read_bytes())
-        _build_id = __version__ + "+" + sha.hexdigest()[:12]
+    package = Path(__file__).resolve().parent.parent
+    hasher = hashlib.sha256()
+    for folder, pattern in ((TEMPLATE_DIR, "*.hip"), (CSRC_DIR, "*.cpp")):
+        for source in sorted(folder.glob(pattern)):
+            _fed(hasher, source.name, source)
+    for source in sorted(package.rglob("*.py")):
+        _fed(hasher, str(source.relative_to(package)), source)
+    _build_id = f"{__version__}+{hasher.hexdigest()[:12]}"
     return _build_id
 
 
@@ -47,7 +53,7 @@ def digest(*parts) -> str:
 def root() -> Path:
     from ..core.session import current_session
 
-    return Path(current_session().cache_root) / "persistent"
+    return Path(current_session().cache_root, "persistent")
 
 
 def superopt_key(program, max_ops: int, split: tuple, concat_matmul: bool) -> str:
@@ -56,10 +62,10 @@ def superopt_key(program, max_ops: int, split: tuple, concat_matmul: bool) -> st
 
 def checkpoint_path(key: str) -> Path:
     """The checkpoint file for ``key``; its directory is created."""
-    folder = root() / "superopt" / key[:2] / key
-    folder.mkdir(parents=True, exist_ok=True)
-    return folder / "checkpoint.json"
+    home = root().joinpath("superopt", key[:2], key)
+    home.mkdir(parents=True, exist_ok=True)
+    return home / "checkpoint.json"
 
 
 def kernel_dir(name: str, key: str) -> Path:
-    return root() / "kernels" / f"{name}-{key[:16]}"
+    return root().joinpath("kernels", name + "-" + key[:16])

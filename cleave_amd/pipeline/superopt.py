@@ -14,170 +14,197 @@ from __future__ import annotations
 
 import json
 import time
-from dataclasses import dataclass, field
-from typing import Any, Callable, Sequence
+from collections.abc import Sequence
 
 from ..core.errors import LoweringRejected, SpecError, SuperoptError
 from . import cache
 from .config import SuperoptConfig
 
 _IO_OPS = ("kn_input_op", "kn_output_op")
+_GRAPH_FIELDS = ("index", "structure", "is_split", "split", "invalid_split", "split_rejection")   # what a checkpoint keeps
 
 
 def program_dtype(program) -> str:
     return str(getattr(program, "dtype", None) or "float16")
 
 
-def _op_name(op_type: str) -> str:
-    name = op_type
-    if name.startswith("kn_"):
-        name = name[3:]
-    if name.endswith("_op"):
-        name = name[:-3]
-    for what in ("sum", "max"):
-        if name.startswith(f"reduce_{what}"):
-            return what
-    return name
+def _short_op(op_type: str) -> str:
+    """``kn_reduce_sum_dim1_op`` -> ``sum``, ``kn_matmul_op`` -> ``matmul``."""
+    core = op_type.removeprefix("kn_").removesuffix("_op")
+    for reduction in ("sum", "max"):
+        if core.startswith("reduce_" + reduction):
+            return reduction
+    return core
 
 
-@dataclass(eq=False)
 class SearchedGraph:
-    index: int
-    structure: list
-    symbol_map: dict | None
-    is_split: bool
-    program: Any = field(repr=False, default=None)
-    split: tuple = ()
-    invalid_split: bool = False
-    split_rejection: str | None = None
+    """One candidate structure: the op list, whether (and over which dims) it is a split form, or
+    why the requested split has none."""
+
+    __slots__ = ("index", "structure", "symbol_map", "is_split", "program", "split", "invalid_split", "split_rejection")
+
+    def __init__(self, index, structure, symbol_map=None, is_split=False, program=None, split=(), invalid_split=False,
+                 split_rejection=None):
+        self.index = index
+        self.structure = structure
+        self.symbol_map = symbol_map
+        self.is_split = bool(is_split)
+        self.program = program
+        self.split = tuple(split)
+        self.invalid_split = bool(invalid_split)
+        self.split_rejection = split_rejection
+
+    dtype = property(lambda self: program_dtype(self.program))
 
     @property
-    def dtype(self) -> str:
-        return program_dtype(self.program)
+    def ops(self) -> list:
+        return [_short_op(entry["op_type"]) for entry in self.structure if entry["op_type"] not in _IO_OPS]
 
     @property
     def kind(self) -> str:
         if self.invalid_split:
             return "invalid-split"
-        return f"split({','.join(self.split)})" if self.is_split else "solo"
-
-    @property
-    def ops(self) -> list:
-        return [_op_name(o["op_type"]) for o in self.structure if o["op_type"] not in _IO_OPS]
+        if self.is_split:
+            return "split(" + ",".join(self.split) + ")"
+        return "solo"
 
     def summary(self) -> str:
-        return f"{self.kind} " + ">".join(self.ops)
+        return self.kind + " " + ">".join(self.ops)
 
     def __repr__(self):
         return f"SearchedGraph({self.index}, {self.summary()})"
 
+    def stored(self) -> dict:
+        return {name: (list(self.split) if name == "split" else getattr(self, name)) for name in _GRAPH_FIELDS}
+
+    @classmethod
+    def restored(cls, doc: dict, program) -> "SearchedGraph":
+        return cls(doc["index"], doc["structure"], None, doc["is_split"], program, doc["split"],
+                   doc.get("invalid_split", False), doc.get("split_rejection"))
+
 
 class GraphSet(Sequence):
+    """The graphs of one program, with how they were obtained."""
+
     def __init__(self, graphs, program=None, config: SuperoptConfig | None = None, *, max_ops=None,
                  checkpoint=None, from_cache=False, seconds=0.0):
         self.graphs = list(graphs)
-        self.program, self.config, self.max_ops = program, config, max_ops
-        self.checkpoint, self.from_cache, self.seconds = checkpoint, from_cache, seconds
+        self.program = program
+        self.config = config
+        self.max_ops = max_ops
+        self.checkpoint = checkpoint
+        self.from_cache = from_cache
+        self.seconds = seconds
+
+    def __getitem__(self, position):
+        return self.graphs[position]
 
     def __len__(self):
         return len(self.graphs)
 
-    def __getitem__(self, i):
-        return self.graphs[i]
+    dtype = property(lambda self: program_dtype(self.program))
 
-    def filter(self, fn: Callable) -> "GraphSet":
-        return GraphSet([g for g in self.graphs if fn(g)], self.program, self.config, max_ops=self.max_ops,
+    def filter(self, keep) -> "GraphSet":
+        return GraphSet(filter(keep, self.graphs), self.program, self.config, max_ops=self.max_ops,
                         checkpoint=self.checkpoint, from_cache=self.from_cache, seconds=self.seconds)
 
-    @property
-    def dtype(self) -> str:
-        return program_dtype(self.program)
+    def __str__(self):
+        how = "cache hit" if self.from_cache else "searched"
+        rows = [f"GraphSet: {len(self)} graph(s) max_ops={self.max_ops} {how} {self.seconds:.2f}s"]
+        rows += [f"  {graph.index}: {graph.summary()}" for graph in self.graphs]
+        return "\n".join(rows)
 
     @classmethod
     def identity(cls, program) -> "GraphSet":
         """The un-optimised program as its only graph."""
-        return cls([SearchedGraph(0, program.to_graph_structure(), None, False, program)], program, None)
+        return cls([SearchedGraph(0, program.to_graph_structure(), program=program)], program)
 
     @classmethod
     def from_structures(cls, program, structures, symbol_map=None, split=()) -> "GraphSet":
         """Wrap structures produced elsewhere (e.g. a superoptimizer checkpoint)."""
-        graphs = []
-        for i, s in enumerate(structures):
-            has_split = any(o["op_type"].startswith("kn_split_") for o in s)
-            graphs.append(SearchedGraph(i, s, symbol_map, has_split, program, tuple(split) if has_split else ()))
-        return cls(graphs, program, None)
+        def wrapped(position, structure):
+            cut = any(entry["op_type"].startswith("kn_split_") for entry in structure)
+            return SearchedGraph(position, structure, symbol_map, cut, program, split if cut else ())
 
-    def __str__(self):
-        head = (f"GraphSet: {len(self)} graph(s) max_ops={self.max_ops} "
-                f"{'cache hit' if self.from_cache else 'searched'} {self.seconds:.2f}s")
-        return "\n".join([head] + [f"  {g.index}: {g.summary()}" for g in self])
+        return cls([wrapped(i, structure) for i, structure in enumerate(structures)], program)
 
 
 def _split_dim_of(program, lowered) -> str | None:
     """Name of the program dim the recognised family can be split over (K or the KV length)."""
     from ..frontend.tensor import Dim
 
+    problem = lowered.problem
     if lowered.family in ("matmul", "rmsnorm_matmul", "lora"):
-        node, axis = lowered.operands["A"], (-2 if lowered.problem["trans_A"] else -1)
+        role, axis = "A", (-2 if problem["trans_A"] else -1)
     elif lowered.family == "attention":
-        node, axis = lowered.operands["K"], (-1 if lowered.problem.get("k_major") else -2)    # feature-major keys: (d, keys)
+        role, axis = "K", (-1 if problem.get("k_major") else -2)      # feature-major keys: (d, keys)
     elif lowered.family == "mla":
-        node, axis = lowered.operands["KV"], -2
+        role, axis = "KV", -2
     else:
         return None                     # no partial/combine form (SwiGLU: the gate is not linear)
+    wanted = lowered.operands[role].name
     for spec in program.inputs:
-        if f"PlaceHolder_{spec.name}" == node.name:
-            d = spec.dims[axis]
-            return d.name if isinstance(d, Dim) else None
+        if "PlaceHolder_" + spec.name == wanted:
+            dim = spec.dims[axis]
+            return dim.name if isinstance(dim, Dim) else None
     return None
 
 
-def superoptimize(program, config: SuperoptConfig | None = None) -> GraphSet:
+def _proposals(program, split) -> list:
+    """The identity structure, and for a requested split the same structure marked split -- or
+    marked as having no split form, with the reason."""
     from ..lower import to_ir
 
+    structure = program.to_graph_structure()
+    graphs = [SearchedGraph(0, structure, program=program)]
+    if not split:
+        return graphs
+    try:
+        lowered = to_ir(structure, dtype=program_dtype(program), input_names=[spec.name for spec in program.inputs]).lowered
+        dim = _split_dim_of(program, lowered)
+        why = f"the {lowered.family} family splits over {dim!r}, not {list(split)}"
+    except LoweringRejected as refusal:
+        dim, why = None, str(refusal)
+    if dim is not None and dim in split:
+        graphs.append(SearchedGraph(1, structure, None, True, program, (dim,)))
+    else:
+        graphs.append(SearchedGraph(1, structure, program=program, split=split, invalid_split=True, split_rejection=why))
+    return graphs
+
+
+def _from_checkpoint(path, program):
+    """The graphs a checkpoint file holds, or None (absent, stale or partial: searched again)."""
+    if not path.exists():
+        return None
+    try:
+        return [SearchedGraph.restored(doc, program) for doc in json.loads(path.read_text())["graphs"]]
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+def superoptimize(program, config: SuperoptConfig | None = None) -> GraphSet:
     config = config or SuperoptConfig()
+    began = time.perf_counter()
     max_ops = config.resolve_max_ops(program)
-    t0 = time.perf_counter()
     program.can_split(config.split)  # SpecError on a dim no input has
-    ckpt, key = None, None
+
+    def result(graphs, path, hit):
+        return GraphSet(graphs, program, config, max_ops=max_ops, checkpoint=None if path is None else str(path),
+                        from_cache=hit, seconds=time.perf_counter() - began)
+
+    path, key = None, None
     if config.cache:
         key = cache.superopt_key(program, max_ops, config.split, config.concat_matmul)
-        ckpt = cache.checkpoint_path(key)
-        if ckpt.exists():
-            try:
-                stored = json.loads(ckpt.read_text())
-                graphs = [SearchedGraph(g["index"], g["structure"], None, g["is_split"], program, tuple(g["split"]),
-                                        g.get("invalid_split", False), g.get("split_rejection"))
-                          for g in stored["graphs"]]
-                return GraphSet(graphs, program, config, max_ops=max_ops, checkpoint=str(ckpt), from_cache=True,
-                                seconds=time.perf_counter() - t0)
-            except (OSError, ValueError, KeyError):
-                pass  # a stale or partial checkpoint is recomputed
+        path = cache.checkpoint_path(key)
+        kept = _from_checkpoint(path, program)
+        if kept is not None:
+            return result(kept, path, True)
     try:
-        structure = program.to_graph_structure()
-        graphs = [SearchedGraph(0, structure, None, False, program)]
-        if config.split:
-            try:
-                lowered = to_ir(structure, dtype=program_dtype(program),
-                                input_names=[s.name for s in program.inputs]).lowered
-                dim = _split_dim_of(program, lowered)
-            except LoweringRejected as e:
-                lowered, dim = None, None
-                reason = str(e)
-            if dim is not None and dim in config.split:
-                graphs.append(SearchedGraph(1, structure, None, True, program, (dim,)))
-            else:
-                why = (f"the {lowered.family} family splits over {dim!r}, not {list(config.split)}"
-                       if lowered is not None else reason)
-                graphs.append(SearchedGraph(1, structure, None, False, program, tuple(config.split),
-                                            invalid_split=True, split_rejection=why))
+        graphs = _proposals(program, tuple(config.split))
     except SpecError:
         raise
-    except Exception as e:  # noqa: BLE001
-        raise SuperoptError(f"graph proposal failed: {type(e).__name__}: {e}") from e
-    if ckpt is not None:
-        ckpt.write_text(json.dumps({"key": key, "graphs": [
-            {"index": g.index, "structure": g.structure, "is_split": g.is_split, "split": list(g.split),
-             "invalid_split": g.invalid_split, "split_rejection": g.split_rejection} for g in graphs]}))
-    return GraphSet(graphs, program, config, max_ops=max_ops, checkpoint=None if ckpt is None else str(ckpt),
-                    from_cache=False, seconds=time.perf_counter() - t0)
+    except Exception as problem:  # noqa: BLE001
+        raise SuperoptError(f"graph proposal failed: {type(problem).__name__}: {problem}") from problem
+    if path is not None:
+        path.write_text(json.dumps({"key": key, "graphs": [graph.stored() for graph in graphs]}))
+    return result(graphs, path, False)

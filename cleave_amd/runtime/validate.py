@@ -78,34 +78,36 @@ def benchmark_compiled_kernel(kernel, input_tensors, *, warmup_iters=0, profile_
                           rotate=rotation_sets(input_tensors))
 
 
-_REFERENCE_FILE = "reference.pt"
+class _ReferenceFile:
+    """Inputs and expected outputs of one graph as a file the children read: written once by the
+    parent (to a temporary name, then moved into place), loaded with ``weights_only`` so that
+    nothing in it is executed.  It also records how the outputs are to be compared."""
+
+    NAME = "reference.pt"
+
+    def __init__(self, folder):
+        self.folder = Path(folder)
+        self.path = self.folder / self.NAME
+
+    def write(self, inputs_by_name, reference, compare):
+        import torch
+
+        self.folder.mkdir(parents=True, exist_ok=True)
+        scratch = self.path.with_name(f"{self.NAME}.tmp.{os.getpid()}")
+        torch.save({"inputs_by_name": {name: t.cpu() for name, t in inputs_by_name.items()},
+                    "reference": [t.cpu() for t in reference], "compare": compare}, scratch)
+        os.replace(scratch, self.path)
+
+    def read(self, device="cuda") -> tuple:
+        """``(inputs by name, expected outputs, compare mode)``."""
+        import torch
+
+        held = torch.load(self.path, map_location=device, weights_only=True)
+        return dict(held["inputs_by_name"]), list(held["reference"]), held.get("compare", "plain")
 
 
 def _reference_path(cache_dir) -> Path:
-    return Path(cache_dir) / _REFERENCE_FILE
-
-
-def publish_reference(reference_cache_dir, graph, dtype, device: str = "cuda"):
-    """Build inputs + reference once in the parent and save them for the workers.
-    Returns ``(out_idx, io_bytes)``; ``io_bytes`` sizes worker parallelism."""
-    import torch
-
-    from .reference import build_inputs_and_reference
-
-    with _gpu_exec_guard():
-        inputs_by_name, reference, out_idx = build_inputs_and_reference(graph, dtype, device)
-        path = _reference_path(reference_cache_dir)
-        os.makedirs(reference_cache_dir, exist_ok=True)
-        tmp = path.with_name(f"{path.name}.tmp.{os.getpid()}")
-        torch.save({"inputs_by_name": {k: v.cpu() for k, v in inputs_by_name.items()},
-                    "reference": [r.cpu() for r in reference], "compare": compare_mode(graph)}, tmp)
-        os.replace(tmp, path)
-        io_bytes = _live_bytes(inputs_by_name.values()) + _live_bytes(reference)
-        del inputs_by_name, reference
-        if torch.cuda.is_available():
-            torch.cuda.synchronize()
-            torch.cuda.empty_cache()
-    return out_idx, io_bytes
+    return _ReferenceFile(cache_dir).path
 
 
 def compare_mode(graph) -> str:
@@ -120,6 +122,30 @@ def compare_mode(graph) -> str:
     return "plain"
 
 
+def publish_reference(reference_cache_dir, graph, dtype, device: str = "cuda"):
+    """The parent's side: inputs and reference of ``graph`` built once and left in
+    ``reference_cache_dir`` for the children.  Returns ``(out_idx, io_bytes)``; ``io_bytes`` (what
+    one child will hold on the device) sizes how many children may run at once."""
+    import torch
+
+    from .reference import build_inputs_and_reference
+
+    with _gpu_exec_guard():
+        inputs_by_name, reference, out_idx = build_inputs_and_reference(graph, dtype, device)
+        io_bytes = _live_bytes(inputs_by_name.values()) + _live_bytes(reference)
+        _ReferenceFile(reference_cache_dir).write(inputs_by_name, reference, compare_mode(graph))
+        del inputs_by_name, reference
+        if torch.cuda.is_available():
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+    return out_idx, io_bytes
+
+
+def _load_reference(reference_cache_dir, device: str = "cuda", with_mode: bool = False):
+    inputs_by_name, reference, mode = _ReferenceFile(reference_cache_dir).read(device)
+    return (inputs_by_name, reference, mode) if with_mode else (inputs_by_name, reference)
+
+
 def _comparable(outputs, mode):
     if mode != "softmax_partial":
         return list(outputs)
@@ -130,18 +156,6 @@ def _comparable(outputs, mode):
     return [lse, po / pl.clamp_min(1e-30).unsqueeze(-1)]
 
 
-def _load_reference(reference_cache_dir, device: str = "cuda", with_mode: bool = False):
-    import torch
-
-    payload = torch.load(_reference_path(reference_cache_dir), map_location=device, weights_only=True)
-    loaded = dict(payload["inputs_by_name"]), list(payload["reference"])
-    return (*loaded, payload.get("compare", "plain")) if with_mode else loaded
-
-
-def _as_list(x):
-    return list(x) if isinstance(x, (tuple, list)) else [x]
-
-
 def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance = DEFAULT_TOLERANCE,
                              compare: str = "plain"):
     """Run ``kernel(*inputs)`` and assert every output is within ``tolerance`` of ``reference``."""
@@ -149,40 +163,42 @@ def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance 
 
     from .reference import reconcile_output_layout
 
-    actual = _as_list(kernel(*inputs))
+    produced = kernel(*inputs)
+    produced = list(produced) if isinstance(produced, (tuple, list)) else [produced]
     torch.cuda.synchronize()
-    assert len(actual) == len(reference), (
-        f"Kernel returned {len(actual)} outputs but the reference has {len(reference)}.")
-    reference = [reconcile_output_layout(want, got.shape).to(got.device) for got, want in zip(actual, reference)]
-    actual, reference = _comparable(actual, compare), _comparable(reference, compare)
-    for got, want in zip(actual, reference):
+    if len(produced) != len(reference):
+        raise AssertionError(f"Kernel returned {len(produced)} outputs but the reference has {len(reference)}.")
+    expected = [reconcile_output_layout(want, got.shape).to(got.device) for got, want in zip(produced, reference)]
+    for got, want in zip(_comparable(produced, compare), _comparable(expected, compare)):
         torch.testing.assert_close(got.float(), want.float().to(got.device), rtol=tolerance.rtol,
                                    atol=tolerance.atol, equal_nan=tolerance.equal_nan)
 
 
 def _check_kernel(kernel, *, graph=None, dtype=None, reference_cache_dir=None,
                   tolerance: Tolerance = DEFAULT_TOLERANCE, benchmark: BenchOptions | None = None):
-    """Validate against the published (or freshly built) reference, then optionally time, all
-    under one hold of the GPU lock.  Returns mean latency in ms, or None without ``benchmark``."""
-    from .reference import build_inputs_and_reference, order_inputs_for_kernel
+    """A child's side: validate against the published reference (or one built here from
+    ``graph`` and ``dtype``), then optionally time, all under one hold of the GPU lock.  Mean
+    latency in ms, or None without ``benchmark``."""
+    from . import reference as ref
 
     with _gpu_exec_guard():
         with _stage("validate"):
-            if reference_cache_dir is not None:
-                inputs_by_name, reference, mode = _load_reference(reference_cache_dir, with_mode=True)
-            else:
-                inputs_by_name, reference, _ = build_inputs_and_reference(graph, dtype)
+            if reference_cache_dir is None:
+                inputs_by_name, expected, _ = ref.build_inputs_and_reference(graph, dtype)
                 mode = compare_mode(graph)
-            inputs = order_inputs_for_kernel(inputs_by_name, kernel)
-            _validate_kernel_outputs(kernel, inputs, reference, tolerance=tolerance, compare=mode)
-        if benchmark is None:
-            return None
-        with _stage("bench"):
-            return benchmark_compiled_kernel(kernel, inputs, warmup_iters=benchmark.warmup,
-                                             profile_iters=benchmark.iters)
+            else:
+                inputs_by_name, expected, mode = _ReferenceFile(reference_cache_dir).read()
+            ordered = ref.order_inputs_for_kernel(inputs_by_name, kernel)
+            _validate_kernel_outputs(kernel, ordered, expected, tolerance=tolerance, compare=mode)
+        if benchmark is not None:
+            with _stage("bench"):
+                return benchmark_compiled_kernel(kernel, ordered, warmup_iters=benchmark.warmup,
+                                                 profile_iters=benchmark.iters)
+    return None
 
 
-def _run_and_validate_kernel(kernel, *, graph=None, dtype=None, reference_cache_dir=None,
-                             tolerance: Tolerance = DEFAULT_TOLERANCE):
-    _check_kernel(kernel, graph=graph, dtype=dtype, reference_cache_dir=reference_cache_dir, tolerance=tolerance)
+def _run_and_validate_kernel(kernel, **where):
+    """``_check_kernel`` without timing; the kernel's source comes back."""
+    where.pop("benchmark", None)
+    _check_kernel(kernel, **where)
     return kernel.get_kernel_source()
