@@ -18,16 +18,35 @@ SPLIT_KINDS = (PAGED_DECODE, PAGED_DECODE_SLAB, MLA_PAGED_DECODE)
 # Layers this back end has a HIP template for (all of them).
 BUILT_KINDS = KINDS + MLA_KINDS
 
-OPTIONAL_FIELDS = ("batch_dim", "tokens_dim", "kv_tokens_dim", "pages_dim", "index_dim", "index_input",
-                   "last_page_len_input", "query_indptr_input", "grid_order")
-FIELDS_READ = {
-    PAGED_DECODE: {"batch_dim", "pages_dim", "index_dim", "index_input", "grid_order"},
-    PAGED_DECODE_SLAB: {"batch_dim", "pages_dim", "index_dim", "index_input", "grid_order", "last_page_len_input"},
-    PAGED_PREFILL_CAUSAL: {"tokens_dim", "pages_dim", "index_dim", "index_input", "query_indptr_input"},
-    RAGGED_PREFILL_CAUSAL: {"tokens_dim", "kv_tokens_dim", "query_indptr_input"},
+# Spec fields only some layers read, each with its readers.  A spec that sets a field its layer
+# does not read is refused (the field would silently do nothing); fields not listed here are
+# read by every layer.
+_READERS = {
+    "batch_dim": (PAGED_DECODE, PAGED_DECODE_SLAB),
+    "tokens_dim": CAUSAL_KINDS,
+    "kv_tokens_dim": (RAGGED_PREFILL_CAUSAL,),
+    "pages_dim": PAGED_KINDS,
+    "index_dim": PAGED_KINDS,
+    "index_input": PAGED_KINDS,
+    "last_page_len_input": SLAB_KINDS,
+    "query_indptr_input": CAUSAL_KINDS,
+    "grid_order": (PAGED_DECODE, PAGED_DECODE_SLAB),
 }
-MLA_OPTIONAL_FIELDS = ("batch_dim", "tokens_dim", "query_indptr_input")
-MLA_FIELDS_READ = {MLA_PAGED_DECODE: {"batch_dim"}, MLA_PAGED_PREFILL_CAUSAL: {"tokens_dim", "query_indptr_input"}}
+_MLA_READERS = {
+    "batch_dim": (MLA_PAGED_DECODE,),
+    "tokens_dim": (MLA_PAGED_PREFILL_CAUSAL,),
+    "query_indptr_input": (MLA_PAGED_PREFILL_CAUSAL,),
+}
+
+
+def _by_layer(readers: dict, layers) -> dict:
+    return {layer: {name for name, who in readers.items() if layer in who} for layer in layers}
+
+
+OPTIONAL_FIELDS = tuple(_READERS)
+FIELDS_READ = _by_layer(_READERS, KINDS)
+MLA_OPTIONAL_FIELDS = tuple(_MLA_READERS)
+MLA_FIELDS_READ = _by_layer(_MLA_READERS, MLA_KINDS)
 
 # Partial tensors of a split-KV pair.  The reference hands over (ROWSUM, VALUE) because it
 # subtracts no maximum; the exact online softmax here also carries the running maximum.

@@ -1,1 +1,1 @@
-"""Compile, validate and time generated kernels."""
+"""What happens to a generated kernel: hiprtc, a check against the reference, a timing; the ctypes binding of the native library."""
