@@ -86,7 +86,7 @@ CL_DEVICE void sk_load(const elem_t* __restrict__ W, const elem_t* __restrict__ 
 // 0, 2, 3, 4) and the 100 MHz wall clock (1, 5) and leaves them in the first bytes of X
 #define SK_MARK(k) do { const unsigned long long t_ = (k) == 1 || (k) == 5 ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); \
     __builtin_amdgcn_sched_barrier(0); sk_stamps[k] = t_; } while (0)
-#define SK_DUMP() do { SK_MARK(4); SK_MARK(5); if (lane == 0) { \
+#define SK_DUMP() do { SK_MARK(4); SK_MARK(5); sk_stamps[6] = __builtin_amdgcn_s_getreg(63492); sk_stamps[7] = __builtin_amdgcn_s_getreg(63508); if (lane == 0) { \
     unsigned long long* dump_ = (unsigned long long*)CL_ARG_X + ((blockIdx.y * gridDim.x + blockIdx.x) * (SK_THREADS / 64) + wave) * 8; \
     _Pragma("unroll") for (int k_ = 0; k_ < 8; ++k_) dump_[k_] = sk_stamps[k_]; } } while (0)
 #else
