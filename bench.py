@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the compile path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops c1,c2,c3,c4,c5,mm[,dyn,copy]] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops c2,c1,c3,c4,c5,mm,...,dyn[,copy]] [--no-cpu]
 
 For every operator the staged pipeline searches candidates (``cleave_amd.compile``, preset
 fast): each candidate is compiled with hiprtc, validated against the torch evaluation of the
@@ -13,7 +13,9 @@ last-level cache cannot be served from it.
 
 One JSON line is printed.  ``value`` is the best-candidate latency in microseconds of the
 headline workload (fused RMSNorm->matmul at the decode shape M=16, K=4096, N=11008, fp16);
-``ops`` carries the same figures for every other operator.  ``roofline`` prices the dominant
+``ops`` carries the same figures for every other operator (the first one named is the headline
+and fails the run if it fails; any other that fails is listed with its error), the registry's
+paged operators last (``dyn``: geomean over their captured workloads).  ``roofline`` prices the dominant
 kernel of the headline workload: algorithmic bytes per launch over its mean duration from
 HIP events on the launch stream, against the published 8 TB/s.  ``cpu_baseline`` is the numpy
 port of the reference's CPU evaluation of the same program, timed on this host.
@@ -561,7 +563,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,rmsmm,lora,mmrs,mm2d,rsdiv,attn,qknorm,mlapf")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,rmsmm,lora,mmrs,mm2d,rsdiv,attn,qknorm,mlapf,dyn")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")
@@ -590,17 +592,14 @@ def main():
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     threads = int(os.environ.get("OMP_NUM_THREADS", cores))
     results = {}
-    for name in wanted:
+    def measure(name):
         if name == "copy":
-            results[name] = run_copy(max(10, args.steps // 4), max(2, args.warmup // 4))
-            continue
+            return run_copy(max(10, args.steps // 4), max(2, args.warmup // 4))
         if name == "dyn":
-            results[name] = {"op": "dyn", "workload": "registry operators (paged GQA / MLA decode, causal prefill) over their captured axes",
-                             "operators": run_dynamic([n for n in args.dyn_ops.split(",") if n] or None)}
-            continue
+            return {"op": "dyn", "workload": "registry operators (paged GQA / MLA decode, causal prefill) over their captured axes",
+                    "operators": run_dynamic([n for n in args.dyn_ops.split(",") if n] or None)}
         if name == "c5":
-            results[name] = run_paged(max(10, args.steps // 4), max(2, args.warmup // 4), not args.no_cpu, args.kernels)
-            continue
+            return run_paged(max(10, args.steps // 4), max(2, args.warmup // 4), not args.no_cpu, args.kernels)
         heavy = ops[name]["bound"] == "mfma" and ops[name]["flops"] > 1e11
         steps = max(50, args.steps // 4) if heavy else args.steps
         res, program = run_dense(name, ops[name], steps, args.warmup, args.search_iters, args.kernels,
@@ -609,8 +608,20 @@ def main():
             cpu_us, runs = cpu_dense(program, ops[name], budget_s=8.0 if name != "c4" else 15.0)
             res["cpu_us"] = round(cpu_us, 1)
             res["cpu_sample"] = f"full workload, median of {runs} runs"
-        results[name] = res
         log(f"[{name}] {res['best_us']} us  hbm {res['hbm']['frac']:.3f}  mfma {res['mfma']['frac']:.3f}")
+        return res
+
+    for name in wanted:
+        # the headline workload fails the run; any other operator that fails is reported as failed
+        # beside the ones that were measured
+        if name == wanted[0]:
+            results[name] = measure(name)
+            continue
+        try:
+            results[name] = measure(name)
+        except Exception as failure:  # noqa: BLE001 - reported in the line, not swallowed
+            log(f"[{name}] FAILED: {type(failure).__name__}: {str(failure)[:300]}")
+            results[name] = {"op": name, "error": f"{type(failure).__name__}: {str(failure)[:300]}"}
     # the headline workload unless left out; failing that the first operator that has a latency
     timed = [n for n in wanted if "best_us" in results[n]]
     if not timed:
