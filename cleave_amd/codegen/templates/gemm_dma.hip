@@ -48,7 +48,7 @@
 #define CL_SPREAD_LOADS 0
 #endif
 #ifndef CL_ASM_LOADS
-#define CL_ASM_LOADS 0
+#define CL_ASM_LOADS 1
 #endif
 #ifndef CL_SWIGLU
 #define CL_SWIGLU 0
@@ -147,15 +147,24 @@ struct GdOperand {
     const int u = wave + i * GD_WAVES;
     if (UNITS % GD_WAVES == 0 || u < UNITS) {
 #if CL_ASM_LOADS
-      // Written as assembly the load is not counted by the compiler: with the builtin in a loop
-      // its bookkeeping of LDS traffic degrades to "wait for every LDS read" (lgkmcnt(0)) before
-      // each matrix op that takes a fragment.  The kernel's own vmcnt(0) at the end of a step
-      // covers these loads.  (Measured: no faster on the large matmul, so the builtin, whose
-      // waits the compiler derives itself, stays the default.)
+      // Written as assembly (the default): the tile's first element of the step stays in scalar
+      // registers and the lane's 32-bit offset goes in as it is, where the builtin forms a 64-bit
+      // address per load in vector registers (two registers and an add each; with the row sums of
+      // squares of the fused norm beside a 128-register accumulator tile that is what made the
+      // compiler spill the offsets and reload them between the loads, each reload waiting for the
+      // loads before it).  The load is then not counted by the compiler; the kernel's own
+      // vmcnt(0) at the end of a step covers it.  On the large matmul the two forms measure alike.
       const unsigned lds_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)(lds + u * 512);
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                   :: "v"(reinterpret_cast<const char*>(base) + goff[i]), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
-                   : "memory", "m0");
+      if constexpr (sizeof(off_t) == 4) {
+        // (scalar base + 32-bit lane offset: no 64-bit address is formed in vector registers)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(goff[i]), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
+                     : "memory", "m0");
+      } else {
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :: "v"(reinterpret_cast<const char*>(base) + goff[i]), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
+                     : "memory", "m0");
+      }
 #else
       __builtin_amdgcn_global_load_lds((gd_gbl_void*)(reinterpret_cast<const char*>(base) + goff[i]),
                                        (gd_lds_void*)(lds + u * 512), 16, 0, 0);

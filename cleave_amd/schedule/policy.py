@@ -135,8 +135,8 @@ def gemm_dma_candidates(low, role, factor, arch: Arch):
         tm, tn = bm // wm // 16, bn // wn // 16
         if tm & (tm - 1) or tn & (tn - 1) or tm * tn * 4 > 128:
             continue
-        if post_norm and tm * tn * 4 > 64:
-            continue      # the row sums of squares need registers a 128-register accumulator tile does not leave (spills)
+        if post_norm and low.dtype == "bfloat16" and tm * tn * 4 > 64 and wm > wn:
+            continue      # bf16 squares go through float conversions: beside a 128-register, 4-row-fragment tile they spill
         # every wave must own whole 1 KiB load units of both tiles or none
         units_a, units_b = bm // 8, bn // 8
         vgprs = tm * tn * 4 + (tm + tn) * 6 + -(-units_a // (wm * wn)) + -(-units_b // (wm * wn)) + 24
