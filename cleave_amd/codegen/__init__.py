@@ -610,6 +610,10 @@ class HipCodeGen:
             if not 1 <= int(t["S_AHEAD"]) <= (p["ckv"] + p["kpe"]) // 32:
                 raise CodegenError("S_AHEAD: between 1 and the key fragments of a step")
             unit.define("CL_S_AHEAD", int(t["S_AHEAD"]))
+        if "S_PANELS" in t:
+            if not 0 <= int(t["S_PANELS"]) < (p["ckv"] + p["kpe"]) // 64:
+                raise CodegenError("S_PANELS: the score waves can load between none and all but one of a step's 64-feature panels")
+            unit.define("CL_S_PANELS", int(t["S_PANELS"]))
         for k in t:
             if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
                 unit.define(f"CL_{k}", 1)

@@ -83,6 +83,11 @@
 #ifndef CL_S_AHEAD
 #define CL_S_AHEAD CL_LDS_AHEAD                 // key fragments a score wave asks for ahead of its matrix ops
 #endif
+#ifndef CL_S_PANELS
+#define CL_S_PANELS 0                           // panels of every image (from the third on) the score waves ask for
+#endif
+#define MD_V_UNITS (MD_PANELS - CL_S_PANELS)    // loads per value wave and step once the score waves share them
+static_assert(CL_S_PANELS >= 0 && CL_S_PANELS < MD_PANELS, "the value waves keep at least one panel");
 static_assert(CL_CKV % 128 == 0 && CL_KPE % 64 == 0, "whole 64-feature panels, the latent ones halved between two value waves");
 static_assert(CL_HEADS % MD_HEADS_PER_BLOCK == 0, "64 heads per workgroup");
 static_assert(CL_SCALE_LOG2E > 0.f, "the largest raw score must be the largest scaled one");
@@ -251,6 +256,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       md_dma16<0>(src, tiles_byte + (unsigned)(2 * MD_TILE * 2 + 1024 * k));
     }
   }
+  // this wave's piece of every panel it loads: token rows 8 loader + lane / 8, the chunk that belongs in slot lane % 8
+  u32 lat_off, pe_off;
+  {
+    const int r = 8 * loader + (lane >> 3);
+    const int chunk = (lane & 7) ^ md_swz(r);
+    lat_off = (u32)((r * CL_CKV + 8 * chunk) * 2);
+    pe_off = (u32)((r * CL_KPE + 8 * chunk) * 2);
+  }
   if (scores) {
     // =========================================================================== score wave
     // Q fragments (B operand): lane (c, g) holds q[head 16 t + c][32 j + 8 g .. + 8] for head tile t
@@ -280,6 +293,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
     MD_MARK(2);
     for (int it = 0; it <= n_own; ++it) {
+#if CL_S_PANELS
+      // this wave's panels of image `it` have landed: at most those of image it + 1 are on their way
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (CL_S_PANELS & 15));
+#endif
       md_barrier();                                 // image `it` has landed (the value waves waited for it)
       MD_MARK(3 + 2 * it);
       if (it == n_own) break;
@@ -300,11 +317,28 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       f32x4 sp[2][2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) sp[t][0] = sp[t][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#if CL_S_PANELS
+      // this wave's share of the loads of image it + 2, from the second iteration on (the value
+      // waves ask for images 0 to 2 whole); past the split's end as in the value waves
+      const int ahead = it + 2 < n_own + 1 ? it + 2 : n_own + 1;
+      const int rel = ahead < n_own - 1 ? ahead : n_own - 1;
+      const int t0_ahead = (step_begin + rel) * MD_STEP;
+      const elem_t* lat_rows = kv + (i64)t0_ahead * CL_CKV;
+      const elem_t* pe_rows = kpe + (i64)t0_ahead * CL_KPE;
+      const unsigned stage_byte = tiles_byte + (unsigned)((ahead % MD_STAGES) * MD_TILE * 2);
+#endif
 #pragma unroll
       for (int j = 0; j < MD_KJ; ++j) {
         const elem8 a = *reinterpret_cast<const elem8*>(tile + (j >> 1) * MD_PANEL + (a_lo ^ ((4 * (j & 1)) << 3)));
 #pragma unroll
         for (int t = 0; t < 2; ++t) sp[t][j & 1] = mfma16(a, qf[t][j], sp[t][j & 1]);
+#if CL_S_PANELS && !defined(CL_DBG_NODMA)
+        if (it > 0) {
+#pragma unroll
+          for (int pn = 0; pn < CL_S_PANELS; ++pn)
+            if ((pn * MD_KJ) / CL_S_PANELS == j) md_issue_panel(pn, lat_off, pe_off, lat_rows, pe_rows, t0_ahead, stage_byte, loader);
+        }
+#endif
       }
       __builtin_amdgcn_sched_group_barrier(0x100, CL_S_AHEAD, 0);
 #pragma unroll
@@ -362,19 +396,15 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     MD_MARK(45);
     MD_MARK_WALL(46);
     MD_DUMP();
+#if CL_S_PANELS
+    __builtin_amdgcn_s_waitcnt(0x0F70);             // no load may still be on its way into LDS when the workgroup ends
+#endif
     return;
   }
 
   // ============================================================================= value wave
   // loads of step index s (relative to the split), clamped onto the split's last step so that the
   // load counter holds the same number of steps at every wait
-  u32 lat_off, pe_off;
-  {
-    const int r = 8 * loader + (lane >> 3);
-    const int chunk = (lane & 7) ^ md_swz(r);
-    lat_off = (u32)((r * CL_CKV + 8 * chunk) * 2);
-    pe_off = (u32)((r * CL_KPE + 8 * chunk) * 2);
-  }
   auto issue = [&](int s) __attribute__((always_inline)) {
 #ifdef CL_DBG_NODMA
     return;
@@ -422,7 +452,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   for (int it = 0; it <= n_own; ++it) {
     // image `it` must have landed before the barrier lets the score waves read it: at most the
     // loads of image it + 1 may be outstanding (none are issued for an empty split)
-    if (n_own > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (MD_UNITS_PER & 15) | ((MD_UNITS_PER >> 4) << 14));
+    // (with the score waves sharing the loads the later images are MD_V_UNITS loads each: waiting
+    // down to that count is the right wait for them and a longer one for the first three)
+    if (n_own > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (MD_V_UNITS & 15) | ((MD_V_UNITS >> 4) << 14));
     md_barrier();
     MD_MARK(3 + 2 * it);
     const elem_t* next_tile = md_tiles + (it % MD_STAGES) * MD_TILE;           // image `it`: there from here on
@@ -490,8 +522,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         operand(next_tile, fb + MD_PRE - MD_FBW, pre_lo[fb % MD_PRE], pre_hi[fb % MD_PRE]);
 #ifndef CL_DBG_NODMA
 #pragma unroll
-      for (int pn = 0; pn < MD_PANELS; ++pn)
-        if ((pn * MD_FBW) / MD_PANELS == fb) md_issue_panel(pn, lat_off, pe_off, lat_rows, pe_rows, t0, stage_byte, loader);
+      for (int pn = CL_S_PANELS; pn < MD_PANELS; ++pn)
+        if (((pn - CL_S_PANELS) * MD_FBW) / MD_V_UNITS == fb) md_issue_panel(pn, lat_off, pe_off, lat_rows, pe_rows, t0, stage_byte, loader);
 #endif
     }
 #pragma unroll

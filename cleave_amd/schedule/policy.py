@@ -465,7 +465,12 @@ def mla_candidates(low, role, factor, arch: Arch):
     duo_lds = mla_lds_bytes(p["ckv"], p["kpe"], 4) + 9 * 1024
     if out and p["heads"] % 64 == 0 and p["ckv"] % 128 == 0 and duo_lds <= arch.lds_bytes:
         best = min(c.score for c in out)
-        for tiling, rel in ((dict(DUO=1), 0.75), (dict(DUO=1, LDS_AHEAD=4), 0.76)):
+        # (third: the score waves ask for about half of every image's panels -- a wave that waits for the
+        # path into the compute unit does not hold up the other wave of its SIMD, and the value
+        # waves are the longer chain of a step; measured 1-2 % ahead)
+        shared = max(1, (p["ckv"] + p["kpe"]) // 64 // 2)
+        for tiling, rel in ((dict(DUO=1), 0.75), (dict(DUO=1, LDS_AHEAD=4), 0.76),
+                            (dict(DUO=1, LDS_AHEAD=4, S_PANELS=shared), 0.755)):
             out.append(TileDict("mla_decode", role, tiling, output_tile=[64, p["ckv"]], rstep_map={"kv": 32},
                                 n_threads=512, split_factor=factor, score=rel * best, lds_bytes=duo_lds, est_vgprs=208))
     return out

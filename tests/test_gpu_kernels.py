@@ -308,6 +308,19 @@ def test_mla_decode_paired_waves_small(split):
         _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(DUO=1), split=split)
 
 
+@pytest.mark.parametrize("split", [None, 2, 3, 8])
+def test_mla_decode_paired_waves_with_shared_loading(split):
+    """The same cases with the score waves asking for part of every image's panels (from the
+    third image on): one, about half, and all but one of them; one to twelve steps per split, so
+    that splits end before, at and after the first shared image."""
+    fn, dt, mk = C.CASES["c4"]
+    for shapes, panels in ((dict(B=2, H=64, D=512, PE=64, SKV=192), 4), (dict(B=1, H=128, D=512, PE=64, SKV=120), 1),
+                           (dict(B=3, H=64, D=512, PE=64, SKV=48), 8), (dict(B=1, H=64, D=256, PE=64, SKV=456), 2),
+                           (dict(B=1, H=64, D=512, PE=64, SKV=384), 4)):
+        _check(fn.trace(dt, **shapes), mk, shapes, template="mla_decode", tiling=dict(DUO=1, LDS_AHEAD=4, S_PANELS=panels),
+               split=split)
+
+
 def test_mla_decode_paired_waves_rising_maximum():
     """Scores that keep growing along the KV axis: the score waves raise their reference points
     several times per split, each token half on its own, and the value waves must rescale
@@ -320,9 +333,9 @@ def test_mla_decode_paired_waves_rising_maximum():
     kv = (kv.float() * 0.2 + ramp * torch.sign(q.float().mean(dim=(1,), keepdim=True))).to(kv.dtype)
     ins = [q, kv, q_pe, k_pe]
     want = po.evaluate(prog, ins)[0]
-    for split in (None, 2, 4):
-        kernel = kernel_for(prog, template="mla_decode", tiling=dict(DUO=1), split=split)
-        print(f"case mla paired waves rising maximum split={split}", flush=True)
+    for split, tiling in ((None, dict(DUO=1)), (2, dict(DUO=1)), (4, dict(DUO=1)), (2, dict(DUO=1, LDS_AHEAD=4, S_PANELS=4))):
+        kernel = kernel_for(prog, template="mla_decode", tiling=tiling, split=split)
+        print(f"case mla paired waves rising maximum split={split} {tiling}", flush=True)
         got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
         np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
 
@@ -337,9 +350,10 @@ def test_mla_decode_paired_waves_read_ahead_depths():
 
 
 @pytest.mark.parametrize("split", [4, 8, 16])
-def test_mla_decode_paired_waves_c4_full(split):
+@pytest.mark.parametrize("tiling", [dict(DUO=1), dict(DUO=1, LDS_AHEAD=4, S_PANELS=4)], ids=["value-waves-load", "shared-loading"])
+def test_mla_decode_paired_waves_c4_full(tiling, split):
     fn, dt, mk = C.CASES["c4"]
-    _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=dict(DUO=1), split=split)
+    _check(fn.trace(dt, **C.FULL["c4"]), mk, C.FULL["c4"], template="mla_decode", tiling=tiling, split=split)
 
 
 def test_graph_replay_timer_matches_eager_results_and_time():

@@ -295,6 +295,8 @@ def test_codegen_refuses_impossible_plans():
     mla = stage_graph(C.mla_decode.trace(cl.bf16, B=2, H=64, D=512, PE=64, SKV=256))
     with pytest.raises(CodegenError, match="LDS_AHEAD"):
         HipCodeGen().gen(apply_tiling(TileDict("mla_decode", "main", dict(DUO=1, LDS_AHEAD=12), flat_graph=mla)))
+    with pytest.raises(CodegenError):      # the value waves keep at least one of the nine panels
+        HipCodeGen().gen(apply_tiling(TileDict("mla_decode", "main", dict(DUO=1, S_PANELS=9), flat_graph=mla)))
     m = parse_manifest(HipCodeGen().gen(apply_tiling(TileDict("mla_decode", "main", dict(DUO=1, LDS_AHEAD=4), flat_graph=mla))))
     assert m["launches"][0]["block"] == [512, 1, 1] and m["launches"][0]["grid"][0] == "2"
     with pytest.raises(CodegenError, match="manifest"):
