@@ -154,6 +154,23 @@ CL_DEVICE float pl_max_over_groups(float x) {
   return a;
 }
 
+// the largest of three (one instruction, and none of the canonicalising copies fmaxf brings along)
+CL_DEVICE float pl_max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// Row sums of the weights on the matrix unit (a product with a fragment of ones beside the value
+// products: the sum of exactly the rounded weights the values are multiplied by) instead of one
+// vector add per weight -- where the vector unit is the busier one, i.e. 64-wide heads (measured
+// on dense attention over 4096 keys: 151 against 158 us at 64 / 64, 256 against 253 at 128 / 128, 1673
+// against 1527 at 192 / 128).  Not where the log-sum-exp is an output: that is held to 1e-3, which the
+// rounding of a handful of 16-bit weights would show, so there the unrounded weights are added up.
+#ifndef CL_PF_MSUMS
+#define CL_PF_MSUMS (CL_HEAD_DIM <= 64 && CL_VDIM <= 64)
+#endif
+#define PL_MATRIX_SUMS (CL_PF_MSUMS && !CL_EMIT_LSE && !CL_LINEAR)
+
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(256, 2)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
@@ -400,6 +417,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 
   float m_run[2] = {CL_NEG_BIG, CL_NEG_BIG};   // running max of the scaled scores (log2 domain), uniform over g
   float l_run[2] = {0.f, 0.f};                 // this lane's share of the sum of the weights
+#if PL_MATRIX_SUMS
+  f32x4 l_acc[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};   // every component: the sum of row c's weights
+  elem8 ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = to_elem(1.0f);
+#endif
   f32x4 acc[2][PL_FB];                         // acc[rt][fb][r] = O[row][16 fb + 4 g + r]
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt)
@@ -576,13 +599,15 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[j][h], qf[rt][j], sn[rt][h]);
 #if !CL_LINEAR
+    // (the lane's own eight scores of each row; a row's four lane groups are compared only when
+    // some lane passes its row's reference: no row does unless one of its lanes does)
     float mx[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-      float v = fmaxf(fmaxf(s[rt][0], s[rt][1]), s[rt][2]);
-      v = fmaxf(fmaxf(v, s[rt][3]), s[rt][4]);
-      v = fmaxf(fmaxf(v, s[rt][5]), s[rt][6]);
-      mx[rt] = pl_max_over_groups(fmaxf(v, s[rt][7])) * scale2;
+      float v = pl_max3(s[rt][0], s[rt][1], s[rt][2]);
+      v = pl_max3(v, s[rt][3], s[rt][4]);
+      v = pl_max3(v, s[rt][5], s[rt][6]);
+      mx[rt] = pl_max3(v, s[rt][7], s[rt][7]) * scale2;
     }
 #pragma unroll
     for (int i = 0; i < 2 * PL_KJ; ++i) {
@@ -594,10 +619,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       // lags the running maximum by less than 8 (log2 domain)
 #pragma unroll
       for (int rt = 0; rt < 2; ++rt) {
+        mx[rt] = pl_max_over_groups(mx[rt]);
         const float m_new = mx[rt] > m_run[rt] + 8.0f ? mx[rt] : m_run[rt];
         const float alpha = fast_exp2(m_run[rt] - m_new);
         m_run[rt] = m_new;
         l_run[rt] *= alpha;
+#if PL_MATRIX_SUMS
+        l_acc[rt] *= alpha;
+#endif
 #pragma unroll
         for (int fb = 0; fb < PL_FB; ++fb) acc[rt][fb] *= alpha;
       }
@@ -617,7 +646,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #else
         const float p = fast_exp2(__builtin_fmaf(s[rt][i], scale2, -m_run[rt]));
 #endif
+#if !PL_MATRIX_SUMS
         psum += p;
+#endif
         pf[rt][i] = to_elem(p);
       }
       l_run[rt] += psum;
@@ -640,6 +671,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // ---- weights of the second row tile beside the value product of the first ----------------
 #pragma unroll
     for (int fb = 0; fb < PL_FB; ++fb) acc[0][fb] = mfma16(vf[fb], pf[0], acc[0][fb]);
+#if PL_MATRIX_SUMS
+    l_acc[0] = mfma16(ones, pf[0], l_acc[0]);
+#endif
     weigh(1);
 #pragma unroll
     for (int i = 0; i < PL_FB; ++i) {
@@ -652,6 +686,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // ---- value product of the second row tile ------------------------------------------------
 #pragma unroll
     for (int fb = 0; fb < PL_FB; ++fb) acc[1][fb] = mfma16(vf[fb], pf[1], acc[1][fb]);
+#if PL_MATRIX_SUMS
+    l_acc[1] = mfma16(ones, pf[1], l_acc[1]);
+#endif
 #if CL_KNORM
     // (and the sums of squares of the keys of step + 1, whose factors go onto its scores)
     f32x4 gram[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};
@@ -692,9 +729,13 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int c_e = lane_e & 15, g_e = lane_e >> 4;
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
+#if PL_MATRIX_SUMS
+    const float l = l_acc[rt][0];
+#else
     float l = l_run[rt];
     l += lane_xor(l, lane_e, 16);
     l += lane_xor(l, lane_e, 32);
+#endif
     const int m = 32 * wave + 16 * rt + c_e;
     if (m >= n_rows) continue;
 #if CL_PF_DBG_NOSTORE
