@@ -366,7 +366,8 @@ class HipCodeGen:
         unit.define("CL_TOTAL_ROWS", total_rows)
         unit.define("CL_EMIT_LSE", emit_lse)
         names = self._by_name(params)
-        ins = [q for q in params if q.role in ("input", "scalar")]
+        # (a `Scratch_*` parameter is written by a launch of this unit ahead of the attention kernel, which reads it)
+        ins = [q for q in params if q.role in ("input", "scalar") or q.name.startswith("Scratch_")]
         outs = [q for q in params if q.role == "output"]
         derived = tuple(name for name, _ in plan.extra.get("derived_dims", ()))
         dyn = tuple(plan.dyn_dims) + derived
@@ -470,26 +471,45 @@ class HipCodeGen:
             raise CodegenError("the split form of the many-row attention kernel has no lse output")
         if d % 64 or d > 256 or p["vdim"] % 64 or p["vdim"] > 256:
             raise CodegenError("the many-row attention kernel needs key and value widths in whole 64-feature panels (<= 256)")
+        norm = p.get("norm_eps") or {}
+        # KPRE: the keys of a QK-norm attention are normalised once by a launch of their own into a
+        # scratch copy, which the attention kernel then reads as plain keys
+        kpre = bool(plan.tiling.get("KPRE"))
+        if kpre:
+            if "k" not in norm or not partial or p.get("k_major") or d not in (64, 128, 256):
+                raise CodegenError("KPRE normalises row-major keys of a QK-norm attention, 64, 128 or 256 wide, ahead of the kernel that reads them")
+            key = self._by_name(params)[op["K"]]
+            at = next(i for i, q in enumerate(params) if q.role in ("scratch", "output"))
+            params.insert(at, ParamSpec("Scratch_kn", key.dtype, key.shape, "scratch"))
         self._attn_common(unit, plan, params, partial, combine, False, p["vdim"], p["units"] * rows, False)
         for k, v in (("CL_DENSE", 1), ("CL_RAGGED", 1), ("CL_HEAD_DIM", d), ("CL_KV_HEADS", 1), ("CL_Q_HEADS", 1),
                      ("CL_ROWS", rows), ("CL_SKV", p["skv"])):
             unit.define(k, v)
         unit.define("CL_SCALE", _f(float(p.get("scale", 1.0))))
-        norm = p.get("norm_eps") or {}
         unit.define("CL_LINEAR", bool(p.get("linear")))
         if p.get("k_major") and p["skv"] % 32:
             raise CodegenError("feature-major keys need a key count in whole 32-key steps")
         unit.define("CL_KT", bool(p.get("k_major")))
         unit.define("CL_QNORM", "q" in norm)
-        unit.define("CL_KNORM", "k" in norm)
+        unit.define("CL_KNORM", "k" in norm and not kpre)
         unit.define("CL_QNORM_EPS", _f(float(norm.get("q", 0.0))))
         unit.define("CL_KNORM_EPS", _f(float(norm.get("k", 0.0))))
         for role, macro in (("Q", "CL_ARG_Q"), ("K", "CL_ARG_K"), ("V", "CL_ARG_V")):
-            unit.define(macro, op[role])
+            unit.define(macro, "Scratch_kn" if kpre and role == "K" else op[role])
         for k, v in plan.tiling.items():
-            if k != "SHARED":
+            if k not in ("SHARED", "KPRE"):
                 unit.define(f"CL_PF_{k}", int(v))
+        unit.define("CL_EMIT_KPRE", kpre)
         unit.templates += ["attn_prefill_lds.hip", "attn_combine.hip"]
+        if kpre:
+            by_name = self._by_name(params)
+            key_rows = p["units"] * p["skv"]
+            unit.define("CL_KPRE_ROWS", key_rows)
+            unit.define("CL_KPRE_SRC", op["K"])
+            unit.define("CL_KPRE_DST", "Scratch_kn")
+            args = unit.signature("CL_KPRE_PARAMS", "CL_KPRE_NAME", ENTRY + "_keys", [by_name[op["K"]], by_name["Scratch_kn"]], ())
+            unit.templates.append("rows_norm.hip")
+            unit.launch(ENTRY + "_keys", (-(-(key_rows * (d // 8)) // 256), 1, 1), 256, 0, args)
         if partial:
             items = -(-(-(-rows // 128)) // 8) * 8              # padded to a multiple of 8 (one eighth of the space per XCD)
             unit.launch(ENTRY, (items, p["units"], splits), 256, 0, self._partial_args)

@@ -394,8 +394,16 @@ def attn_many_rows_candidates(low, role, factor, arch: Arch):
     steps = _ceil(_ceil(p["skv"], 32), splits)
     # a workgroup-step is 32 matrix ops per wave beside as many vector ops; two workgroups per CU
     score = _waves_time(items, 2, arch) * (steps * 2200 + 9000)
-    return [TileDict("attn_prefill", role, dict(SHARED=1), output_tile=[128, vd], rstep_map={"kv": 32}, n_threads=256,
-                     split_factor=factor, score=score, lds_bytes=4 * 32 * (d + vd) * 2, est_vgprs=230)]
+    out = [TileDict("attn_prefill", role, dict(SHARED=1), output_tile=[128, vd], rstep_map={"kv": 32}, n_threads=256,
+                    split_factor=factor, score=score, lds_bytes=4 * 32 * (d + vd) * 2, est_vgprs=230)]
+    # normalised keys: every workgroup of a unit normalises all of its keys again (a quarter more
+    # matrix ops per step and the scaling of the scores); with many row blocks per unit a launch
+    # that normalises them once into a scratch copy is cheaper
+    if "k" in (p.get("norm_eps") or {}) and not p.get("k_major") and d in (64, 128, 256) and rows >= 512:
+        out.append(TileDict("attn_prefill", role, dict(SHARED=1, KPRE=1), output_tile=[128, vd], rstep_map={"kv": 32},
+                            n_threads=256, split_factor=factor, score=0.8 * score, lds_bytes=4 * 32 * (d + vd) * 2,
+                            est_vgprs=230))
+    return out
 
 
 # ----------------------------------------------------------------------------- MLA decode

@@ -17,11 +17,12 @@ from cleave_amd.pipeline.direct import kernel_for, stage_graph
 pytestmark = pytest.mark.gpu
 
 
-def _check(fn, dtype, shapes, seed=7):
+def _check(fn, dtype, shapes, seed=7, **how):
     prog = fn.trace(dtype, **shapes)
     args = prog.random_inputs(seed=seed)
-    print(f"dense prefill case {prog.name} {dtype} {shapes}", flush=True)
-    out = kernel_for(prog, template="attn_prefill", tiling=dict(SHARED=1))(*args)
+    how = how or dict(template="attn_prefill", tiling=dict(SHARED=1))
+    print(f"dense prefill case {prog.name} {dtype} {shapes} {how}", flush=True)
+    out = kernel_for(prog, **how)(*args)
     torch.cuda.synchronize()
     want = program_oracle.evaluate(prog, list(args))[0]
     np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)
@@ -77,17 +78,24 @@ def test_qk_norm_attention():
     _check(C.qknorm, cl.bf16, dict(HQ=4, HKV=4, SQ=70, SKV=45, D=64))
     _check(k_only, cl.f16, dict(HQ=8, HKV=1, SQ=33, SKV=200, D=128))
     _check(q_only, cl.f16, dict(HQ=2, HKV=2, SQ=96, SKV=64, D=64))
+    # (the keys normalised by a launch of their own ahead of the attention kernel)
+    pre = dict(template="attn_prefill", tiling=dict(SHARED=1, KPRE=1))
+    _check(C.qknorm, cl.f16, dict(HQ=8, HKV=2, SQ=100, SKV=300, D=128), **pre)
+    _check(C.qknorm, cl.bf16, dict(HQ=4, HKV=4, SQ=70, SKV=45, D=64), **pre)
+    _check(k_only, cl.f16, dict(HQ=8, HKV=1, SQ=33, SKV=200, D=128), **pre)
+    _check(C.qknorm, cl.f16, dict(HQ=8, HKV=2, SQ=256, SKV=512, D=128), split=4, **pre)
     shapes = dict(HQ=64, HKV=8, SQ=4096, SKV=4096, D=128)
     prog = C.qknorm.trace(cl.f16, **shapes)
     q, k, v = prog.random_inputs(seed=19)
-    out = kernel_for(prog)(q, k, v)
-    torch.cuda.synchronize()
-    gen = np.random.default_rng(3)
     norm = lambda x: x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)   # noqa: E731
-    for h, s in zip(gen.integers(0, 64, 32), gen.integers(0, 4096, 32)):
-        w = torch.softmax((norm(k[h // 8].double()) @ norm(q[h, s].double())) / 128 ** 0.5, dim=0)
-        np.testing.assert_allclose(out[h, s].float().cpu().numpy(), (w @ v[h // 8].double()).float().cpu().numpy(),
-                                   rtol=1e-2, atol=1e-2)
+    for how in (dict(template="attn_prefill", tiling=dict(SHARED=1)), pre):
+        out = kernel_for(prog, **how)(q, k, v)
+        torch.cuda.synchronize()
+        gen = np.random.default_rng(3)
+        for h, s in zip(gen.integers(0, 64, 32), gen.integers(0, 4096, 32)):
+            w = torch.softmax((norm(k[h // 8].double()) @ norm(q[h, s].double())) / 128 ** 0.5, dim=0)
+            np.testing.assert_allclose(out[h, s].float().cpu().numpy(), (w @ v[h // 8].double()).float().cpu().numpy(),
+                                       rtol=1e-2, atol=1e-2)
 
 
 @pytest.mark.parametrize("waves", [1, 2, 4])

@@ -129,7 +129,14 @@ def test_qk_norm_attention_is_attention_with_normalised_operands():
     assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}     # the streaming kernel has no norm form
     with pytest.raises(ScheduleRejected, match="many-row kernel"):
         search_tiling(stage_graph(C.qknorm.trace(cl.f16, HQ=4, HKV=4, SQ=1, SKV=256, D=128)))
+    # the first candidate normalises the keys once, by a launch of its own into a scratch copy the attention kernel reads
     m = parse_manifest(source_for(C.qknorm.trace(cl.f16, HQ=64, HKV=8, SQ=4096, SKV=4096, D=128)))
+    assert [launch["entry"] for launch in m["launches"]] == ["main_kernel_keys", "main_kernel"]
+    assert m["launches"][0]["args"] == ["PlaceHolder_k", "Scratch_kn"] and m["launches"][0]["grid"] == ["2048", "1", "1"]
+    assert m["launches"][1]["args"] == ["PlaceHolder_q", "PlaceHolder_k", "PlaceHolder_v", "Scratch_kn", "OutputNode_0"]
+    assert [p["role"] for p in m["params"]] == ["input", "input", "input", "scratch", "output"]
+    m = parse_manifest(source_for(C.qknorm.trace(cl.f16, HQ=64, HKV=8, SQ=4096, SKV=4096, D=128), template="attn_prefill",
+                                  tiling=dict(SHARED=1)))
     assert m["launches"][0]["grid"] == ["256", "8", "1"] and m["launches"][0]["block"][0] == 256
 
 
