@@ -45,6 +45,10 @@ def _f(x: float) -> str:
     return text + "f"
 
 
+def tail_requested(tile) -> bool:
+    return bool(int(tile.get("TAIL", 0)))
+
+
 def _c_param(p: ParamSpec) -> str:
     if p.role == "scalar":
         return f"{_C_TYPES[p.dtype]} {p.name}"
@@ -295,6 +299,15 @@ class HipCodeGen:
             if (not p["trans_B"] and p["N"] % 8) or (p["trans_A"] and p["M"] % 8) or p["K"] % 8:
                 raise CodegenError("16-byte global chunks need the minor extent of each operand to be a multiple of 8")
             grid = (1 if rowsum else -(-p["N"] // out_bn), -(-p["M"] // tile["BM"]), batch * splits)
+            stages = int(tile.get("STAGES", 2))
+            if stages != 2:
+                waves = tile["WM"] * tile["WN"]
+                if (stages != 3 or rowsum or not int(tile.get("ASM_LOADS", 1)) or 3 * (tile["BM"] + tile["BN"]) * 128 > 160 * 1024
+                        or (tile["BM"] // 8) % waves or (tile["BN"] // 8) % waves
+                        or (tail_requested(tile) and (tile["BM"] // 16) % waves)):
+                    raise CodegenError("three LDS stages: tiles of which three images fit 160 KiB, every wave loading the same "
+                                       "number of 1 KiB units of each (of a tail's half-height A tile as well), assembly tile "
+                                       "loads, no row-sum walk")
             tail = int(tile.get("TAIL", 0))
             if tail:
                 # the last `tail` tiles run as two half-height workgroups each, on a one-dimensional grid

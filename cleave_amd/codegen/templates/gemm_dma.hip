@@ -85,6 +85,23 @@ __shared__ __attribute__((aligned(1024))) elem_t gd_a0[GD_A_ELEMS];
 __shared__ __attribute__((aligned(1024))) elem_t gd_a1[GD_A_ELEMS];
 __shared__ __attribute__((aligned(1024))) elem_t gd_b0[GD_B_ELEMS];
 __shared__ __attribute__((aligned(1024))) elem_t gd_b1[GD_B_ELEMS];
+// CL_STAGES = 3 (tiles of which three images fit LDS): the loads of a step are asked for two steps
+// ahead, one slice in front of every row of matrix ops over the whole length of a step, instead
+// of all at the top of the step before.  The path from L2 into the compute unit takes a step's
+// 64 loads in about a third of the step; asked for all at once, or within half a step, they queue
+// and every wave stands still at its loads (measured: 14 % of the kernel with every load an L2
+// hit); spread over a whole step they do not, and a load has a whole step more to arrive.
+#ifndef CL_STAGES
+#define CL_STAGES 2
+#endif
+#if CL_STAGES == 3
+__shared__ __attribute__((aligned(1024))) elem_t gd_a2[GD_A_ELEMS];
+__shared__ __attribute__((aligned(1024))) elem_t gd_b2[GD_B_ELEMS];
+#if !CL_ASM_LOADS || CL_ROWSUM
+#error "three stages: assembly tile loads (the kernel counts its own loads in flight), no row-sum walk"
+#endif
+#endif
+static_assert(CL_STAGES == 2 || CL_STAGES == 3, "two or three LDS stages");
 
 // ---- K-minor image: row r at r * 64, chunk ch at slot ch ^ swz(r) ------------------------------
 // (row & 6: measured at the full rate of a linear read for the operand shape, lane = row l % 16, chunk l / 16)
@@ -424,7 +441,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }                                                                                               \
     GD_STEP_SCHED()                                                                                 \
   }
-#if CL_SPREAD_LOADS || CL_ASM_MFMA
+#if CL_SPREAD_LOADS || CL_ASM_MFMA || CL_STAGES == 3
 // every row of matrix ops closes with a scheduling barrier: the order of the source (this row's
 // loads of the next step, its matrix ops, the fragment reads for two rows on) is the order of the
 // instruction stream
@@ -483,6 +500,39 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // Two steps per trip, one on each stage, with no branch inside: the loads issued in the second
   // half are clamped onto the last step (for an even step count the final trip fetches that step
   // once more into the idle stage, which nobody reads).
+#if CL_STAGES == 3
+  {
+    constexpr int per_step_ = decltype(opa)::PER + decltype(opb)::PER;     // loads per wave and step
+    static_assert(decltype(opa)::UNITS % GD_WAVES == 0 && decltype(opb)::UNITS % GD_WAVES == 0 && per_step_ < 32,
+                  "three stages: every wave issues the same number of loads per step (the wait counts them)");
+    // at most the loads this wave asked for during the step just done (those of two steps on) are
+    // still on their way: the next step's images have landed; after the barrier, everybody's
+#define GD_STEP_END3()                                                                              \
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (per_step_ & 15) | ((per_step_ >> 4) << 14));               \
+    __syncthreads();
+#define GD_AHEAD(kt) ((kt) + 2 < KT ? (kt) + 2 : KT - 1)
+#define GD_NEXT_S2(r) GD_ISSUE_SLICE(r, GD_AHEAD(kt), gd_a2, gd_b2)
+#define GD_NEXT_S0(r) GD_ISSUE_SLICE(r, GD_AHEAD(kt), gd_a0, gd_b0)
+#define GD_NEXT_S1(r) GD_ISSUE_SLICE(r, GD_AHEAD(kt), gd_a1, gd_b1)
+    GD_ISSUE(0, gd_a0, gd_b0)
+    GD_ISSUE((1 < KT ? 1 : KT - 1), gd_a1, gd_b1)
+    GD_STEP_END3()
+    // (past the last step the loads are clamped onto it and go into the stage left a step ago,
+    // which nobody reads again: every step issues the same number of loads)
+    for (int kt = 0;;) {
+      GD_COMPUTE(gd_a0, gd_b0, GD_NEXT_S2)
+      GD_STEP_END3()
+      if (++kt >= KT) break;
+      GD_COMPUTE(gd_a1, gd_b1, GD_NEXT_S0)
+      GD_STEP_END3()
+      if (++kt >= KT) break;
+      GD_COMPUTE(gd_a2, gd_b2, GD_NEXT_S1)
+      GD_STEP_END3()
+      if (++kt >= KT) break;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // no load may still be on its way into LDS past this point
+  }
+#else
   GD_ISSUE(0, gd_a0, gd_b0)
   GD_STEP_END()
 #if CL_SPREAD_LOADS
@@ -505,6 +555,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 #endif
   if constexpr (KT % 2 == 1) GD_COMPUTE(gd_a0, gd_b0, GD_NO_NEXT)     // an odd number of steps ends on stage 0
+#endif  // CL_STAGES
 
   // ---- epilogue: acc[i][j][r] = C[m0 + am + 16 i + c][n0 + bn + 16 j + 4 g + r] ----------------
   gd_acc_drain();

@@ -100,6 +100,11 @@ def gemm_candidates(low, role, factor, arch: Arch):
         lds_clk = live * (tm + tn) * 16 * wm * wn * kps * 2 / 256.0
         pass_clk = max(mfma_clk, l1_clk, lds_clk) + 2500 + 1200 * (kps // bk) / max(1, min(live, 2))
         score = passes * pass_clk
+        # (where the direct-to-LDS kernel offers the same tile it has measured a quarter to a third
+        # faster -- 2048 x 4096 x 4096 on 128 x 128 tiles: 67 against 91 us -- while this model ranked the
+        # register-staged one ahead: its candidates go behind)
+        if low.family == "matmul" and bm * bn >= 64 * 64:
+            score *= 1.5
         tiling = dict(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, GDEPTH=depth)
         out.append(TileDict("gemm", role, tiling, output_tile=[bm, bn], rstep_map={"k": bk}, n_threads=threads,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
@@ -164,6 +169,14 @@ def gemm_dma_candidates(low, role, factor, arch: Arch):
         tiling = dict(BM=bm, BN=bn, BK=64, WM=wm, WN=wn)
         out.append(TileDict("gemm_dma", role, tiling, output_tile=[bm, bn], rstep_map={"k": 64}, n_threads=threads,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+        # Three LDS stages where three images fit beside as many workgroups per compute unit as two
+        # allow: the loads of a step asked for two steps ahead and spread over the whole step
+        # (256 x 128 tiles on 4096 x 14336 x 4096: 426 us against 526).
+        if (3 * (bm + bn) * 128 * per_cu <= arch.lds_bytes and units_a % (wm * wn) == 0 and units_b % (wm * wn) == 0
+                and not post_norm):
+            out.append(TileDict("gemm_dma", role, dict(tiling, STAGES=3), output_tile=[bm, bn], rstep_map={"k": 64},
+                                n_threads=threads, split_factor=factor, score=0.85 * score, lds_bytes=3 * lds // 2,
+                                est_vgprs=vgprs))
         # A last round that fills at most half of the machine: its tiles as two half-height
         # workgroups each (row-major A, one workgroup per compute unit, unsplit, unbatched).
         tail = blocks % arch.compute_units

@@ -71,6 +71,30 @@ def test_matmul_gemm_dma(tiling, split):
     _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling, split=split)
 
 
+@pytest.mark.parametrize("k", [64, 128, 192, 256, 448, 576])
+@pytest.mark.parametrize("tiling", [dict(BM=64, BN=64, BK=64, WM=2, WN=2, STAGES=3), dict(BM=256, BN=128, BK=64, WM=4, WN=2, STAGES=3),
+                                    dict(BM=128, BN=256, BK=64, WM=2, WN=4, STAGES=3, GROUP_M=2)],
+                         ids=lambda t: "x".join(str(v) for v in t.values()))
+def test_matmul_gemm_dma_three_stages(tiling, k):
+    """Three LDS stages (loads asked for two steps ahead, spread over a step's rows, the kernel
+    counting its own loads in flight): one to nine K steps, so that the walk ends on each of the
+    three stages and the clamped loads past the last step land in an idle one; ragged tiles on both
+    axes; split over K (three steps per split) and the transposed-weight, bf16 form as well."""
+    fn, dt, mk = C.CASES["c1"]
+    shapes = dict(M=600, N=776, K=k)
+    _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling)
+    if k == 576:
+        _check(fn.trace(dt, **shapes), mk, shapes, template="gemm_dma", tiling=tiling, split=3)
+        prog = matmul_nt.trace(cl.bf16, **shapes)
+        g = torch.Generator(device="cpu").manual_seed(5)
+        ins = [((torch.rand(*shp, generator=g) * 2 - 1) / 24).to(torch.bfloat16) for shp in ((600, 576), (776, 576))]
+        want = po.evaluate(prog, ins)[0]
+        kernel = kernel_for(prog, template="gemm_dma", tiling=tiling)
+        print(f"case matmul_nt bf16 gemm_dma {tiling}", flush=True)
+        got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("tiling", [dict(BM=64, BN=64, BK=64, WM=2, WN=2, TAIL=24), dict(BM=64, BN=64, BK=64, WM=2, WN=2, TAIL=5),
                                     dict(BM=256, BN=128, BK=64, WM=4, WN=2, TAIL=6),
                                     dict(BM=256, BN=256, BK=64, WM=2, WN=2, TAIL=8),
