@@ -100,11 +100,11 @@ def gemm_candidates(low, role, factor, arch: Arch):
         lds_clk = live * (tm + tn) * 16 * wm * wn * kps * 2 / 256.0
         pass_clk = max(mfma_clk, l1_clk, lds_clk) + 2500 + 1200 * (kps // bk) / max(1, min(live, 2))
         score = passes * pass_clk
-        # (where the direct-to-LDS kernel offers the same tile it has measured a quarter to a third
-        # faster -- 2048 x 4096 x 4096 on 128 x 128 tiles: 67 against 91 us -- while this model ranked the
-        # register-staged one ahead: its candidates go behind)
-        if low.family == "matmul" and bm * bn >= 64 * 64:
-            score *= 1.5
+        # (where the direct-to-LDS kernel offers the same tile it has measured a quarter to two thirds
+        # faster -- 2048 x 4096 x 4096 on 128 x 128 tiles: 67 against 91 us; 512 x 512 x 4096 on 16 x 32 tiles:
+        # 14 against 42 -- while this model ranked the register-staged one ahead: its candidates go behind)
+        if low.family == "matmul":
+            score *= 2.0
         tiling = dict(BM=bm, BN=bn, BK=bk, WM=wm, WN=wn, GDEPTH=depth)
         out.append(TileDict("gemm", role, tiling, output_tile=[bm, bn], rstep_map={"k": bk}, n_threads=threads,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
@@ -165,7 +165,8 @@ def gemm_dma_candidates(low, role, factor, arch: Arch):
         lds_clk = waves_per_simd * kps * 2 * 16 * (tm / a_rate + tn / b_rate)
         fetch_clk = live * ((bm + bn) * kps * 2) / 24.0
         pass_clk = max(mfma_clk, lds_clk, fetch_clk) + 2500 + 1500 * (kps // 64) / max(1, min(live, 2))
-        score = passes * pass_clk
+        # (equal tiles: the wave grids with more waves have measured a few per cent faster -- more loads in flight)
+        score = passes * pass_clk * (1.0 + 0.03 / (wm * wn))
         tiling = dict(BM=bm, BN=bn, BK=64, WM=wm, WN=wn)
         out.append(TileDict("gemm_dma", role, tiling, output_tile=[bm, bn], rstep_map={"k": 64}, n_threads=threads,
                             split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
