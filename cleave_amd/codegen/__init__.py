@@ -365,6 +365,9 @@ class HipCodeGen:
             lds = skinny_lds_bytes(-(-p["M"] // 16), tile["WAVES_N"], tile["WAVES_K"])
             if lora:
                 lds = lora_lds_bytes(-(-p["M"] // 16), tile["WAVES_N"], tile["WAVES_K"], p["R"])
+            if lds > 160 * 1024:
+                raise CodegenError(f"the few-row matmul's cross-wave reduction would need {lds} bytes of LDS at "
+                                   f"WAVES_N={tile['WAVES_N']} WAVES_K={tile['WAVES_K']} and {p['M']} rows (160 KiB per workgroup)")
             unit.launch(ENTRY, grid, tile["WAVES_N"] * tile["WAVES_K"] * 64, lds, self._partial_args)
         if combine:
             entry, args, blocks = self._combine_args

@@ -296,6 +296,9 @@ def test_codegen_refuses_impossible_plans():
                                                split_factor=None)).__class__(**{**apply_tiling(
                                                    TileDict("gemm", "main", dict(BM=64, BN=64, BK=64, WM=2, WN=2),
                                                             flat_graph=g)).__dict__, "problem": {**g.lowered.problem, "K": 4100}}))
+    with pytest.raises(CodegenError, match="bytes of LDS"):          # 64 rows reduced over eight waves: 197 KB
+        HipCodeGen().gen(apply_tiling(TileDict("skinny", "main", dict(WAVES_N=2, WAVES_K=4), flat_graph=stage_graph(
+            C.rmsnorm_matmul.trace(cl.f16, M=64, N=1024, K=1024)))))
     with pytest.raises(CodegenError, match="three LDS stages"):      # three 64 KB images do not fit
         HipCodeGen().gen(apply_tiling(TileDict("gemm_dma", "main", dict(BM=256, BN=256, BK=64, WM=2, WN=4, STAGES=3), flat_graph=g)))
     with pytest.raises(CodegenError, match="no template"):
