@@ -20,6 +20,7 @@ from oracle import program_oracle as po
 
 pytestmark = pytest.mark.gpu
 DRAWS = 36
+PAGED_DRAWS = 24
 
 
 def _draw(rng, n):
@@ -82,3 +83,26 @@ def test_drawn_shapes_and_tilings_against_the_oracle(seed):
         np.testing.assert_allclose(got.reshape(want.shape), want, rtol=1e-2, atol=1e-2, err_msg=f"{label} {how}")
         ran += 1
     assert 3 * ran >= 2 * DRAWS, f"only {ran} of {DRAWS} draws ran"
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_drawn_paged_decode_requests_against_the_oracle(seed):
+    """Paged decode over drawn page sizes, head groups, request lengths (empty, one token, under a
+    page, many pages), wave counts, splits and chunked work items; the log-sum-exp row of an empty
+    request is -inf and its output row zero."""
+    from tests.test_gpu_paged import check
+    rng = random.Random(seed)
+    for n in range(PAGED_DRAWS):
+        page = rng.choice([1, 16, 64])
+        kv_heads, group = rng.choice([2, 4, 8]), rng.choice([2, 4, 8])
+        if kv_heads * group > 32:
+            kv_heads = 32 // group
+        lens = [rng.choice([0, 1, rng.randrange(1, 70), rng.randrange(1, 2000)]) for _ in range(rng.randrange(1, 12))]
+        pages = sum(-(-length // page) for length in lens) + rng.randrange(1, 50)
+        args = C.paged_workload(lens, page_size=page, num_pages=pages, hq=kv_heads * group, hkv=kv_heads, seed=1000 * seed + n)
+        if page == 1:
+            args = args[:5] + args[6:]
+        how = dict(waves=rng.choice([1, 2, 4, 8]), split=rng.choice([None, 2, 4, 8]), hq=kv_heads * group, hkv=kv_heads)
+        if how["split"] and page == 64 and rng.random() < 0.5:
+            how.update(chunk_pages=rng.choice([1, 3, 16, -1]), prefetch=rng.choice([1, 2]), waves=8)
+        check(args, lens, page, **how)
