@@ -24,7 +24,7 @@ import math
 from dataclasses import dataclass, field
 
 from ..core.errors import LoweringRejected
-from .graph import ComputeOpNode, Graph, Node, OutputNode, PlaceHolderNode
+from .graph import ComputeOpNode, Graph, Node, OutputNode, PlaceHolderNode, hoist_splits
 
 
 @dataclass
@@ -516,6 +516,8 @@ def recognize(graph: Graph) -> Lowered:
     outs = graph.outputs
     if len(outs) != 1:
         raise LoweringRejected(f"{graph.name}: kernels are built for single-output programs, got {len(outs)} outputs")
+    graph = hoist_splits(graph)
+    outs = graph.outputs
     view = _View(graph)
     for matcher in _MATCHERS:
         hit = matcher(view, outs[0].source)

@@ -150,3 +150,94 @@ def to_ir(structure, symbol_map=None, dtype: str = "float16", out_dtype: str | N
     if not n_out:
         raise LoweringRejected("structure has no output op")
     return Graph(nodes, dtype, name)
+
+
+_POINTWISE = ("add", "sub", "mul", "div", "exp", "sqrt", "rsqrt", "silu")
+
+
+def _split_shape(shape, dim, factor) -> tuple:
+    if shape[dim] % factor:
+        raise LoweringRejected(f"extent {shape[dim]} of axis {dim} does not divide into {factor} splits")
+    return (factor,) + tuple(shape[:dim]) + (shape[dim] // factor,) + tuple(shape[dim + 1:])
+
+
+def hoist_splits(graph: Graph) -> Graph:
+    """The same program with every split that sits on a computed tensor moved up to the graph inputs.
+
+    The superoptimizer may place the split of a split-KV attention anywhere between the key
+    product and the exponential (``tests/integration/graph_structures/gqa/*valid_{2..5}.graph``);
+    everything from the keys to that point works on each key position by itself, so splitting
+    the scores there and splitting the keys are one program.  A split moves through a pointwise
+    op onto its tensor operand(s) of the same shape, and through a matmul onto the operand that
+    owns the split axis (rows: A, columns: B).  It does not move through a reduction, a
+    broadcast operand or a batch axis of a matmul: such a graph is refused.  Producers that are
+    left without consumers are dropped; a producer that is still read unsplit stays, and the
+    input it reads is then consumed both ways, which the family recognition refuses.  The given
+    graph is left as it is."""
+    if not any(n.op == "split" and isinstance(n.inputs[0], ComputeOpNode) for n in graph.ops):
+        return graph
+    clone = {}
+    for n in graph.nodes:
+        if isinstance(n, ComputeOpNode):
+            clone[id(n)] = ComputeOpNode(n.name, n.shape, n.dtype, op=n.op, inputs=[clone[id(i)] for i in n.inputs],
+                                         scalar=n.scalar, scalar_on_left=n.scalar_on_left, attrs=dict(n.attrs))
+        elif isinstance(n, OutputNode):
+            clone[id(n)] = OutputNode(n.name, n.shape, n.dtype, source=clone[id(n.source)])
+        else:
+            clone[id(n)] = n
+    nodes = [clone[id(n)] for n in graph.nodes]
+    serial = 0
+    while True:
+        split = next((n for n in nodes if isinstance(n, ComputeOpNode) and n.op == "split"
+                      and isinstance(n.inputs[0], ComputeOpNode)), None)
+        if split is None:
+            break
+        producer, dim, factor = split.inputs[0], split.attrs["dim"], split.shape[0]
+        refusal = LoweringRejected(f"split of a computed tensor ({producer.name}) has no partial/combine cut")
+        moved = []          # (operand index, axis) of the producer's operands that take the split
+
+        if producer.op in _POINTWISE:
+            for k, operand in enumerate(producer.inputs):
+                if tuple(operand.shape) != tuple(producer.shape):
+                    raise refusal                      # a broadcast operand: the split axis is not its own
+                moved.append((k, dim))
+        elif producer.op == "matmul":
+            a, b = producer.inputs
+            rank = len(producer.shape)
+            if dim == rank - 1:
+                moved.append((1, len(b.shape) - (2 if producer.attrs.get("trans_B") else 1)))
+            elif dim == rank - 2:
+                moved.append((0, len(a.shape) - (1 if producer.attrs.get("trans_A") else 2)))
+            else:
+                raise refusal
+        else:
+            raise refusal
+        fresh, operands = [], list(producer.inputs)
+        for k, axis in moved:
+            serial += 1
+            piece = ComputeOpNode(f"split_hoisted{serial}_{operands[k].name}", _split_shape(operands[k].shape, axis, factor),
+                                  operands[k].dtype, op="split", inputs=[operands[k]], attrs={"dim": axis})
+            fresh.append(piece)
+            operands[k] = piece
+        serial += 1
+        lifted = ComputeOpNode(f"{producer.name}_hoisted{serial}", split.shape, producer.dtype, op=producer.op,
+                               inputs=operands, scalar=producer.scalar, scalar_on_left=producer.scalar_on_left,
+                               attrs=dict(producer.attrs))
+        at = nodes.index(split)
+        nodes[at:at + 1] = fresh + [lifted]
+        for n in nodes:
+            if isinstance(n, ComputeOpNode):
+                n.inputs = [lifted if i is split else i for i in n.inputs]
+            elif isinstance(n, OutputNode) and n.source is split:
+                n.source = lifted
+        # drop what nobody reads any more
+        while True:
+            read = {id(i) for n in nodes if isinstance(n, ComputeOpNode) for i in n.inputs}
+            read |= {id(n.source) for n in nodes if isinstance(n, OutputNode)}
+            dead = [n for n in nodes if isinstance(n, ComputeOpNode) and id(n) not in read]
+            if not dead:
+                break
+            nodes = [n for n in nodes if not any(n is d for d in dead)]
+    out = Graph(nodes, graph.dtype, graph.name)
+    out.dyn_dims = list(graph.dyn_dims)
+    return out
