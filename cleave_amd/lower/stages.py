@@ -84,17 +84,61 @@ def split_stages(graph: StageGraph, factor: int) -> list:
     return [partial, combine]
 
 
+def join_cut_pair(partial, combine) -> list:
+    """One structure from an already cut ``[partial, combine]`` pair as the reference's split pass
+    leaves it (``python/cleave/lower/split.py:701-717``; stored examples:
+    ``tests/integration/graph_structures/*/after_split_*.graph``): both halves number their tensors
+    from the same start, and the k-th output of the partial is the k-th input of the combine.  The
+    halves are joined there, so that the operator is recognised as a whole and cut again into the
+    partial and combine kernels this back end has for it."""
+    def tensors(entry, key):
+        return list(entry.get(key, ()))
+
+    handed = [tensors(e, "input_tensors")[0] for e in partial if e["op_type"] == "kn_output_op"]
+    taken = [tensors(e, "output_tensors")[0] for e in combine if e["op_type"] == "kn_input_op"]
+    if len(handed) != len(taken) or not handed:
+        raise LoweringRejected(f"cut pair: the partial hands over {len(handed)} tensors, the combine takes {len(taken)}")
+    shift = 1 + max(t["guid"] for e in partial for key in ("input_tensors", "output_tensors") for t in tensors(e, key))
+    rename = {}
+    for out_t, in_t in zip(handed, taken):
+        if [d for d in out_t["dim"] if d] != [d for d in in_t["dim"] if d]:
+            raise LoweringRejected(f"cut pair: partial output {out_t['dim']} does not fit combine input {in_t['dim']}")
+        rename[in_t["guid"]] = out_t["guid"]
+
+    def moved(t):
+        return dict(t, guid=rename.get(t["guid"], t["guid"] + shift))
+
+    joined = [e for e in partial if e["op_type"] != "kn_output_op"]
+    for e in combine:
+        if e["op_type"] == "kn_input_op":
+            continue
+        e = dict(e)
+        for key in ("input_tensors", "output_tensors"):
+            if key in e:
+                e[key] = [moved(t) for t in e[key]]
+        joined.append(e)
+    return joined
+
+
+def _is_cut_pair(structure) -> bool:
+    return len(structure) == 2 and all(isinstance(half, (list, tuple)) for half in structure)
+
+
 def to_bundles(structures, symbol_map=None, split_factors=None, dtype="float16", out_dtype=None,
                input_names=None, **_ignored) -> list:
     """One bundle per structure: ``[main]`` or, with ``split_factors=[f]``, ``[partial, combine]``.
-    A structure given as ``[partial_structure, combine_structure]`` (an already cut pair from a
-    stored file) is recognised from its partial side only when it is a plain split of a known
-    family; otherwise it is refused."""
+    A structure given as ``[partial_structure, combine_structure]`` (an already cut pair) is
+    joined, recognised as one operator and cut into this back end's own stages, at
+    ``split_factors[0]`` or, without it, at the split count the pair's split ops state."""
     out = []
     for s in structures:
-        g = to_ir(s, symbol_map, dtype, out_dtype, input_names)
-        if split_factors:
-            out.append(split_stages(g, int(split_factors[0])))
-        else:
-            out.append([g])
+        pair = _is_cut_pair(s)
+        g = to_ir(join_cut_pair(*s) if pair else s, symbol_map, dtype, out_dtype, input_names)
+        factor = int(split_factors[0]) if split_factors else None
+        if pair and factor is None:
+            stated = {n.shape[0] for n in g.nodes if getattr(n, "op", None) == "split"}
+            if len(stated) != 1:
+                raise LoweringRejected(f"cut pair: split ops state the split counts {sorted(stated)}")
+            factor = stated.pop()
+        out.append(split_stages(g, factor) if factor else [g])
     return out

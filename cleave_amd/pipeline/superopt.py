@@ -121,8 +121,13 @@ class GraphSet(Sequence):
 
     @classmethod
     def from_structures(cls, program, structures, symbol_map=None, split=()) -> "GraphSet":
-        """Wrap structures produced elsewhere (e.g. a superoptimizer checkpoint)."""
+        """Wrap structures produced elsewhere (e.g. a superoptimizer checkpoint); a ``[partial,
+        combine]`` pair left by the reference's split pass is joined into the one structure it cuts."""
+        from ..lower.stages import _is_cut_pair, join_cut_pair
+
         def wrapped(position, structure):
+            if _is_cut_pair(structure):
+                structure = join_cut_pair(*structure)
             cut = any(entry["op_type"].startswith("kn_split_") for entry in structure)
             return SearchedGraph(position, structure, symbol_map, cut, program, split if cut else ())
 

@@ -147,3 +147,94 @@ def test_unread_producers_are_dropped_and_read_ones_kept():
     both = hoist_splits(stored("before_split_gqa_graph_structure_invalid_6.graph"))
     assert both.op_kinds().count("exp") == 2        # the unsplit exponential is still read: K is consumed both ways
     assert any(isinstance(n, ComputeOpNode) and n.op == "split" for n in both.nodes)
+
+
+# ---- what the reference's split pass makes of those structures (after_split_*): a [partial, combine]
+# pair where it cuts, the structure itself where there is nothing to cut, an empty list where it refuses
+from cleave_amd.lower import to_bundles  # noqa: E402
+from cleave_amd.lower.stages import join_cut_pair  # noqa: E402
+
+AFTER = sorted(p.name for p in STRUCT.glob("after_split_*.graph"))
+
+
+def _after(name):
+    return json.loads((STRUCT / name).read_text())
+
+
+def _sizes(name):
+    return {12: 4096} if "rmsnorm" in name else None
+
+
+@pytest.mark.parametrize("name", AFTER)
+def test_output_of_the_reference_s_split_pass_is_taken_as_it_comes(name):
+    after, before_name = _after(name), name.replace("after_split", "before_split")
+    if not after:
+        assert "invalid" in name
+        with pytest.raises(LoweringRejected):
+            to_bundles([after])
+        return
+    stages, = to_bundles([after], symbol_map=_sizes(name))
+    whole = recognize(stored(before_name, symbol_map=_sizes(name)))
+    assert stages[0].lowered.family == whole.family and stages[0].lowered.problem == whole.problem
+    if isinstance(after[0], list):
+        assert [(g.role, g.split_factor) for g in stages] == [("partial", 2), ("combine", 2)]
+        assert stages[0].lowered.split_dim == whole.split_dim is not None
+        assert sorted(stages[0].lowered.split_axes.values()) == sorted(whole.split_axes.values())
+    else:
+        assert [g.role for g in stages] == ["main"] and whole.split_dim is None
+
+
+def _spelling(graph):
+    """Ops of a graph without names: kind, constants, attributes and operands as positions."""
+    place = {id(n): ("in", k) for k, n in enumerate(graph.placeholders)}
+    rows = []
+    for n in graph.ops:
+        attrs = {k: v for k, v in n.attrs.items() if not (k == "squeeze" and n.attrs.get("dim") != 0)}
+        rows.append((n.op, n.scalar, tuple(sorted(attrs.items())), tuple(place[id(i)] for i in n.inputs), tuple(n.shape)))
+        place[id(n)] = ("op", len(rows) - 1)
+    return sorted(rows, key=repr)
+
+
+@pytest.mark.parametrize("case", [2, 3, 4, 5])
+def test_moved_splits_agree_with_the_reference_s_cut(case):
+    """The reference cuts all five split-KV spellings into one and the same pair; joined again,
+    that pair spells what moving the split to the inputs gives here (as multisets of ops with
+    their constants, axes and shapes; operand positions are compared on the cut pair's own order)."""
+    moved = hoist_splits(stored(f"before_split_gqa_graph_structure_valid_{case}.graph"))
+    cut = to_ir(join_cut_pair(*_after(f"after_split_gqa_graph_structure_valid_{case}.graph")), dtype="float16")
+    strip = lambda rows: sorted(((op, scalar, attrs, shape) for op, scalar, attrs, _, shape in rows), key=repr)  # noqa: E731
+    assert strip(_spelling(moved)) == strip(_spelling(cut))
+    split_inputs = lambda g: sorted((g.placeholders.index(n.inputs[0]), n.attrs["dim"]) for n in g.ops if n.op == "split")  # noqa: E731
+    assert split_inputs(moved) == split_inputs(cut) == [(1, 1), (2, 1)]
+
+
+@pytest.mark.parametrize("name", [n for n in AFTER if "invalid" not in n])
+def test_a_joined_pair_computes_what_the_uncut_structure_computes(name):
+    after = _after(name)
+    joined = to_ir(join_cut_pair(*after) if isinstance(after[0], list) else after, dtype="float16")
+    whole = stored(name.replace("after_split", "before_split"))
+    rng = np.random.default_rng(11)
+    values = [rng.standard_normal(p.shape) for p in whole.placeholders]
+    assert [p.shape for p in joined.placeholders] == [p.shape for p in whole.placeholders]
+    got, = interpret(joined, {p.name: v for p, v in zip(joined.placeholders, values)})
+    want, = interpret(whole, {p.name: v for p, v in zip(whole.placeholders, values)})
+    np.testing.assert_allclose(got.reshape(want.shape), want, rtol=1e-12, atol=1e-12)
+
+
+def test_a_pair_whose_halves_do_not_fit_is_refused():
+    partial, combine = _after("after_split_matmul_split_k_graph_structure.graph")
+    with pytest.raises(LoweringRejected, match="hands over"):
+        join_cut_pair(partial, _after("after_split_gqa_graph_structure_valid_1.graph")[1])
+    widened = json.loads(json.dumps(combine))
+    widened[0]["output_tensors"][0]["dim"][2] = 16
+    with pytest.raises(LoweringRejected, match="does not fit"):
+        join_cut_pair(partial, widened)
+
+
+def test_graph_set_takes_cut_pairs_and_uncut_structures_alike():
+    from cleave_amd.pipeline import GraphSet
+    graphs = GraphSet.from_structures(None, [_after("after_split_gqa_graph_structure_valid_2.graph"),
+                                             _after("after_split_gqa_graph_structure_valid_6.graph"),
+                                             json.loads((STRUCT / "before_split_gqa_graph_structure_valid_4.graph").read_text())])
+    assert [g.is_split for g in graphs] == [True, False, True]
+    assert graphs[0].ops.count("matmul") == 2 and all(isinstance(entry, dict) for entry in graphs[0].structure)
