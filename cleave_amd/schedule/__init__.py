@@ -31,7 +31,11 @@ def _candidates(graph, arch):
     if fam == "swiglu":
         return policy.swiglu_candidates(low, role, factor, arch)
     if fam == "matmul_rowsum":
-        return policy.rowsum_candidates(low, role, factor, arch)
+        cands = policy.rowsum_candidates(low, role, factor, arch)
+        if not cands:
+            raise ScheduleRejected("matmul + row sum walks whole column tiles with one set of accumulators: unsplit, K % 64 == 0 "
+                                   f"and N % 16 == 0 (N = {low.problem['N']}, K = {low.problem['K']})")
+        return cands
     if fam == "rowsum":
         return policy.rowsum_only_candidates(low, role, factor, arch)
     if fam == "lora":
@@ -47,9 +51,9 @@ def _candidates(graph, arch):
         many = policy.attn_many_rows_candidates(low, role, factor, arch)
         if low.problem.get("norm_eps") or low.problem.get("linear"):
             if not many:
-                raise ScheduleRejected("QK-norm attention and chained matmuls run on the many-row kernel only: at least "
-                                       "64 query rows per unit, widths in 64-feature panels, keys split into equal ranges "
-                                       "(whole 32-key steps when feature-major)")
+                raise ScheduleRejected("QK-norm attention and chained matmuls run on the many-row kernel only: widths in "
+                                       "64-feature panels up to 256, keys split into equal ranges (whole 32-key steps "
+                                       "when feature-major)")
             return many
         return policy.attn_candidates(low, role, factor, arch) + many
     if fam == "mla":

@@ -241,3 +241,33 @@ def test_dense_prefill_compiles_end_to_end(cache_root):
     args = prog.random_inputs(seed=2)
     np.testing.assert_allclose(kernel(*args).float().cpu().numpy(), program_oracle.evaluate(prog, list(args))[0],
                                rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("rows", [1, 3, 17, 40, 63])
+def test_few_row_units_of_the_operators_that_exist_in_this_kernel_only(rows):
+    """QK-norm attention and the chained matmuls have no streaming (decode) form: with fewer than 64
+    query rows per unit the search still hands them to the LDS-shared kernel (one workgroup per
+    unit, the rest of its 128 rows masked), split over the keys or not."""
+    from cleave_amd.schedule import search_tiling
+
+    def chained(fn, shapes, **how):
+        # first operand scaled and the tolerance following the outputs' magnitude, as in the chained tests above
+        prog = fn.trace(cl.f16, **shapes)
+        first, *rest = prog.random_inputs(seed=7)
+        args = [(first.float() / 8).to(first.dtype), *rest]
+        print(f"few-row chained case {prog.name} {shapes} {how}", flush=True)
+        out = kernel_for(prog, **how)(*args)
+        torch.cuda.synchronize()
+        want = program_oracle.evaluate(prog, args)[0]
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2 + np.abs(want).max() * 2.0 ** -9)
+
+    searched = dict(template=None)
+    for shapes in (dict(HQ=4, HKV=2, SQ=rows, SKV=300, D=128), dict(HQ=2, HKV=2, SQ=rows, SKV=64, D=64)):
+        assert search_tiling(stage_graph(C.qknorm.trace(cl.f16, **shapes)))[0].template == "attn_prefill"
+        _check(C.qknorm, cl.f16, shapes, **searched)
+        _check(C.qknorm, cl.f16, shapes, split=4, **searched)
+    shapes = dict(H=2, SQ=rows, SKV=100, D=64)
+    assert search_tiling(stage_graph(C.matmul_matmul.trace(cl.f16, **shapes)))[0].template == "attn_prefill"
+    chained(C.matmul_matmul, shapes)
+    chained(C.matmul_matmul, shapes, split=4)
+    chained(C.matmul_matmul_2d, dict(M=rows, N=96, K=64))

@@ -128,7 +128,7 @@ def test_qk_norm_attention_is_attention_with_normalised_operands():
     assert (low.problem["units"], low.problem["group"]) == (8, 8)
     assert {c.template for c in search_tiling(g, topk=100)} == {"attn_prefill"}     # the streaming kernel has no norm form
     with pytest.raises(ScheduleRejected, match="many-row kernel"):
-        search_tiling(stage_graph(C.qknorm.trace(cl.f16, HQ=4, HKV=4, SQ=1, SKV=256, D=128)))
+        search_tiling(stage_graph(C.qknorm.trace(cl.f16, HQ=4, HKV=4, SQ=1, SKV=256, D=384)))
     # the first candidate normalises the keys once, by a launch of its own into a scratch copy the attention kernel reads
     m = parse_manifest(source_for(C.qknorm.trace(cl.f16, HQ=64, HKV=8, SQ=4096, SKV=4096, D=128)))
     assert [launch["entry"] for launch in m["launches"]] == ["main_kernel_keys", "main_kernel"]
@@ -313,3 +313,20 @@ def test_codegen_refuses_impossible_plans():
     assert m["launches"][0]["block"] == [512, 1, 1] and m["launches"][0]["grid"][0] == "2"
     with pytest.raises(CodegenError, match="manifest"):
         parse_manifest("__global__ void k() {}")
+
+
+def test_matmul_rowsum_with_a_ragged_column_tile_is_refused_with_its_reason():
+    """One set of accumulators sums every column tile of a row block, so a ragged last tile cannot be masked."""
+    with pytest.raises(ScheduleRejected, match="N % 16 == 0"):
+        search_tiling(stage_graph(C.matmul_rowsum.trace(cl.f16, M=255, N=264, K=128)))
+    assert search_tiling(stage_graph(C.matmul_rowsum.trace(cl.f16, M=255, N=272, K=128)))
+
+
+def test_few_row_units_go_to_the_streaming_kernel_unless_the_operator_has_none():
+    plain = search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=4, HKV=2, SQ=5, SKV=300, D=128)), topk=50)
+    assert {c.template for c in plain} == {"attn_decode"}
+    for fn, shapes in ((C.qknorm, dict(HQ=4, HKV=2, SQ=5, SKV=300, D=128)), (C.matmul_matmul, dict(H=2, SQ=1, SKV=100, D=64))):
+        normed = search_tiling(stage_graph(fn.trace(cl.f16, **shapes)), topk=50)
+        assert normed and {c.template for c in normed} == {"attn_prefill"}
+    with pytest.raises(ScheduleRejected, match="64-feature panels"):
+        search_tiling(stage_graph(C.qknorm.trace(cl.f16, HQ=4, HKV=2, SQ=5, SKV=300, D=384)))
