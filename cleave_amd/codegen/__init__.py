@@ -256,8 +256,8 @@ class HipCodeGen:
         if partial:
             from ..schedule.policy import gemm_lds_bytes
 
-            if p["K"] % (splits * tile["BK"]):
-                raise CodegenError(f"K={p['K']} is not a multiple of splits*BK={splits * tile['BK']}")
+            if p["K"] % (splits * tile["BK"]) and (splits > 1 or p["K"] % 8):
+                raise CodegenError(f"K={p['K']} is neither a multiple of splits*BK={splits * tile['BK']} nor, unsplit, of 8")
             grid = (-(-p["N"] // tile["BN"]), -(-p["M"] // tile["BM"]), batch * splits)
             lds = gemm_lds_bytes(tile["BM"], tile["BN"], tile["BK"], plan.family == "rmsnorm_matmul")
             unit.launch(ENTRY, grid, tile["WM"] * tile["WN"] * 64, lds, self._partial_args)

@@ -8,7 +8,7 @@
 // matrix cores (register-staged; two LDS stages, one barrier per step), and workgroups are
 // renumbered so that each XCD (which owns one L2) works on a compact patch of C.
 //
-//   CL_M CL_N CL_K            problem size per batch entry (K % (CL_SPLITS*CL_BK) == 0)
+//   CL_M CL_N CL_K            problem size per batch entry (K % (CL_SPLITS*CL_BK) == 0, or unsplit with K % 8 == 0)
 //   CL_BM CL_BN CL_BK         workgroup tile;  CL_WM x CL_WN waves, each (BM/WM) x (BN/WN)
 //   CL_TRANS_A / CL_TRANS_B   1 when the operand is stored with K as its major / minor axis
 //                             opposite to the default (A: (M,K), B: (K,N))
@@ -37,20 +37,30 @@ static_assert((GM_TM & (GM_TM - 1)) == 0 && (GM_TN & (GM_TN - 1)) == 0,
 CL_DEVICE int gm_swz(int row) { return ((row >> 1) ^ (row >> 3)) & 7; }
 CL_DEVICE int gm_lds_off(int row, int ch) { return row * GM_LD + ((ch ^ gm_swz(row)) << 3); }
 #define GM_BATCH (CL_BATCH_A > CL_BATCH_B ? CL_BATCH_A : CL_BATCH_B)
+// A contraction length that is not a whole number of BK-wide steps (unsplit, K % 8 == 0): the last
+// step's chunks at or past `k_lim` are fetched from the last valid chunk instead and zeroed on
+// their way to LDS, in both operands.
+#define GM_RAGGED_K ((CL_K / CL_SPLITS) % CL_BK != 0)
+static_assert(!GM_RAGGED_K || (CL_SPLITS == 1 && CL_K % 8 == 0), "a ragged last K step needs an unsplit product and 16-byte rows");
 
 // ---- K-minor operand: rows x BK tile, chunk q -> (row q / KC, chunk q % KC) -------------------
 template <int ROWS>
 struct GmDirect {
   static constexpr int PER = (ROWS * GM_KC + GM_THREADS - 1) / GM_THREADS;
   u32x4 v[PER];
-  CL_METHOD void load(const elem_t* __restrict__ base, i64 pitch, int row0, int row_lim, int k0) {
+  CL_METHOD void load(const elem_t* __restrict__ base, i64 pitch, int row0, int row_lim, int k0, int k_lim) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int q = threadIdx.x + i * GM_THREADS;
       int row = row0 + q / GM_KC;
       row = row < row_lim ? row : row_lim - 1;
-      if (ROWS * GM_KC % GM_THREADS == 0 || q < ROWS * GM_KC)
-        v[i] = ld16(base + (i64)row * pitch + k0 + 8 * (q % GM_KC));
+      int k = k0 + 8 * (q % GM_KC);
+      const bool past = GM_RAGGED_K && k >= k_lim;
+      if (GM_RAGGED_K) k = past ? k_lim - 8 : k;
+      if (ROWS * GM_KC % GM_THREADS == 0 || q < ROWS * GM_KC) {
+        v[i] = ld16(base + (i64)row * pitch + k);
+        if (past) v[i] = (u32x4){0u, 0u, 0u, 0u};
+      }
     }
   }
   CL_METHOD void store(elem_t* lds) const {
@@ -75,16 +85,22 @@ struct GmTransposed {
   static CL_METHOD int cblock(int q) { return NB < 8 ? q % NB : (q & 7) + 8 * (q / (8 * GM_KC)); }
   static CL_METHOD int kblock(int q) { return NB < 8 ? q / NB : (q >> 3) % GM_KC; }
   u32x4 v[PER][8];
-  CL_METHOD void load(const elem_t* __restrict__ base, i64 pitch, int col0, int col_lim, int k0) {
+  CL_METHOD void load(const elem_t* __restrict__ base, i64 pitch, int col0, int col_lim, int k0, int k_lim) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int q = threadIdx.x + i * GM_THREADS;
       if (BLOCKS % GM_THREADS == 0 || q < BLOCKS) {
         int col = col0 + 8 * cblock(q);
         col = col < col_lim - 8 ? col : col_lim - 8;
-        const elem_t* p = base + (i64)(k0 + 8 * kblock(q)) * pitch + col;
+        int k = k0 + 8 * kblock(q);
+        const bool past = GM_RAGGED_K && k >= k_lim;
+        if (GM_RAGGED_K) k = past ? k_lim - 8 : k;
+        const elem_t* p = base + (i64)k * pitch + col;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[i][e] = ld16(p + (i64)e * pitch);
+        for (int e = 0; e < 8; ++e) {
+          v[i][e] = ld16(p + (i64)e * pitch);
+          if (past) v[i][e] = (u32x4){0u, 0u, 0u, 0u};
+        }
       }
     }
   }
@@ -117,16 +133,22 @@ struct GmTransposedHalf {
   static CL_METHOD int kblock(int u) { return (u >> 4) % GM_KC; }
   static CL_METHOD int half(int u) { return (u >> 3) & 1; }
   u32x4 v[PER][4];
-  CL_METHOD void load(const elem_t* __restrict__ base, i64 pitch, int col0, int col_lim, int k0) {
+  CL_METHOD void load(const elem_t* __restrict__ base, i64 pitch, int col0, int col_lim, int k0, int k_lim) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int u = threadIdx.x + i * GM_THREADS;
       if (UNITS % GM_THREADS == 0 || u < UNITS) {
         int col = col0 + 8 * cblock(u);
         col = col < col_lim - 8 ? col : col_lim - 8;
-        const elem_t* p = base + (i64)(k0 + 8 * kblock(u) + 4 * half(u)) * pitch + col;
+        int k = k0 + 8 * kblock(u);
+        const bool past = GM_RAGGED_K && k >= k_lim;
+        if (GM_RAGGED_K) k = past ? k_lim - 8 : k;
+        const elem_t* p = base + (i64)(k + 4 * half(u)) * pitch + col;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[i][e] = ld16(p + (i64)e * pitch);
+        for (int e = 0; e < 4; ++e) {
+          v[i][e] = ld16(p + (i64)e * pitch);
+          if (past) v[i][e] = (u32x4){0u, 0u, 0u, 0u};
+        }
       }
     }
   }
@@ -207,7 +229,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int batch = blockIdx.z / CL_SPLITS, split = blockIdx.z % CL_SPLITS;
   constexpr int k_per_split = CL_K / CL_SPLITS;
   const int k_begin = split * k_per_split;
-  constexpr int KT = k_per_split / CL_BK;
+  constexpr int KT = (k_per_split + CL_BK - 1) / CL_BK;
+  const int k_lim = k_begin + k_per_split;
 
   const elem_t* A = CL_ARG_A + (i64)(batch / (GM_BATCH / CL_BATCH_A)) * CL_M * CL_K;
   const elem_t* B = CL_ARG_B + (i64)(batch / (GM_BATCH / CL_BATCH_B)) * CL_K * CL_N;
@@ -224,17 +247,17 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 
 #if CL_TRANS_A
   typedef GM_TRANSPOSED(CL_BM) LoaderA;
-#define GM_LOAD_A(set, kk) set.load(A, CL_M, m0, CL_M, (kk))
+#define GM_LOAD_A(set, kk) set.load(A, CL_M, m0, CL_M, (kk), k_lim)
 #else
   typedef GmDirect<CL_BM> LoaderA;
-#define GM_LOAD_A(set, kk) set.load(A, CL_K, m0, CL_M, (kk))
+#define GM_LOAD_A(set, kk) set.load(A, CL_K, m0, CL_M, (kk), k_lim)
 #endif
 #if CL_TRANS_B
   typedef GmDirect<CL_BN> LoaderB;
-#define GM_LOAD_B(set, kk) set.load(B, CL_K, n0, CL_N, (kk))
+#define GM_LOAD_B(set, kk) set.load(B, CL_K, n0, CL_N, (kk), k_lim)
 #else
   typedef GM_TRANSPOSED(CL_BN) LoaderB;
-#define GM_LOAD_B(set, kk) set.load(B, CL_N, n0, CL_N, (kk))
+#define GM_LOAD_B(set, kk) set.load(B, CL_N, n0, CL_N, (kk), k_lim)
 #endif
   LoaderA la0;
   LoaderB lb0;
@@ -270,7 +293,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GM_GAMMA_A(kk)                                                                              \
   {                                                                                                 \
     const int q = threadIdx.x + i * GM_THREADS;                                                     \
-    elem8 gm = as_elem8(ld16(CL_ARG_GAMMA + (kk) + 8 * (q % GM_KC)));                               \
+    int gk = (kk) + 8 * (q % GM_KC);                                                                \
+    gk = gk < CL_K - 8 ? gk : CL_K - 8;          /* (a chunk past K is zero already) */             \
+    elem8 gm = as_elem8(ld16(CL_ARG_GAMMA + gk));                                                   \
     _Pragma("unroll") for (int e = 0; e < 8; ++e) x[e] = to_elem(to_f32(x[e]) * to_f32(gm[e]));    \
   }
 #else

@@ -27,6 +27,11 @@ def _candidates(graph, arch):
         if not (fam == "rmsnorm_matmul" and low.problem["trans_A"]):
             cands += policy.gemm_candidates(low, role, factor, arch)
         cands += policy.gemm_dma_candidates(low, role, factor, arch)
+        if not cands:
+            p = low.problem
+            raise ScheduleRejected("the matmul kernels move 16-byte chunks: K % 8 == 0 (K % 64 == 0 per split when split), and the "
+                                   f"extent along which each operand is contiguous a multiple of 8 (M = {p['M']}, N = {p['N']}, "
+                                   f"K = {p['K']}, split = {factor or 1})")
         return cands
     if fam == "swiglu":
         return policy.swiglu_candidates(low, role, factor, arch)

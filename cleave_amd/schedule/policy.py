@@ -55,7 +55,9 @@ def gemm_candidates(low, role, factor, arch: Arch):
     shapes = (16, 32, 64, 128, 256)
     for bm, bn, bk, (wm, wn), depth in itertools.product(
             shapes, shapes, (64,), ((1, 1), (1, 2), (2, 1), (2, 2), (1, 4), (4, 1), (2, 4), (4, 2)), (1, 2)):
-        if bm % (16 * wm) or bn % (16 * wn) or kps % bk:
+        if bm % (16 * wm) or bn % (16 * wn):
+            continue
+        if kps % bk and (splits > 1 or K % 8):       # a ragged last step: unsplit, rows of whole 16-byte chunks
             continue
         if bm > max(16, 2 * M) or bn > max(16, 2 * N):
             continue
@@ -89,7 +91,7 @@ def gemm_candidates(low, role, factor, arch: Arch):
         per_cu = arch.blocks_per_cu(threads, lds, vgprs)
         if per_cu < 1:
             continue
-        if depth == 2 and (kps // bk < 4 or per_cu * threads > 512 and vgprs > 128):
+        if depth == 2 and (_ceil(kps, bk) < 4 or per_cu * threads > 512 and vgprs > 128):
             continue
         passes = _waves_time(blocks, per_cu, arch)
         live = min(per_cu, _ceil(blocks, arch.compute_units))         # blocks a CU really holds
@@ -98,7 +100,7 @@ def gemm_candidates(low, role, factor, arch: Arch):
         mfma_clk = live * (bm * bn * kps * 2) / 4096.0 / min(1.0, live * wm * wn / 8.0)
         l1_clk = live * ((bm + bn) * kps * 2) / (24.0 * (1.6 if depth == 2 else 1.0))
         lds_clk = live * (tm + tn) * 16 * wm * wn * kps * 2 / 256.0
-        pass_clk = max(mfma_clk, l1_clk, lds_clk) + 2500 + 1200 * (kps // bk) / max(1, min(live, 2))
+        pass_clk = max(mfma_clk, l1_clk, lds_clk) + 2500 + 1200 * _ceil(kps, bk) / max(1, min(live, 2))
         score = passes * pass_clk
         # (where the direct-to-LDS kernel offers the same tile it has measured a quarter to two thirds
         # faster -- 2048 x 4096 x 4096 on 128 x 128 tiles: 67 against 91 us; 512 x 512 x 4096 on 16 x 32 tiles:

@@ -402,3 +402,32 @@ def test_graph_replay_timer_matches_eager_results_and_time():
         assert torch.equal(kernel.last_timed_outputs[0], want)
         assert torch.equal(kernel(*args), want)            # eager work between the replays
     assert all(0 < t < 5 * eager_ms for t in times) and min(times) < 1.5 * eager_ms
+
+
+@pytest.mark.parametrize("k", [8, 40, 72, 96, 200, 1000, 4104])
+def test_matmul_with_a_ragged_last_k_step(k):
+    """K a multiple of 8 but not of the 64-wide step: the register-staged kernel zeroes the chunks
+    past K on their way to LDS.  Row-major and both transposed layouts (each loader form), both
+    prefetch depths, tiles with whole and half transposed blocks, the searched best plan, a batched
+    product and the fused RMSNorm (with and without the learned weight)."""
+    fn, dt, mk = C.CASES["c1"]
+    shapes = dict(M=100, N=136, K=k)
+    for tiling in (dict(BM=32, BN=32, BK=64, WM=1, WN=1), dict(BM=64, BN=64, BK=64, WM=2, WN=2, GDEPTH=2),
+                   dict(BM=16, BN=128, BK=64, WM=1, WN=4)):
+        _check(fn.trace(dt, **shapes), mk, shapes, template="gemm", tiling=tiling)
+    _check(fn.trace(dt, **shapes), mk, shapes)
+    g = torch.Generator(device="cpu").manual_seed(k)
+    for prog, dims in ((matmul_nt.trace(cl.f16, **shapes), ((100, k), (136, k))), (matmul_tn.trace(cl.bf16, **shapes), ((k, 104), (k, 136)))):
+        if prog.name == "matmul_tn":
+            prog = matmul_tn.trace(cl.bf16, M=104, N=136, K=k)
+        ins = [((torch.rand(*shp, generator=g) * 2 - 1) / k ** 0.5).to(torch.bfloat16 if prog.name == "matmul_tn" else torch.float16)
+               for shp in dims]
+        want = po.evaluate(prog, ins)[0]
+        print(f"case {prog.name} ragged K={k}", flush=True)
+        got = kernel_for(prog, template="gemm", tiling=dict(BM=64, BN=64, BK=64, WM=2, WN=2))(*[t.cuda() for t in ins])
+        np.testing.assert_allclose(got.float().cpu().numpy().reshape(want.shape), want, rtol=RTOL, atol=ATOL)
+    bshapes = dict(BX=4, BW=2, M=70, N=64, K=k)
+    _check(C.batched_matmul.trace(cl.f16, **bshapes), C.inputs_batched, bshapes)
+    nshapes = dict(M=130, N=72, K=k)
+    _check(C.rmsnorm_matmul.trace(cl.f16, **nshapes), C.inputs_c2, nshapes)
+    _check(C.rmsnorm_matmul_eps.trace(cl.f16, **nshapes), C.inputs_plain_norm, nshapes)

@@ -330,3 +330,21 @@ def test_few_row_units_go_to_the_streaming_kernel_unless_the_operator_has_none()
         assert normed and {c.template for c in normed} == {"attn_prefill"}
     with pytest.raises(ScheduleRejected, match="64-feature panels"):
         search_tiling(stage_graph(C.qknorm.trace(cl.f16, HQ=4, HKV=2, SQ=5, SKV=300, D=384)))
+
+
+def test_contraction_lengths_off_the_64_wide_step():
+    """K % 8 == 0 is enough unsplit (the register-staged kernel zeroes the last step's tail); a split wants
+    whole steps per range; anything else is refused with the alignment rule."""
+    for k in (8, 40, 96, 4104):
+        cands = search_tiling(stage_graph(C.matmul.trace(cl.f16, M=100, N=64, K=k)), topk=100)
+        assert cands and {c.template for c in cands} == {"gemm"}
+    whole = search_tiling(stage_graph(C.matmul.trace(cl.f16, M=100, N=64, K=128)), topk=200)
+    assert {"gemm", "gemm_dma"} <= {c.template for c in whole}
+    part = split_stages(stage_graph(C.matmul.trace(cl.f16, M=100, N=64, K=192)), 2)[0]
+    with pytest.raises(ScheduleRejected, match="16-byte chunks"):
+        search_tiling(part)
+    for shapes in (dict(M=100, N=64, K=100), dict(M=100, N=60, K=64)):
+        with pytest.raises(ScheduleRejected, match="16-byte chunks"):
+            search_tiling(stage_graph(C.matmul.trace(cl.f16, **shapes)))
+    with pytest.raises(CodegenError, match="nor, unsplit, of 8"):
+        source_for(C.matmul.trace(cl.f16, M=100, N=64, K=100), template="gemm", tiling=dict(BM=32, BN=32, BK=64, WM=1, WN=1))
