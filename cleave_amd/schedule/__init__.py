@@ -34,7 +34,11 @@ def _candidates(graph, arch):
                                    f"K = {p['K']}, split = {factor or 1})")
         return cands
     if fam == "swiglu":
-        return policy.swiglu_candidates(low, role, factor, arch)
+        cands = policy.swiglu_candidates(low, role, factor, arch)
+        if not cands:
+            raise ScheduleRejected("SwiGLU runs on the direct-to-LDS matmul, unsplit: K % 64 == 0 and N a multiple of half a "
+                                   f"column tile (N % 16 == 0; N = {low.problem['N']}, K = {low.problem['K']})")
+        return cands
     if fam == "matmul_rowsum":
         cands = policy.rowsum_candidates(low, role, factor, arch)
         if not cands:
@@ -42,7 +46,10 @@ def _candidates(graph, arch):
                                    f"and N % 16 == 0 (N = {low.problem['N']}, K = {low.problem['K']})")
         return cands
     if fam == "rowsum":
-        return policy.rowsum_only_candidates(low, role, factor, arch)
+        cands = policy.rowsum_only_candidates(low, role, factor, arch)
+        if not cands:
+            raise ScheduleRejected(f"row reductions read 16-byte chunks, unsplit: N % 8 == 0 (N = {low.problem['N']})")
+        return cands
     if fam == "lora":
         cands = policy.lora_candidates(low, role, factor, arch)
         if not cands:
@@ -50,9 +57,8 @@ def _candidates(graph, arch):
                                    "(N % 256 == 0 when split), rank a multiple of 8 up to 64")
         return cands
     if fam == "attention":
-        if not policy.attn_ok(low):
-            raise ScheduleRejected(f"decode attention template needs head_dim % 32 == 0 and a value width of 64 or "
-                                   f"a multiple of 128, got {low.problem['head_dim']}/{low.problem['vdim']}")
+        # the LDS-shared many-row kernel takes widths in 64-feature panels up to 256; the streaming kernel
+        # head_dim % 32 == 0 with a value width of 64 or a multiple of 128
         many = policy.attn_many_rows_candidates(low, role, factor, arch)
         if low.problem.get("norm_eps") or low.problem.get("linear"):
             if not many:
@@ -60,7 +66,14 @@ def _candidates(graph, arch):
                                        "64-feature panels up to 256, keys split into equal ranges (whole 32-key steps "
                                        "when feature-major)")
             return many
-        return policy.attn_candidates(low, role, factor, arch) + many
+        cands = (policy.attn_candidates(low, role, factor, arch) if policy.attn_ok(low) else []) + many
+        if not cands:
+            raise ScheduleRejected(f"no attention kernel for key/value widths {low.problem['head_dim']}/{low.problem['vdim']} "
+                                   f"with {low.problem['group'] * low.problem['sq']} query rows per unit: the streaming "
+                                   "(decode) kernel needs head_dim % 32 == 0 and a value width of 64 or a multiple of 128 "
+                                   "that fits its registers, the many-row kernel at least 64 rows and widths that are "
+                                   "multiples of 64 up to 256")
+        return cands
     if fam == "mla":
         if not policy.mla_ok(low):
             raise ScheduleRejected("MLA template needs heads % 16 == 0 and widths that are multiples of 32")

@@ -271,3 +271,15 @@ def test_few_row_units_of_the_operators_that_exist_in_this_kernel_only(rows):
     chained(C.matmul_matmul, shapes)
     chained(C.matmul_matmul, shapes, split=4)
     chained(C.matmul_matmul_2d, dict(M=rows, N=96, K=64))
+
+
+def test_widths_only_the_many_row_kernel_takes():
+    """192-wide keys and values: the streaming kernel has no form for a 192-wide value (64 or a
+    multiple of 128), the LDS-shared kernel works in 64-feature panels; the search hands it over."""
+    from cleave_amd.schedule import search_tiling
+
+    shapes = dict(HQ=4, HKV=2, SQ=100, SKV=300, D=192)
+    assert {c.template for c in search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, **shapes)))} == {"attn_prefill"}
+    _check(C.gqa_decode_exact, cl.f16, shapes, template=None)
+    _check(C.gqa_decode_exact, cl.bf16, dict(HQ=2, HKV=2, SQ=64, SKV=512, D=192), template=None, split=4)
+    _check(C.gqa_decode_shift, cl.f16, dict(HQ=8, HKV=1, SQ=70, SKV=77, D=192), template=None)
