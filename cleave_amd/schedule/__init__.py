@@ -71,8 +71,7 @@ def _candidates(graph, arch):
             raise ScheduleRejected(f"no attention kernel for key/value widths {low.problem['head_dim']}/{low.problem['vdim']} "
                                    f"with {low.problem['group'] * low.problem['sq']} query rows per unit: the streaming "
                                    "(decode) kernel needs head_dim % 32 == 0 and a value width of 64 or a multiple of 128 "
-                                   "that fits its registers, the many-row kernel at least 64 rows and widths that are "
-                                   "multiples of 64 up to 256")
+                                   "that fits its registers, the many-row kernel widths that are multiples of 64 up to 256")
         return cands
     if fam == "mla":
         if not policy.mla_ok(low):

@@ -400,10 +400,10 @@ def attn_many_rows_candidates(low, role, factor, arch: Arch):
     rows, d = p["group"] * p["sq"], p["head_dim"]
     vd = p["vdim"]
     splits = factor or 1
-    # plain softmax attention with few rows per unit belongs to the streaming decode kernel; QK-norm and
-    # the chained matmul exist in this kernel only, so there it takes units of any height (one
-    # workgroup per unit, most of its 128 rows masked)
-    only_here = bool(p.get("norm_eps") or p.get("linear"))
+    # plain softmax attention with few rows per unit belongs to the streaming decode kernel; QK-norm, the
+    # chained matmul and widths the streaming kernel has no form for (a 192-wide value) exist in this
+    # kernel only, so there it takes units of any height (one workgroup per unit, most of its 128 rows masked)
+    only_here = bool(p.get("norm_eps") or p.get("linear")) or not attn_ok(low)
     if (rows < 64 and not only_here) or d % 64 or d > 256 or vd % 64 or vd > 256 or p["skv"] < 1:
         return []
     if splits > 1 and p.get("emit_lse"):

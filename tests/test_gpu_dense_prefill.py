@@ -283,3 +283,6 @@ def test_widths_only_the_many_row_kernel_takes():
     _check(C.gqa_decode_exact, cl.f16, shapes, template=None)
     _check(C.gqa_decode_exact, cl.bf16, dict(HQ=2, HKV=2, SQ=64, SKV=512, D=192), template=None, split=4)
     _check(C.gqa_decode_shift, cl.f16, dict(HQ=8, HKV=1, SQ=70, SKV=77, D=192), template=None)
+    # decode-shaped units of that width have no other kernel either
+    _check(C.gqa_decode_exact, cl.f16, dict(HQ=8, HKV=2, SQ=1, SKV=1000, D=192), template=None)
+    _check(C.gqa_decode_exact, cl.f16, dict(HQ=8, HKV=2, SQ=3, SKV=1024, D=192), template=None, split=8)

@@ -354,9 +354,10 @@ def test_searches_that_find_nothing_say_why():
     for prog, reason in ((C.swiglu.trace(cl.f16, M=100, N=72, K=128), "N % 16 == 0"),
                          (C.swiglu.trace(cl.f16, M=100, N=128, K=96), "K % 64 == 0"),
                          (C.rowsum.trace(cl.f16, M=100, N=100), "N % 8 == 0"),
-                         (C.gqa_decode_exact.trace(cl.f16, HQ=8, HKV=2, SQ=1, SKV=1000, D=192), "192/192 with 4 query rows"),
+                         (C.gqa_decode_exact.trace(cl.f16, HQ=8, HKV=2, SQ=1, SKV=1000, D=160), "160/160 with 4 query rows"),
                          (C.gqa_decode_exact.trace(cl.f16, HQ=8, HKV=2, SQ=512, SKV=1000, D=96), "multiples of 64 up to 256")):
         with pytest.raises(ScheduleRejected, match=reason):
             search_tiling(stage_graph(prog))
-    wide = search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=8, HKV=2, SQ=512, SKV=1000, D=192)))
-    assert wide and {c.template for c in wide} == {"attn_prefill"}
+    for rows in (512, 1):
+        wide = search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=8, HKV=2, SQ=rows, SKV=1000, D=192)))
+        assert wide and {c.template for c in wide} == {"attn_prefill"}
