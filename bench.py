@@ -11,11 +11,12 @@ partial + combine pair) on one set of seeded synthetic inputs already resident i
 rotate through several independent input sets so a working set smaller than the 256 MB
 last-level cache cannot be served from it.
 
-One JSON line is printed.  ``value`` is the best-candidate latency in microseconds of the
-headline workload (fused RMSNorm->matmul at the decode shape M=16, K=4096, N=11008, fp16);
-``ops`` carries the same figures for every other operator (the first one named is the headline
-and fails the run if it fails; any other that fails is listed with its error), the registry's
-paged operators last (``dyn``: geomean over their captured workloads).  ``roofline`` prices the dominant
+One JSON line of under 4 KB is printed.  ``value`` is the best-candidate latency in microseconds
+of the headline workload (fused RMSNorm->matmul at the decode shape M=16, K=4096, N=11008, fp16);
+``ops`` carries one compact row per operator (the first one named is the headline and fails
+the run if it fails; any other that fails is listed with its error), the registry's paged
+operators last (``dyn``: geomean over their captured workloads).  Every operator's full record
+(plan, probes, per-workload tables) goes to the file named by ``--full``.  ``roofline`` prices the dominant
 kernel of the headline workload: algorithmic bytes per launch over its mean duration from
 HIP events on the launch stream, against the published 8 TB/s.  ``cpu_baseline`` is the numpy
 port of the reference's CPU evaluation of the same program, timed on this host.
@@ -561,6 +562,49 @@ def run_stream_probe(mib=2048, steps=10, warmup=3):
     return best
 
 
+# ----------------------------------------------------------------------------- the one stdout line
+LINE_LIMIT = 4096      # bytes; the harness that runs this file keeps only the tail of stdout
+
+
+def compact(rec):
+    """What the stdout line says of one operator: its name, whole-op and dominant-kernel latency and the
+    fraction of the roofline that bounds it.  Plans, probes, per-workload tables and the reference's H100
+    figures are in the full record (stderr, and the file named by --full)."""
+    if "error" in rec:
+        return {"op": rec["op"], "error": rec["error"][:80]}
+    if "operators" in rec:          # the registry's paged operators: geomean over their captured workloads
+        return {"op": rec["op"], "geomean_us": {r["op"]: r["geomean_us"] for r in rec["operators"]}}
+    return {"op": rec["op"], "best_us": rec["best_us"], "dominant_kernel_us": rec["dominant_kernel_us"],
+            "frac": rec["roofline"]["frac"], "bound": rec["roofline"]["bound"]}
+
+
+def final_line(results, wanted, steps, warmup, cpu_threads):
+    """The JSON object printed on stdout: headline keys of the first timed operator (C2 when it ran), its
+    roofline and CPU baseline, and a compact row per operator.  Kept under LINE_LIMIT bytes whatever ran."""
+    timed = [n for n in wanted if "best_us" in results[n]]
+    if not timed:
+        return {"metric": "registry paged operators: geomean us over their captured workloads", "n_gpus": 1,
+                "dtype": "bf16", "data": "synthetic", "ops": [compact(results[n]) for n in wanted]}
+    head = results["c2"] if "c2" in results and "best_us" in results["c2"] else results[timed[0]]
+    roof = {k: head["roofline"].get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+    line = {
+        "metric": "best-candidate us and % HBM/MFMA roofline per op on 1 MI355X vs CPU ref",
+        "value": head["best_us"], "unit": "us", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(head["best_us"] / 1e3, 6), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": head["workload"], "variant": head.get("variant"), "plan": (head.get("plan") or "")[:160]},
+        "roofline": roof,
+        "cpu_baseline": None if cpu_threads is None else {
+            "value": head.get("cpu_us"), "unit": "us", "cores": cpu_threads, "kind": "port",
+            "sample": head.get("cpu_sample")},
+        "ops": [compact(results[n]) for n in wanted],
+    }
+    if len(json.dumps(line)) >= LINE_LIMIT:        # never let the record grow past what the harness keeps
+        line["ops"] = [{"op": r["op"], "frac": r.get("frac")} if "frac" in r else {"op": r["op"]} for r in line["ops"]]
+    return line
+
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -573,6 +617,9 @@ def main():
     ap.add_argument("--kernels", default=None, metavar="DIR",
                     help="save each op's selected kernel source under DIR; when DIR already holds one, time it "
                          "without searching (so a profiler sees only the timed launches)")
+    ap.add_argument("--full", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"), metavar="FILE",
+                    help="where every operator's full record goes (plans, probes, per-workload tables, the "
+                         "reference's H100 figures); stdout carries the compact line only")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU form (its units are independent per "
@@ -625,25 +672,18 @@ def main():
         except Exception as failure:  # noqa: BLE001 - reported in the line, not swallowed
             log(f"[{name}] FAILED: {type(failure).__name__}: {str(failure)[:300]}")
             results[name] = {"op": name, "error": f"{type(failure).__name__}: {str(failure)[:300]}"}
-    # the headline workload unless left out; failing that the first operator that has a latency
-    timed = [n for n in wanted if "best_us" in results[n]]
-    if not timed:
-        print(json.dumps({"metric": "registry paged operators: geomean us over their captured workloads", "n_gpus": 1,
-                          "dtype": "bf16", "data": "synthetic", "ops": [results[n] for n in wanted]}))
-        return
-    head = results["c2"] if "c2" in results else results[timed[0]]
-    line = {
-        "metric": "best-candidate us and % HBM/MFMA roofline per op on 1 MI355X vs CPU ref",
-        "value": head["best_us"], "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(head["best_us"] / 1e3, 6), "higher_is_better": False, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": head["workload"], "variant": head["variant"], "plan": head["plan"]},
-        "roofline": head["roofline"],
-        "cpu_baseline": None if args.no_cpu else {
-            "value": head.get("cpu_us"), "unit": "us", "cores": min(threads, cores), "kind": "port",
-            "sample": head.get("cpu_sample")},
-        "ops": [results[n] for n in wanted],
-    }
+    threads = min(threads, cores)
+    full = {"probes": {"stream_gbps": STREAM_GBPS, "matrix_tflops": MATRIX_TFLOPS}, "ops": [results[n] for n in wanted]}
+    try:
+        os.makedirs(os.path.dirname(os.path.abspath(args.full)), exist_ok=True)
+        with open(args.full, "w") as f:
+            json.dump(full, f, indent=1)
+        log(f"[full] every operator's full record: {args.full}")
+    except OSError as e:                       # a read-only tree must not cost the run its line
+        log(f"[full] not written ({e}); full record follows\n" + json.dumps(full))
+    line = final_line(results, wanted, args.steps, args.warmup, None if args.no_cpu else threads)
+    for row in line["ops"]:                    # the same rows as a table at the end of stderr
+        log("[row] " + " ".join(f"{k}={v}" for k, v in row.items() if k != "geomean_us"))
     print(json.dumps(line))
 
 
