@@ -106,6 +106,10 @@ class HipCodeGen:
         emit = getattr(self, f"_emit_{plan.template}", None)
         if emit is None:
             raise CodegenError(f"no template named {plan.template!r}")
+        probes = sorted(k for k in (plan.tiling or {}) if str(k).startswith("DBG_"))
+        if probes:
+            # (the shipped templates hold no measurement switches: a key that asks for one would be ignored)
+            raise CodegenError(f"tiling keys {probes} name measurement switches, which the templates do not have")
         splits = plan.split_factor or 1
         if plan.role == "main" and splits != 1:
             raise CodegenError("a main kernel cannot carry a split factor")
@@ -444,9 +448,6 @@ class HipCodeGen:
         unit.define("CL_ROWS", rows)
         unit.define("CL_WAVES", waves)
         unit.define("CL_PREFETCH", int(t.get("PREFETCH", 1)))
-        for k in t:
-            if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
-                unit.define(f"CL_{k}", 1)
         chunk_pages = bool(t.get("CHUNK_PAGES", 0)) and paged and (plan.split_factor or 1) > 1
         unit.define("CL_CHUNK_PAGES", chunk_pages)
         unit.define("CL_PAGED", paged)
@@ -601,9 +602,6 @@ class HipCodeGen:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
         if "OCC" in t:
             unit.define("CL_OCC", int(t["OCC"]))
-        for k in t:
-            if k.startswith("DBG_"):
-                unit.define(f"CL_{k}", 1)
         # split partials of this family are stored in the element type (normalised per split)
         unit.define("CL_PO_ELEM", 1)
         unit.define("CL_SCALE_LOG2E", _f(float(p["scale"]) * LOG2E))
@@ -650,9 +648,6 @@ class HipCodeGen:
             if not 0 <= int(t["S_PANELS"]) < (p["ckv"] + p["kpe"]) // 64:
                 raise CodegenError("S_PANELS: the score waves can load between none and all but one of a step's 64-feature panels")
             unit.define("CL_S_PANELS", int(t["S_PANELS"]))
-        for k in t:
-            if k.startswith("DBG_"):          # measurement switches of the template (wrong results by design)
-                unit.define(f"CL_{k}", 1)
         unit.define("CL_SCALE_LOG2E", _f(float(p["scale"]) * LOG2E))
         for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE")):
             if role in op:

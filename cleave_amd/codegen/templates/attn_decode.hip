@@ -113,23 +113,10 @@ CL_DEVICE int att_clamp_ptr(int p, int n_idx) { return p < 0 ? 0 : (p > n_idx ? 
 #endif
 
 #if CL_EMIT_PARTIAL
-#ifdef CL_DBG_TIME
-// measurement switch (the result is wrong by design): every wave stamps the shader clock (slots
-// 0, 2, 3, 4) and the 100 MHz wall clock (1, 5) into the first bytes of the Q operand
-#define ATT_MARK(k) do { const unsigned long long t_ = (k) == 1 || (k) == 5 ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); \
-    __builtin_amdgcn_sched_barrier(0); if (lane == 0) att_stamps[k] = t_; } while (0)
-#else
-#define ATT_MARK(k)
-#endif
 extern "C" __global__ void __launch_bounds__(CL_WAVES * 64)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
-#ifdef CL_DBG_TIME
-  unsigned long long att_stamps[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
-  ATT_MARK(0);
-  ATT_MARK(1);
 #if CL_CHUNK_PAGES
   const int split = 0, tile_id = 0;
   const int item = blockIdx.x;
@@ -281,10 +268,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       att_load(u, sidx * ATT_STEP, c, g, ring[i]);
     }
   }
-#ifdef CL_DBG_TIME
-  asm volatile("" :: "v"(qf[0]));
-#endif
-  ATT_MARK(2);
   for (int base = step0; base < step_end; base += (CL_PREFETCH + 1) * ATT_WSTRIDE) {
 #pragma unroll
     for (int r = 0; r <= CL_PREFETCH; ++r) {
@@ -355,10 +338,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
   }
 
-#ifdef CL_DBG_TIME
-  asm volatile("" :: "v"(acc[0][0]));
-#endif
-  ATT_MARK(3);
   // ---- merge the workgroup's waves through LDS ----------------------------------------------
   l_run += lane_xor(l_run, lane, 16);
   l_run += lane_xor(l_run, lane, 32);
@@ -426,16 +405,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
   }
 #endif  // CL_CHUNK_PAGES
-#ifdef CL_DBG_TIME
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  ATT_MARK(4);
-  ATT_MARK(5);
-  if (lane == 0) {
-    unsigned long long* dump = (unsigned long long*)CL_ARG_Q + ((blockIdx.y * gridDim.x + blockIdx.x) * CL_WAVES + wave) * 8;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) dump[k] = att_stamps[k];
-  }
-#endif
 }
 #endif  // CL_EMIT_PARTIAL
 

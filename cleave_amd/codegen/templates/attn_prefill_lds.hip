@@ -52,19 +52,11 @@
 // registers); the lanes on the diagonal take the reciprocal root and the lanes of each score
 // fetch the factor of its key.
 //
-// CL_PF_XCD / CL_PF_REVERSE (default 1) switch the XCD mapping and the walking order; the
-// CL_PF_DBG_* switches leave parts of the kernel out for measurement (wrong results by design).
+// CL_PF_XCD / CL_PF_REVERSE (default 1) switch the XCD mapping and the walking order.
 //
 //   CL_HEAD_DIM (multiple of 64)  CL_KV_HEADS  CL_Q_HEADS (group divides 16)  CL_RAGGED
 //   run-time: batch, total_q, n_idx (table length / total_kv), num_pages (table form), sm_scale
 
-#if CL_PF_DBG_TIME
-// measurement switch (the result is wrong by design): every wave keeps the shader clock at its
-// marks, the clocks it spent waiting at the step barriers and between them, and the 100 MHz wall
-// clock at both ends, and leaves the eight numbers in the first bytes of Q
-#define PL_CLOCK() __builtin_amdgcn_s_memtime()
-#define PL_WALL() __builtin_amdgcn_s_memrealtime()
-#endif
 #ifndef CL_PF_XCD
 #define CL_PF_XCD 1
 #endif
@@ -176,10 +168,6 @@ extern "C" __global__ void __launch_bounds__(256, 2)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
-#if CL_PF_DBG_TIME
-  const unsigned long long pl_t_entry = PL_CLOCK(), pl_w_entry = PL_WALL();
-  unsigned long long pl_t_loop = 0, pl_t_prev = 0, pl_sync = 0, pl_work = 0;
-#endif
   // Workgroups go to the 8 XCDs round-robin in launch order; every XCD has its own L2.  XCD x
   // takes the x-th eighth of the (kv head, item) space (the item axis is padded to a multiple of
   // 8), so the workgroups resident on an XCD are neighbouring items of one kv head and re-read
@@ -301,11 +289,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const char* kbase = reinterpret_cast<const char*>(CL_ARG_K) + (i64)head * CL_HEAD_DIM * 2;
   const char* vbase = reinterpret_cast<const char*>(CL_ARG_V) + (i64)head * CL_VDIM * 2;
 #endif
-#if CL_PF_DBG_ONESTEP
-  const int n_steps = 1;
-#else
   const int n_steps = (ext + PL_STEP - 1) / PL_STEP;
-#endif
   const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)pl_tiles;
 
   // This wave's share of step s (clamped onto the last step: a step past the end reloads the last
@@ -391,11 +375,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     const elem_t* row = CL_ARG_Q + orow[rt] * CL_HEAD_DIM + 8 * g;
 #pragma unroll
     for (int j = 0; j < PL_KJ; ++j) {
-#if CL_PF_DBG_NOQ
-      u32x4 raw = (u32x4){(unsigned)lane, 0x3c003c00u, (unsigned)j, 0x3c003c00u};
-#else
       u32x4 raw = ld16(row + 32 * j);
-#endif
       if (!live[rt]) raw = (u32x4){0u, 0u, 0u, 0u};
       qf[rt][j] = as_elem8(raw ^ q_sign);
     }
@@ -533,20 +513,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // the images of step + 1 have landed when at most the loads of step + 2 are outstanding; the
     // barrier makes that everybody's share and frees the stage step - 1 has left, which the
     // loads of step + 3 fill
-#if CL_PF_DBG_TIME
-    const unsigned long long pl_t0 = PL_CLOCK();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     PL_WAITCNT(PL_UNITS_PER);
     __syncthreads();
-#if CL_PF_DBG_TIME
-    __builtin_amdgcn_sched_barrier(0);
-    const unsigned long long pl_t1 = PL_CLOCK();
-    pl_sync += pl_t1 - pl_t0;
-    if (pl_t_prev) pl_work += pl_t0 - pl_t_prev; else pl_t_loop = pl_t0;
-    pl_t_prev = pl_t1;
-    __builtin_amdgcn_sched_barrier(0);
-#endif
 #if CL_RAGGED
     const int row_ahead = row_of(step + 3);
 #else
@@ -554,11 +522,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     const int row_ahead = fetched_row(step + 3);
     fetch_id(step + 4);
 #endif
-#if CL_PF_DBG_NOLOADS
-#define PL_ISSUE(place)
-#else
 #define PL_ISSUE(place) issue_quarter(row_ahead, (SLOT + 3) % PL_STAGES, PlC<place>{})
-#endif
     PL_ISSUE(0);
 
     // operands of this body's matrix work: K of step + 1, V of step (8 + 16 LDS reads)
@@ -717,9 +681,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
   // no load may still be on its way into LDS when the workgroup ends
   PL_WAITCNT(0);
-#if CL_PF_DBG_TIME
-  const unsigned long long pl_t_done = PL_CLOCK();
-#endif
 
   // ---- each lane writes its rows' features (a row that saw no key: 0 and lse -inf) --------------
   // (row coordinates are worked out again from the lane number, behind a barrier for the
@@ -738,9 +699,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
     const int m = 32 * wave + 16 * rt + c_e;
     if (m >= n_rows) continue;
-#if CL_PF_DBG_NOSTORE
-    if (l != 12345.f) continue;
-#endif
 #if CL_LINEAR
     const float inv = 1.0f;
 #else
@@ -790,16 +748,5 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
 #endif
   }
-#if CL_PF_DBG_TIME
-  {
-    const unsigned long long pl_t_end = PL_CLOCK(), pl_w_end = PL_WALL();
-    if (lane == 0) {
-      unsigned long long* dump = (unsigned long long*)CL_ARG_Q +
-          ((((unsigned long long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 4 + wave) * 8;
-      dump[0] = pl_t_entry; dump[1] = pl_w_entry; dump[2] = pl_t_loop; dump[3] = pl_sync;
-      dump[4] = pl_work; dump[5] = pl_t_done; dump[6] = pl_t_end; dump[7] = pl_w_end;
-    }
-  }
-#endif
 }
 #endif  // CL_EMIT_PARTIAL

@@ -353,37 +353,22 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       old_a.store(As + ((cur) ^ 1) * A_STAGE);                    \
       old_b.store(Bs + ((cur) ^ 1) * B_STAGE);                    \
     }
-#ifdef CL_DBG_NOLOAD
-#define GM_DBG_LOAD(x)
-#else
-#define GM_DBG_LOAD(x) x
-#endif
-#ifdef CL_DBG_NOSTORE
-#define GM_DBG_STORE(x)
-#else
-#define GM_DBG_STORE(x) x
-#endif
-#ifdef CL_DBG_NOCOMPUTE
-#define GM_DBG_COMPUTE(x)
-#else
-#define GM_DBG_COMPUTE(x) x
-#endif
 #if CL_GDEPTH > 1
 #define GM_STEP(kt, cur, new_a, new_b, old_a, old_b)              \
   {                                                               \
-    GM_DBG_LOAD(GM_LOAD_A(new_a, GM_KOFF((kt) + CL_GDEPTH));)     \
-    GM_DBG_LOAD(GM_LOAD_B(new_b, GM_KOFF((kt) + CL_GDEPTH));)     \
-    GM_DBG_STORE(GM_STORE_NEXT(kt, cur, old_a, old_b))            \
-    GM_DBG_COMPUTE(GM_COMPUTE(cur))                               \
+    GM_LOAD_A(new_a, GM_KOFF((kt) + CL_GDEPTH));     \
+    GM_LOAD_B(new_b, GM_KOFF((kt) + CL_GDEPTH));     \
+    GM_STORE_NEXT(kt, cur, old_a, old_b)            \
+    GM_COMPUTE(cur)                               \
     __syncthreads();                                              \
   }
 #else
 #define GM_STEP(kt, cur, new_a, new_b, old_a, old_b)              \
   {                                                               \
-    GM_DBG_LOAD(GM_LOAD_A(new_a, GM_KOFF((kt) + CL_GDEPTH));)     \
-    GM_DBG_LOAD(GM_LOAD_B(new_b, GM_KOFF((kt) + CL_GDEPTH));)     \
-    GM_DBG_COMPUTE(GM_COMPUTE(cur))                               \
-    GM_DBG_STORE(GM_STORE_NEXT(kt, cur, old_a, old_b))            \
+    GM_LOAD_A(new_a, GM_KOFF((kt) + CL_GDEPTH));     \
+    GM_LOAD_B(new_b, GM_KOFF((kt) + CL_GDEPTH));     \
+    GM_COMPUTE(cur)                               \
+    GM_STORE_NEXT(kt, cur, old_a, old_b)            \
     __syncthreads();                                              \
   }
 #endif

@@ -462,17 +462,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // issuing its whole share at the top of a step stops the matrix cores for the length of the
   // transfer.  CL_SPREAD_LOADS: row r of a step's matrix work is preceded by the r-th slice of
   // the wave's loads instead (measured: no faster on the large matmul; off by default).
-#ifdef CL_DBG_NODMA
-#define GD_ISSUE(kt, a_lds, b_lds)
-#define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)
-#else
 #if CL_ROWSUM
 #define GD_A_AT(kt) (a_base + (i64)((kt) % KT_K) * a_step)
 #define GD_B_AT(kt) (b_base + (i64)((kt) % KT_K) * b_step + (i64)((kt) / KT_K) * (CL_TRANS_B ? (i64)CL_BN * CL_K : (i64)CL_BN))
-#elif defined(CL_DBG_HOT)
-// (timing probe: every workgroup fetches the first tile's first two steps, which stay in L2)
-#define GD_A_AT(kt) (A + (i64)((kt) & 1) * a_step)
-#define GD_B_AT(kt) (B + (i64)((kt) & 1) * b_step)
 #else
 #define GD_A_AT(kt) (a_base + (i64)(kt) * a_step)
 #define GD_B_AT(kt) (b_base + (i64)(kt) * b_step)
@@ -490,11 +482,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, GD_B_AT(kt), b_lds);                        \
     }                                                                                               \
   }
-#endif
-#ifdef CL_DBG_NOCOMPUTE
-#undef GD_COMPUTE
-#define GD_COMPUTE(a_tile, b_tile, NEXT)
-#endif
 #define GD_NO_NEXT(r)
 
   // Two steps per trip, one on each stage, with no branch inside: the loads issued in the second

@@ -147,13 +147,6 @@ CL_DEVICE void ml_issue_from(const MlLoader& ld, const elem_t* lat_rows, const e
   }
 }
 
-#ifdef CL_DBG_TIMING
-// debugging aid: wave 0 of every workgroup leaves cycle-counter readings in its PL rows
-#define ML_STAMP(k) if (threadIdx.x == 0) reinterpret_cast<unsigned*>(CL_ARG_PL)[(blockIdx.y * gridDim.x + blockIdx.x) * 32 + (k)] = (unsigned)__builtin_readcyclecounter();
-#else
-#define ML_STAMP(k)
-#endif
-
 #if CL_EMIT_PARTIAL
 #ifndef CL_OCC
 #define CL_OCC 1
@@ -163,7 +156,6 @@ CL_DEVICE void ml_issue_from(const MlLoader& ld, const elem_t* lat_rows, const e
 // the other's matrix work
 extern "C" __global__ void __launch_bounds__(ML_THREADS, (CL_OCC * CL_WAVES + 3) / 4)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
-  ML_STAMP(0)
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   // Workgroups go to the eight XCDs (one L2 each) round-robin in launch order.  The head blocks
@@ -235,12 +227,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define ML_FRONT(s)                                                                                   \
   __builtin_amdgcn_s_waitcnt(0x0F70 | (ML_WAIT_N & 15) | ((ML_WAIT_N >> 4) << 14));                   \
   __syncthreads();                                                                                    \
-  ML_DBG_ISSUE((s) + ML_AHEAD)
-#ifdef CL_DBG_NODMA
-#define ML_DBG_ISSUE(s)
-#else
-#define ML_DBG_ISSUE(s) ML_ISSUE(s)
-#endif
+  ML_ISSUE((s) + ML_AHEAD)
 
   // The first ML_AHEAD steps' tile loads go out first, the Q fragments right behind them, and one
   // wait covers both (their latencies overlap).  After it the wave's vector-memory counter only
@@ -265,9 +252,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
   if (step_begin < step_end) {
     __syncthreads();
-    ML_DBG_ISSUE(step_begin + ML_AHEAD)
+    ML_ISSUE(step_begin + ML_AHEAD)
   }
-  ML_STAMP(1)
 
   // this lane's operand offsets inside an image (elements):
   //   score operand: token row c of a 16-token half, chunk g of a 32-feature block
@@ -299,12 +285,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int j = 0; j < ML_KJ; ++j) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-#ifdef CL_DBG_NOSREAD
-          const elem8 a = *reinterpret_cast<const elem8*>(tile + 16 * h * 64 + a_lo);
-#else
           const elem8 a = *reinterpret_cast<const elem8*>(tile + (j >> 1) * ML_PANEL + 16 * h * 64 +
                                                           (a_lo ^ ((4 * (j & 1)) << 3)));
-#endif
 #pragma unroll
           for (int hg = 0; hg < CL_HG; ++hg) st[hg][h] = mfma16(a, qf[hg][j], st[hg][h]);
         }
@@ -350,7 +332,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         raise_any = true;
         break;
       }
-      ML_STAMP(4 + 3 * (step - step_begin < 8 ? step - step_begin : 8))
 
       elem8 pf[CL_HG];
 #pragma unroll
@@ -366,11 +347,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int hg = 0; hg < CL_HG; ++hg) l_acc[hg] = mfma16(ones, pf[hg], l_acc[hg]);
 #pragma unroll
       for (int fb = 0; fb < ML_FBW; ++fb) {
-#ifdef CL_DBG_NOVREAD
-        const elem_t* p = tile + (v_lo ^ (((2 * (fb & 1)) & 7) << 3));
-#else
         const elem_t* p = tile + (fb >> 2) * ML_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
-#endif
         const ml_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ml_lds_s16x4*)(p));
         const ml_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ml_lds_s16x4*)(p + 16 * 64));
         const elem8 a = __builtin_bit_cast(elem8, (ml_s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -387,11 +364,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       __builtin_amdgcn_sched_group_barrier(0x008, CL_HG * (ML_LDS_AHEAD / 2), 0);
 
       ++step;
-      ML_STAMP(2 + 3 * (step - step_begin < 8 ? step - step_begin : 8))
       if (step < step_end) {
         ML_FRONT(step)
       }
-      ML_STAMP(3 + 3 * (step - step_begin < 8 ? step - step_begin : 8))
     }
     if (!raise_any) break;
     // cold: raise the reference of the heads that need it and rescale what they have accumulated
@@ -412,7 +387,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // no load may still be on its way into LDS when the workgroup ends
   __builtin_amdgcn_s_waitcnt(0x0F70);
 
-  ML_STAMP(29)
   // ---- write this wave's heads (no cross-wave merge needed: a wave owns its heads) -------------
 #pragma unroll
   for (int hg = 0; hg < CL_HG; ++hg) {
@@ -434,12 +408,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #if CL_SPLITS > 1
     const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
     elem_t* dst_row = CL_ARG_PO + prow * CL_CKV;
-#ifndef CL_DBG_TIMING
     if (g == 0 && vhalf == 0) {
       CL_ARG_PM[prow] = l > 0.f ? m + fast_log2(l) : CL_NEG_BIG;
       CL_ARG_PL[prow] = l > 0.f ? 1.0f : 0.f;
     }
-#endif
 #else
     elem_t* dst_row = CL_ARG_OUT + orow * CL_CKV;
 #if CL_EMIT_LSE
@@ -455,6 +427,5 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
 #endif
   }
-  ML_STAMP(30)
 }
 #endif  // CL_EMIT_PARTIAL

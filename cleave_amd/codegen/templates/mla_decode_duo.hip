@@ -101,24 +101,6 @@ __shared__ __attribute__((aligned(16))) u32x2 md_weights[2][2][2][64][2];
 // [step parity][head set][head tile][head][token half]: the reference point those weights stand against
 __shared__ __attribute__((aligned(8))) float md_ref[2][2][2][16][2];
 
-#ifdef CL_DBG_TIME
-// measurement switch (the result is wrong by design): every wave stamps the shader clock at the
-// marks below, and when a workgroup ends its stamps overwrite a piece of the Q operand
-__shared__ unsigned long long md_stamps[8][48];
-#define MD_MARK(k) do { md_last = __builtin_amdgcn_s_memtime(); if (lane == 0) md_stamps[wave][(k)] = md_last; } while (0)
-// time since the previous MD_MARK / MD_SUB of this wave, added up in slot 38 + k
-#define MD_SUB(k) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long now_ = __builtin_amdgcn_s_memtime(); \
-    md_sub[k] += now_ - md_last; md_last = now_; __builtin_amdgcn_sched_barrier(0); } while (0)
-#define MD_MARK_WALL(k) do { if (lane == 0) md_stamps[wave][(k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#define MD_DUMP() do { if (lane < 4) md_stamps[wave][38 + lane] = md_sub[lane]; __builtin_amdgcn_s_waitcnt(0xC07F); if (lane < 48) \
-    ((unsigned long long*)CL_ARG_Q)[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 48 + lane] = md_stamps[wave][lane]; } while (0)
-#else
-#define MD_MARK(k)
-#define MD_SUB(k)
-#define MD_MARK_WALL(k)
-#define MD_DUMP()
-#endif
-
 typedef short md_s16x4 __attribute__((ext_vector_type(4)));
 typedef short md_s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) md_s16x4 md_lds_s16x4;
@@ -232,12 +214,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   step_end = step_end < n_steps ? step_end : n_steps;
   const int n_own = step_end > step_begin ? step_end - step_begin : 0;       // steps of this split
   const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)md_tiles;
-#ifdef CL_DBG_TIME
-  if (lane < 48) md_stamps[wave][lane] = 0;
-  unsigned long long md_last = 0, md_sub[4] = {0, 0, 0, 0};
-#endif
-  MD_MARK(0);
-  MD_MARK_WALL(1);
 
   // The Q rows of the 64 heads go through LDS: every wave asks for its share as whole 1 KiB runs
   // (64 consecutive 16-byte slots each), into the two images' worth of LDS the loop fills last;
@@ -288,22 +264,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     const int half = fhalf;
     const int a_lo = (16 * half + c) * 64 + ((g ^ md_swz(c)) << 3);
 
-#ifdef CL_DBG_TIME
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-#endif
-    MD_MARK(2);
     for (int it = 0; it <= n_own; ++it) {
 #if CL_S_PANELS
       // this wave's panels of image `it` have landed: at most those of image it + 1 are on their way
       __builtin_amdgcn_s_waitcnt(0x0F70 | (CL_S_PANELS & 15));
 #endif
       md_barrier();                                 // image `it` has landed (the value waves waited for it)
-      MD_MARK(3 + 2 * it);
       if (it == n_own) break;
       const elem_t* tile = md_tiles + (it % MD_STAGES) * MD_TILE;
-#ifdef CL_DBG_NOS
-      continue;
-#endif
       // the points the other token half used one step ago: asked for first, so that the answer is
       // there when the matrix ops are done
       float other[2] = {CL_NEG_BIG, CL_NEG_BIG};
@@ -332,7 +300,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         const elem8 a = *reinterpret_cast<const elem8*>(tile + (j >> 1) * MD_PANEL + (a_lo ^ ((4 * (j & 1)) << 3)));
 #pragma unroll
         for (int t = 0; t < 2; ++t) sp[t][j & 1] = mfma16(a, qf[t][j], sp[t][j & 1]);
-#if CL_S_PANELS && !defined(CL_DBG_NODMA)
+#if CL_S_PANELS
         if (it > 0) {
 #pragma unroll
           for (int pn = 0; pn < CL_S_PANELS; ++pn)
@@ -350,10 +318,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       f32x4 st[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) st[t] = sp[t][0] + sp[t][1];
-#ifdef CL_DBG_TIME
-      asm volatile("" :: "v"(st[0]), "v"(st[1]));
-#endif
-      MD_SUB(0);
 
       if (MD_RAGGED) {
         const int t0 = (step_begin + it) * MD_STEP + 16 * half + 4 * g;
@@ -390,12 +354,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         md_weights[it & 1][set][t][lane][half] = __builtin_bit_cast(u32x2, pf);
         if (g == 0) md_ref[it & 1][set][t][c][half] = m_run[t];
       }
-      MD_SUB(1);
-      MD_MARK(4 + 2 * it);
     }
-    MD_MARK(45);
-    MD_MARK_WALL(46);
-    MD_DUMP();
 #if CL_S_PANELS
     __builtin_amdgcn_s_waitcnt(0x0F70);             // no load may still be on its way into LDS when the workgroup ends
 #endif
@@ -406,9 +365,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // loads of step index s (relative to the split), clamped onto the split's last step so that the
   // load counter holds the same number of steps at every wait
   auto issue = [&](int s) __attribute__((always_inline)) {
-#ifdef CL_DBG_NODMA
-    return;
-#endif
     int rel = s < n_own - 1 ? s : n_own - 1;
     rel = rel > 0 ? rel : 0;
     const int t0 = (step_begin + rel) * MD_STEP;
@@ -436,7 +392,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * MD_UNITS_PER) & 15) | (((2 * MD_UNITS_PER) >> 4) << 14));
     md_barrier();
   }
-  MD_MARK(2);
   // the value operands of the first MD_PRE feature blocks of the next image: read at the end of an
   // iteration, they are on their way while the waves meet at the barrier
   constexpr int MD_PRE = CL_LDS_AHEAD / 2;
@@ -456,21 +411,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // down to that count is the right wait for them and a longer one for the first three)
     if (n_own > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (MD_V_UNITS & 15) | ((MD_V_UNITS >> 4) << 14));
     md_barrier();
-    MD_MARK(3 + 2 * it);
     const elem_t* next_tile = md_tiles + (it % MD_STAGES) * MD_TILE;           // image `it`: there from here on
     if (it == 0) {
       if (it < n_own) issue(it + 2);
-#ifndef CL_DBG_NOV
 #pragma unroll
       for (int fb = 0; fb < MD_PRE; ++fb) operand(next_tile, fb, pre_lo[fb], pre_hi[fb]);
-#endif
       continue;
     }
     const elem_t* tile = md_tiles + ((it - 1) % MD_STAGES) * MD_TILE;
-#ifdef CL_DBG_NOV
-    if (it < n_own) issue(it + 2);
-    continue;
-#endif
     elem8 pf[2];
     f32x2 ref[2];
 #pragma unroll
@@ -494,10 +442,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         for (int i = 0; i < 8; ++i) pf[t][i] = to_elem(to_f32(pf[t][i]) * (i < 4 ? f_lo : f_hi));
       }
     }
-#ifdef CL_DBG_TIME
-    asm volatile("" :: "v"(pf[0]), "v"(pf[1]));
-#endif
-    MD_SUB(1);
     // The loads of image it + 2 (into the slot image it - 2 has left) are asked for between the
     // matrix ops, panel p after feature block p * MD_FBW / MD_PANELS.  Past the split's end the
     // last image is asked for again, into the slot of image n_own + 1 (which holds or awaits the
@@ -520,11 +464,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         operand(tile, fb + MD_PRE, pre_lo[fb % MD_PRE], pre_hi[fb % MD_PRE]);
       else
         operand(next_tile, fb + MD_PRE - MD_FBW, pre_lo[fb % MD_PRE], pre_hi[fb % MD_PRE]);
-#ifndef CL_DBG_NODMA
 #pragma unroll
       for (int pn = CL_S_PANELS; pn < MD_PANELS; ++pn)
         if (((pn - CL_S_PANELS) * MD_FBW) / MD_V_UNITS == fb) md_issue_panel(pn, lat_off, pe_off, lat_rows, pe_rows, t0, stage_byte, loader);
-#endif
     }
 #pragma unroll
     for (int n = 0; n < MD_FBW; ++n) {
@@ -533,11 +475,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
 #pragma unroll
     for (int t = 0; t < 2; ++t) l_acc[t] = mfma16(ones, pf[t], l_acc[t]);      // row sums of exactly the weights used
-    MD_SUB(2);
-    MD_MARK(4 + 2 * it);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);               // no load may still be on its way into LDS when the workgroup ends
-  MD_MARK(44);
 
   // ---- this wave writes its half of the features of its head set --------------------------------
   // Through LDS, so that a store instruction covers whole half rows (two of 512 bytes at a latent
@@ -580,11 +519,5 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       *reinterpret_cast<u32x4*>(dst + (i64)r * (CL_CKV * 2) + 16 * piece) = *reinterpret_cast<const u32x4*>(rows + r * MD_OROW + 16 * piece);
     }
   }
-#ifdef CL_DBG_TIME
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-#endif
-  MD_MARK(45);
-  MD_MARK_WALL(46);
-  MD_DUMP();
 }
 #endif  // CL_EMIT_PARTIAL

@@ -81,28 +81,11 @@ CL_DEVICE void sk_load(const elem_t* __restrict__ W, const elem_t* __restrict__ 
 #endif
 }
 
-#ifdef CL_DBG_TIME
-// measurement switch (the result is wrong by design): every wave stamps the shader clock (slots
-// 0, 2, 3, 4) and the 100 MHz wall clock (1, 5) and leaves them in the first bytes of X
-#define SK_MARK(k) do { const unsigned long long t_ = (k) == 1 || (k) == 5 ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); \
-    __builtin_amdgcn_sched_barrier(0); sk_stamps[k] = t_; } while (0)
-#define SK_DUMP() do { SK_MARK(4); SK_MARK(5); sk_stamps[6] = __builtin_amdgcn_s_getreg(63492); sk_stamps[7] = __builtin_amdgcn_s_getreg(63508); if (lane == 0) { \
-    unsigned long long* dump_ = (unsigned long long*)CL_ARG_X + ((blockIdx.y * gridDim.x + blockIdx.x) * (SK_THREADS / 64) + wave) * 8; \
-    _Pragma("unroll") for (int k_ = 0; k_ < 8; ++k_) dump_[k_] = sk_stamps[k_]; } } while (0)
-#else
-#define SK_MARK(k)
-#define SK_DUMP()
-#endif
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(SK_THREADS)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // (readfirstlane: everything derived from the wave index is uniform and stays in scalar registers)
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-#ifdef CL_DBG_TIME
-  unsigned long long sk_stamps[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
-  SK_MARK(0);
-  SK_MARK(1);
   const int c = lane & 15, g = lane >> 4;
   const int wn = wave % CL_WAVES_N, wk = wave / CL_WAVES_N;
   const int split = blockIdx.y;
@@ -243,10 +226,6 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     }
   }
 
-#ifdef CL_DBG_TIME
-  asm volatile("" :: "v"(acc[0][0]));
-#endif
-  SK_MARK(2);
   // ---- reduce across the waves that share a column slab ------------------------------------
   // acc[mt][j][r] = Y[16 mt + 4 g + r][n_base + 8 c + j]
 #if CL_NORM
@@ -290,10 +269,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   }
 #endif
   __syncthreads();
-  SK_MARK(3);
 #if !CL_LORA
   if (wk != 0) {
-    SK_DUMP();
     return;
   }
 #endif
@@ -395,6 +372,5 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
     }
   }
-  SK_DUMP();
 }
 #endif  // CL_EMIT_PARTIAL

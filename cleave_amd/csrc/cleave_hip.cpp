@@ -116,6 +116,7 @@ namespace {
 constexpr int kMaxDevices = 64;
 constexpr int kMaxSeq = 8;          // launches per call of the fixed-scratch entry point
 constexpr int kMaxArgs = 64;        // arguments per launch there
+constexpr int kMaxScratchRefs = 64; // scratch arguments per call there
 
 // Device address of `scratch` on the current device, resolved once per device with that device
 // current (every GPU holds its own copy of the array at its own address).
@@ -330,6 +331,7 @@ int chip_launch_seq_fixed_scratch(const chip_launch_desc* seq, int n, void* stre
   if (!seq || n <= 0) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: empty sequence");
   if (n > kMaxSeq) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: more than 8 launches in one call");
   if (nrefs < 0 || (nrefs > 0 && !refs)) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: bad scratch argument list");
+  if (nrefs > kMaxScratchRefs) return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: more than 64 scratch arguments");
   if (scratch_bytes > CHIP_FIXED_SCRATCH_BYTES) {
     char buf[200];
     snprintf(buf, sizeof buf, "chip_launch_seq_fixed_scratch: %llu bytes of scratch asked for, the fixed array holds %llu",
@@ -345,6 +347,9 @@ int chip_launch_seq_fixed_scratch(const chip_launch_desc* seq, int n, void* stre
       return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: scratch argument names no argument of the sequence");
     if (a.offset % 256 || a.offset >= scratch_bytes)
       return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: scratch offset not a multiple of 256 or outside scratch_bytes");
+    for (int q = 0; q < r; ++q)
+      if (refs[q].launch == a.launch && refs[q].arg == a.arg)
+        return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: one argument is named by two scratch entries");
   }
   unsigned char* base = nullptr;
   int rc = fixed_scratch_ptr(&base);
@@ -360,15 +365,13 @@ int chip_launch_seq_fixed_scratch(const chip_launch_desc* seq, int n, void* stre
   }
   // the caller's argument arrays are left as they are: each launch gets a copy of its pointer
   // array (on this stack) whose scratch slots point at addresses inside the fixed array
-  void* values[kMaxSeq * 4 + 32];
+  void* values[kMaxScratchRefs];
   int used = 0;
   for (int i = 0; i < n; ++i) {
     void* args[kMaxArgs];
     for (int j = 0; j < seq[i].nargs; ++j) args[j] = seq[i].args[j];
     for (int r = 0; r < nrefs; ++r) {
       if (refs[r].launch != i) continue;
-      if (used >= (int)(sizeof values / sizeof values[0]))
-        return fail(CHIP_ERR_INVALID, "chip_launch_seq_fixed_scratch: more than 64 scratch arguments");
       values[used] = base + refs[r].offset;
       args[refs[r].arg] = &values[used++];
     }

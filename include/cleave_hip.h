@@ -172,8 +172,10 @@ typedef struct chip_scratch_arg {
  * address `array + offset` (whatever the caller's slot holds is ignored and
  * left untouched); `scratch_bytes` is the extent the caller's layout uses.
  *   - scratch_bytes above CHIP_FIXED_SCRATCH_BYTES, an offset that is not a
- *     multiple of 256 or lies outside scratch_bytes, more than 8 launches or
- *     64 arguments per launch: CHIP_ERR_INVALID, nothing is launched;
+ *     multiple of 256 or lies outside scratch_bytes, more than 8 launches,
+ *     64 arguments per launch or 64 entries in `refs`, or two entries that
+ *     name the same argument: CHIP_ERR_INVALID, nothing is launched (every
+ *     check runs before the fill kernel and the first launch);
  *   - the call makes no hipMalloc / hipFree and no other allocating call;
  *   - all calls on one GPU share that GPU's array and it keeps the previous
  *     call's contents: `clear` != 0 zeroes the first scratch_bytes with a fill

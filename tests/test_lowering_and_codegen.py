@@ -315,6 +315,20 @@ def test_codegen_refuses_impossible_plans():
         parse_manifest("__global__ void k() {}")
 
 
+def test_tiling_keys_that_ask_for_a_measurement_switch_are_refused():
+    """The shipped templates hold no probes; a DBG_ key in a tiling is an error, not a silent no-op."""
+    g = stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=32, HKV=8, SQ=1, SKV=1024, D=128))
+    for template, tiling in (("attn_decode", dict(WAVES=1, DBG_TIME=1)),):
+        with pytest.raises(CodegenError, match="measurement switches"):
+            HipCodeGen().gen(apply_tiling(TileDict(template, "main", tiling, flat_graph=g)))
+    mla = stage_graph(C.mla_decode.trace(cl.bf16, B=2, H=64, D=512, PE=64, SKV=256))
+    with pytest.raises(CodegenError, match="measurement switches"):
+        HipCodeGen().gen(apply_tiling(TileDict("mla_decode", "main", dict(DUO=1, DBG_NODMA=1), flat_graph=mla)))
+    templates = Path(C.__file__).parent / "codegen" / "templates"
+    for f in templates.glob("*.hip"):
+        assert "DBG_" not in f.read_text(), f.name
+
+
 def test_matmul_rowsum_with_a_ragged_column_tile_is_refused_with_its_reason():
     """One set of accumulators sums every column tile of a row block, so a ragged last tile cannot be masked."""
     with pytest.raises(ScheduleRejected, match="N % 16 == 0"):

@@ -76,4 +76,12 @@ def test_sizes_beyond_the_array_are_refused():
         shim.launch_seq_fixed_scratch(descs, 0, [(0, 0, 128)], 4096)
     with pytest.raises(shim.HipError, match="names no argument"):
         shim.launch_seq_fixed_scratch(descs, 0, [(len(descs), 0, 0)], 4096)
+    with pytest.raises(shim.HipError, match="more than 64 scratch arguments"):
+        shim.launch_seq_fixed_scratch(descs, 0, [(0, 0, 256 * i) for i in range(65)], 65 * 256)
+    with pytest.raises(shim.HipError, match="named by two scratch entries"):
+        shim.launch_seq_fixed_scratch(descs, 0, [(0, 0, 0), (0, 0, 256)], 4096)
+    # (the refusals above come before anything is launched: the outputs of the last good call stand)
+    torch.cuda.synchronize()
+    again = own(*args)
+    assert torch.equal(again[0], out) and torch.equal(again[1], lse)
     del keep
