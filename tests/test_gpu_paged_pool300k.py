@@ -12,7 +12,10 @@ chunk and a fixed-split plan:
     whose bits encode (page, slot, head) -- a page id truncated to 32-bit byte offsets, a wrong
     slot or a wrong head changes bits;
   * the attention output equals the numpy oracle's on the named pages compacted into a small pool
-    (reference ``python/cleave/dynamic/reference.py:143-200``), rtol = atol = 1e-2, lse 1e-3.
+    (reference ``python/cleave/dynamic/reference.py:143-200``), rtol = atol = 1e-2, lse 1e-3;
+  * the same comparison at the request lengths the configuration states: 32 requests with lengths
+    drawn uniformly from [256, 16384] (up to 256 pages a request, several thousand pages in all),
+    placed at seeded ids across the whole pool.
 """
 
 import numpy as np
@@ -126,3 +129,48 @@ def test_gather_out_of_high_pages_is_bit_exact(pools, plan):
                 want = v_small[pos, slot, h // (HQ // HKV)].float().numpy()
                 assert np.array_equal(got_o[b, h], want), (b, h, int(ids[pos]), slot)
     assert set(FORCED) <= tested
+
+
+def _stated_draw(seed=5):
+    """The benchmark's own draw (bench.py ``run_paged``): 32 lengths U[256, 16384] from the seed, the table a
+    seeded permutation of the whole pool (``python/cleave/dynamic/reference.py:44-49``), with the pool's last
+    page put in so that the highest address is among the ones read."""
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    lens = torch.randint(256, 16384 + 1, (32,), generator=gen).tolist()
+    pages = [-(-n // PAGE) for n in lens]
+    total = sum(pages)
+    ids = torch.randperm(POOL, generator=gen)[:total]
+    if POOL - 1 not in ids.tolist():
+        ids[total // 2] = POOL - 1
+    indptr = torch.tensor([0] + np.cumsum(pages).tolist(), dtype=torch.int32)
+    last = torch.tensor([n - (p - 1) * PAGE for n, p in zip(lens, pages)], dtype=torch.int32)
+    return gen, lens, ids.to(torch.int32), indptr, last
+
+
+@pytest.fixture(scope="module")
+def stated():
+    """The draw, its operands and the oracle's answer, made once for the three plans (the oracle takes ~12 s)."""
+    gen, lens, ids, indptr, last = _stated_draw()
+    n = len(ids)
+    k_small = torch.randn(n, PAGE, HKV, D, generator=gen).to(torch.float16)
+    v_small = torch.randn(n, PAGE, HKV, D, generator=gen).to(torch.float16)
+    q = torch.randn(len(lens), HQ, D, generator=gen).to(torch.float16)
+    want = paged_oracle.decode(q, k_small, v_small, indptr, torch.arange(n, dtype=torch.int32), lens, PAGE, D ** -0.5,
+                               out_dtype="float16")
+    return lens, ids, indptr, last, q, k_small, v_small, want
+
+
+@pytest.mark.parametrize("plan", PLANS, ids=lambda p: "-".join(f"{k}{v}" for k, v in p.items()))
+def test_the_stated_request_lengths_match_the_oracle(pools, stated, plan):
+    k_pool, v_pool = pools
+    lens, ids, indptr, last, q, k_small, v_small, (want_o, want_l) = stated
+    n = len(ids)
+    assert min(lens) >= 256 and max(lens) > 12_000 and int((indptr[1:] - indptr[:-1]).max()) > 190 and n > 3000
+    assert int(ids.max()) == POOL - 1 and int((ids >= 16_384).sum()) > 0.9 * n and len(set(ids.tolist())) == n
+    k_pool[ids.long().cuda()] = k_small.cuda()
+    v_pool[ids.long().cuda()] = v_small.cuda()
+    print(f"pool300k stated lengths plan={plan}: {sum(lens)} tokens in {n} pages, longest {max(lens)}", flush=True)
+    kernel = paged_kernel(page_size=PAGE, **plan)
+    got_o, got_l = _run(kernel, [q.cuda(), k_pool, v_pool, indptr.cuda(), ids.cuda(), last.cuda(), D ** -0.5])
+    np.testing.assert_allclose(got_o, want_o, rtol=1e-2, atol=1e-2)
+    np.testing.assert_allclose(got_l, want_l, rtol=1e-3, atol=1e-3)
