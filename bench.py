@@ -63,6 +63,13 @@ def op_table():
         "mm": dict(title="matmul f16 4096x14336x4096", fn=C.matmul, dtype=cl.f16, shapes=dict(M=4096, N=14336, K=4096),
                    inputs=C.inputs_c1, split=False, bytes=2 * (4096 * 4096 + 4096 * 14336 + 4096 * 14336),
                    flops=2 * 4096 * 14336 * 4096, bound="mfma", sets=2),
+        "mm_nt": dict(title="matmul f16 4096x14336x4096, weight given (N, K): x @ w.T", fn=C.matmul_nt, dtype=cl.f16,
+                      shapes=dict(M=4096, N=14336, K=4096), inputs=C.inputs_nt, split=False,
+                      bytes=2 * (4096 * 4096 + 4096 * 14336 + 4096 * 14336), flops=2 * 4096 * 14336 * 4096, bound="mfma",
+                      sets=2, cpu=False),
+        "mm8k": dict(title="matmul bf16 8192x8192x8192, weight given (N, K): x @ w.T", fn=C.matmul_nt, dtype=cl.bf16,
+                     shapes=dict(M=8192, N=8192, K=8192), inputs=C.inputs_nt_bf16, split=False,
+                     bytes=2 * 3 * 8192 * 8192, flops=2 * 8192 ** 3, bound="mfma", sets=2, cpu=False),
         "swiglu": dict(title="SwiGLU f16 (x@w_up)*silu(x@w_gate) 4096x14336x4096", fn=C.swiglu, dtype=cl.f16,
                        shapes=C.FULL["swiglu"], inputs=C.inputs_swiglu, split=False,
                        bytes=2 * (4096 * 4096 + 2 * 4096 * 14336 + 4096 * 14336), flops=4 * 4096 * 14336 * 4096,
@@ -610,7 +617,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,swiglu,rmsmm,lora,mmrs,mm2d,rsdiv,attn,qknorm,mlapf,dyn")
+    ap.add_argument("--ops", default="c2,c1,c3,c4,c5,mm,mm_nt,mm8k,swiglu,rmsmm,lora,mmrs,mm2d,rsdiv,attn,qknorm,mlapf,dyn")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--search-iters", type=int, default=30)
     ap.add_argument("--dyn-ops", default="", help="with --ops dyn: comma-separated registry operators (default: all)")

@@ -450,6 +450,14 @@ class HipCodeGen:
         unit.define("CL_PREFETCH", int(t.get("PREFETCH", 1)))
         chunk_pages = bool(t.get("CHUNK_PAGES", 0)) and paged and (plan.split_factor or 1) > 1
         unit.define("CL_CHUNK_PAGES", chunk_pages)
+        skew = int(t.get("SKEW", 0))
+        if skew:
+            # the rotation of units over the XCDs assumes that launch index % 8 is blockIdx.x % 8
+            per_x = (p["kv_heads"] if paged else p["units"]) * (-(-rows // 16))
+            if (plan.split_factor or 1) % 2 or chunk_pages or per_x % 8 or not 0 < skew <= 500 or not partial:
+                raise CodegenError("SKEW (split ranges skewed between even and odd XCDs, in thousandths of a pair's steps, "
+                                   "1..500) needs an even split count, a grid of whole groups of eight unit tiles and no chunked items")
+            unit.define("CL_SKEW", skew)
         unit.define("CL_PAGED", paged)
         unit.define("CL_PAGE_SIZE", p.get("page_size", 1))
         unit.define("CL_KV_HEADS", p.get("kv_heads", 1))

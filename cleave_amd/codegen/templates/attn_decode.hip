@@ -20,6 +20,16 @@
 //   CL_SCALE_LOG2E softmax scale * log2(e) (dense; paged passes sm_scale at run time)
 //   CL_EMIT_LSE  also write the base-2 log-sum-exp
 //   CL_PREFETCH  steps of K/V in flight ahead of the one being computed (1 or 2)
+//   CL_SKEW      0 = off.  The hardware deals workgroups out to the eight XCDs round-robin in launch
+//                order, so with a grid whose x extent is a multiple of eight all splits of a unit
+//                land on one XCD, and the XCDs do not stream equally fast (measured: the
+//                odd-numbered ones about 5 % slower, whatever data they are given), so a kernel
+//                dealt out in equal shares ends with its slowest XCD.  With CL_SKEW the units of
+//                each group of eight are rotated by the split index, which spreads a unit's
+//                splits over all XCDs, and of every pair of neighbouring splits the one on the
+//                even XCD takes CL_SKEW thousandths of the pair's steps from the one on the odd
+//                XCD.  Every step still belongs to exactly one split.  (Even split counts, grid x
+//                a multiple of eight; the search times a few values.)
 //   CL_CHUNK_PAGES  paged only, 0 = off.  1: work is cut into items of at most `chunk_pages`
 //                pages (a run-time argument, 1..64, chosen by the host from the table length)
 //                instead of a fixed number of splits per request, and a workgroup holds one wave
@@ -29,6 +39,12 @@
 #define ATT_RAISE_BY 8.0f
 #ifndef CL_CHUNK_PAGES
 #define CL_CHUNK_PAGES 0
+#endif
+#ifndef CL_SKEW
+#define CL_SKEW 0
+#endif
+#if CL_SKEW && (CL_CHUNK_PAGES || CL_SPLITS % 2)
+#error "skewed split ranges: an even number of splits, no chunked items"
 #endif
 #define ATT_STEP 32
 #define ATT_KJ (CL_HEAD_DIM / 32)            // score MFMAs per 16 tokens
@@ -122,8 +138,16 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int item = blockIdx.x;
 #else
   const int split = blockIdx.y;
-  const int tile_id = blockIdx.x % ATT_ROW_TILES;
-  const int unit = blockIdx.x / ATT_ROW_TILES;
+#if CL_SKEW
+  // this workgroup runs on XCD blockIdx.x % 8 (grid x is a multiple of eight); the unit tile it
+  // works for is rotated within its group of eight by the split index
+  const int xcd = blockIdx.x & 7;
+  const int unit_tile = (blockIdx.x & ~7) | ((xcd + split) & 7);
+#else
+  const int unit_tile = blockIdx.x;
+#endif
+  const int tile_id = unit_tile % ATT_ROW_TILES;
+  const int unit = unit_tile / ATT_ROW_TILES;
 #endif
 
   AttUnit u;
@@ -215,6 +239,23 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #if CL_CHUNK_PAGES
   const int step_begin = 0, step_end = n_steps;      // the item is the unit of work: no further cut
   (void)split;
+#elif CL_SKEW
+  // splits 2k and 2k + 1 share ceil(n_steps / (SPLITS / 2)) steps; the one on the even XCD takes
+  // the larger share.  XCD parity = parity of (unit tile - split): exactly one of a pair is even.
+  int step_begin, step_end;
+  {
+    const int per_pair = (n_steps + CL_SPLITS / 2 - 1) / (CL_SPLITS / 2);
+    int lo = (split >> 1) * per_pair, hi = lo + per_pair;
+    lo = lo < n_steps ? lo : n_steps;
+    hi = hi < n_steps ? hi : n_steps;
+    const int len = hi - lo;
+    int big = (len + 1) / 2 + ((len / 2) * CL_SKEW + 500) / 1000;
+    big = big < len ? big : len;
+    const bool even_xcd = (xcd & 1) == 0;
+    const int first = (split & 1) == 0 ? (even_xcd ? big : len - big) : (even_xcd ? len - big : big);
+    step_begin = (split & 1) == 0 ? lo : lo + first;
+    step_end = (split & 1) == 0 ? lo + first : hi;
+  }
 #else
   const int per_split = (n_steps + CL_SPLITS - 1) / CL_SPLITS;
   const int step_begin = split * per_split;
@@ -254,93 +295,138 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define ATT_WSTRIDE CL_WAVES
   const int step0 = step_begin + wave;
 #endif
-  // Prefetch loads are issued unconditionally: a step past the end is clamped onto this wave's
-  // last real step (an L2 hit, its tile is never consumed).  A branch around the loads would
-  // make the hardware load counter differ between paths, and the waits the compiler then has
-  // to insert drain the prefetch before every value product.
-  int last_step = step0;
-  if (step_end > step0) last_step = step0 + ((step_end - 1 - step0) / ATT_WSTRIDE) * ATT_WSTRIDE;
+  // Inside the loop prefetch loads are issued unconditionally (a branch around them would make the
+  // hardware load counter differ between paths, and the waits the compiler then has to insert drain
+  // the prefetch before every value product): the loop runs only while the step CL_PREFETCH ahead of
+  // each of its steps exists, and the last steps follow as straight-line code that asks for nothing
+  // past the wave's last step.
+// One 32-token step: asks for the step CL_PREFETCH ahead into the ring slot the previous step left, then
+// multiplies the slot R: scores^T for the two 16-token halves, weights, value product.
+// The softmax reference point of a row is raised only when a score passes it by more than 8 (a factor
+// 2^8: weights stay below 256, softmax does not depend on the reference point), so after the first steps
+// of a split the maxima are not even compared across the four lane groups and the accumulators are not
+// rescaled: both happen only when some lane asks (the two ballots are wave-uniform and cold).  Masked
+// slots hold CL_NEG_BIG; while a whole row is still masked its reference equals it too, so the weights
+// test the mask itself rather than trusting exp2 of a zero difference.  The row sum adds up the weights
+// as rounded to the element type, the ones the value product really sees.
+// (A macro, so that the loop below holds no branch out of its body: with one, the compiler must assume
+// at the loop head that loads of the skipped part are still on their way into registers it is about to
+// reuse for addresses, and it waits for the current tile before it asks for the next.)
+#define ATT_ONE_STEP(R, STEP, LOAD)                                                                 \
+    {                                                                                               \
+      if (LOAD) att_load(u, ((STEP) + CL_PREFETCH * ATT_WSTRIDE) * ATT_STEP, c, g, ring[((R) + CL_PREFETCH) % (CL_PREFETCH + 1)]); \
+      const AttTile& cur = ring[R];                                                                 \
+      const int t0 = (STEP) * ATT_STEP;                                                             \
+                                                                                                    \
+      float s[8];                                                                                   \
+_Pragma("unroll")                                                                                   \
+      for (int h = 0; h < 2; ++h) {                                                                 \
+        f32x4 st = (f32x4){0.f, 0.f, 0.f, 0.f};                                                     \
+_Pragma("unroll")                                                                                   \
+        for (int j = 0; j < ATT_KJ; ++j) st = mfma16(as_elem8(cur.k[h][j]), qf[j], st);             \
+_Pragma("unroll")                                                                                   \
+        for (int q = 0; q < 4; ++q) {                                                               \
+          const int t = t0 + 16 * h + 4 * g + q;                                                    \
+          s[4 * h + q] = t < u.kv_len ? st[q] * scale2 : CL_NEG_BIG;                                \
+        }                                                                                           \
+      }                                                                                             \
+      float mx = s[0];                                                                              \
+_Pragma("unroll")                                                                                   \
+      for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);                                             \
+      float alpha = 1.0f;                                                                           \
+      if (__builtin_amdgcn_ballot_w64(mx > m_run + ATT_RAISE_BY)) {                                 \
+        mx = fmaxf(mx, lane_xor(mx, lane, 16));                                                     \
+        mx = fmaxf(mx, lane_xor(mx, lane, 32));                                                     \
+        if (mx > m_run + ATT_RAISE_BY) {                                                            \
+          alpha = fast_exp2(m_run - mx);                                                            \
+          m_run = mx;                                                                               \
+        }                                                                                           \
+      }                                                                                             \
+      const float m_new = m_run;                                                                    \
+      elem8 pf;                                                                                     \
+      float psum = 0.f;                                                                             \
+_Pragma("unroll")                                                                                   \
+      for (int i = 0; i < 8; ++i) {                                                                 \
+        float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;                         \
+        elem_t pe = to_elem(p);                                                                     \
+        psum += to_f32(pe);                                                                         \
+        pf[i] = pe;                                                                                 \
+      }                                                                                             \
+      l_run = l_run * alpha + psum;                                                                 \
+                                                                                                    \
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {                                             \
+_Pragma("unroll")                                                                                   \
+        for (int vc = 0; vc < ATT_VC; ++vc)                                                         \
+_Pragma("unroll")                                                                                   \
+          for (int j = 0; j < 8; ++j) acc[vc][j] *= alpha;                                          \
+      }                                                                                             \
+_Pragma("unroll")                                                                                   \
+      for (int vc = 0; vc < ATT_VC; ++vc) {                                                         \
+        u32x4 vt[8];                                                                                \
+        transpose8x8(cur.v[vc], vt);                                                                \
+_Pragma("unroll")                                                                                   \
+        for (int j = 0; j < 8; ++j) acc[vc][j] = mfma16(as_elem8(vt[j]), pf, acc[vc][j]);           \
+      }                                                                                             \
+    }
+  // A wave with steps of its own (one branch around prologue and loop together, so that the wait for
+  // the Q fragments sits behind the first tiles' loads, not at a join that knows nothing of them).
   if (step0 < step_end) {
 #pragma unroll
-    for (int i = 0; i < CL_PREFETCH; ++i) {
-      int sidx = step0 + i * ATT_WSTRIDE;
-      sidx = sidx < last_step ? sidx : last_step;
-      att_load(u, sidx * ATT_STEP, c, g, ring[i]);
+    for (int i = 0; i < CL_PREFETCH; ++i)
+      if (step0 + i * ATT_WSTRIDE < step_end) att_load(u, (step0 + i * ATT_WSTRIDE) * ATT_STEP, c, g, ring[i]);
+    int base = step0;
+    for (; base + 2 * CL_PREFETCH * ATT_WSTRIDE < step_end; base += (CL_PREFETCH + 1) * ATT_WSTRIDE) {
+#pragma unroll
+      for (int r = 0; r <= CL_PREFETCH; ++r) ATT_ONE_STEP(r, base + r * ATT_WSTRIDE, true)
     }
-  }
-  for (int base = step0; base < step_end; base += (CL_PREFETCH + 1) * ATT_WSTRIDE) {
+    // (at most 2 * CL_PREFETCH steps are left)
 #pragma unroll
-    for (int r = 0; r <= CL_PREFETCH; ++r) {
-      const int step = base + r * ATT_WSTRIDE;
-      if (step >= step_end) break;
-      int ahead = step + CL_PREFETCH * ATT_WSTRIDE;
-      ahead = ahead < last_step ? ahead : last_step;
-      att_load(u, ahead * ATT_STEP, c, g, ring[(r + CL_PREFETCH) % (CL_PREFETCH + 1)]);
-      const AttTile& cur = ring[r];
-      const int t0 = step * ATT_STEP;
-
-      // scores^T for the two 16-token halves
-      float s[8];
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        f32x4 st = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < ATT_KJ; ++j) st = mfma16(as_elem8(cur.k[h][j]), qf[j], st);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int t = t0 + 16 * h + 4 * g + q;
-          s[4 * h + q] = t < u.kv_len ? st[q] * scale2 : CL_NEG_BIG;
-        }
-      }
-      // The softmax reference point of a row is raised only when a score passes it by more than 8
-      // (a factor 2^8: weights stay below 256, softmax does not depend on the reference point), so
-      // after the first steps of a split the maxima are not even compared across the four lane
-      // groups and the accumulators are not rescaled: both happen only when some lane asks.
-      float mx = s[0];
-#pragma unroll
-      for (int i = 1; i < 8; ++i) mx = fmaxf(mx, s[i]);
-      float alpha = 1.0f;
-      if (__builtin_amdgcn_ballot_w64(mx > m_run + ATT_RAISE_BY)) {     // wave-uniform, cold
-        mx = fmaxf(mx, lane_xor(mx, lane, 16));
-        mx = fmaxf(mx, lane_xor(mx, lane, 32));
-        if (mx > m_run + ATT_RAISE_BY) {
-          alpha = fast_exp2(m_run - mx);
-          m_run = mx;
-        }
-      }
-      const float m_new = m_run;
-      elem8 pf;
-      float psum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        // masked slots hold CL_NEG_BIG; when the whole row is still masked m_new equals it too,
-        // so test the mask itself rather than trusting exp2 of a zero difference
-        float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;
-        elem_t pe = to_elem(p);
-        psum += to_f32(pe);            // the sum uses the weights the value product really sees
-        pf[i] = pe;
-      }
-      l_run = l_run * alpha + psum;
-
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {   // wave-uniform: skip when no max moved
-#pragma unroll
-        for (int vc = 0; vc < ATT_VC; ++vc)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) acc[vc][j] *= alpha;
-      }
-#pragma unroll
-      for (int vc = 0; vc < ATT_VC; ++vc) {
-        u32x4 vt[8];
-        transpose8x8(cur.v[vc], vt);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[vc][j] = mfma16(as_elem8(vt[j]), pf, acc[vc][j]);
-      }
-    }
+    for (int r = 0; r < 2 * CL_PREFETCH; ++r)
+      if (base + r * ATT_WSTRIDE < step_end)
+        ATT_ONE_STEP(r % (CL_PREFETCH + 1), base + r * ATT_WSTRIDE, base + (r + CL_PREFETCH) * ATT_WSTRIDE < step_end)
   }
 
-  // ---- merge the workgroup's waves through LDS ----------------------------------------------
   l_run += lane_xor(l_run, lane, 16);
   l_run += lane_xor(l_run, lane, 32);
+#if CL_WAVES == 1 && !CL_CHUNK_PAGES
+  // ---- one wave: its rows leave straight from the accumulators (lane (c, g) holds, of row c, the
+  // eight neighbours from 128 vc + 32 g + 8 r on for every r) ----------------------------------
+  if (c < u.rows) {
+    const i64 orow = u.out_row + c;
+#if CL_SPLITS > 1
+    const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
+    float* dst = CL_ARG_PO + prow * CL_VDIM;
+#else
+    elem_t* dst = CL_ARG_OUT + orow * CL_VDIM;
+    const float inv_l = 1.0f / fmaxf(l_run, 1.0e-30f);     // an empty request has l == 0: 0 / floor = 0
+#endif
+#pragma unroll
+    for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int d0 = 128 * vc + 32 * g + 8 * r;
+        if (CL_VDIM % 128 != 0 && d0 >= CL_VDIM) continue;
+#if CL_SPLITS > 1
+        *reinterpret_cast<f32x4*>(dst + d0) = (f32x4){acc[vc][0][r], acc[vc][1][r], acc[vc][2][r], acc[vc][3][r]};
+        *reinterpret_cast<f32x4*>(dst + d0 + 4) = (f32x4){acc[vc][4][r], acc[vc][5][r], acc[vc][6][r], acc[vc][7][r]};
+#else
+        elem8 y;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = to_elem(acc[vc][j][r] * inv_l);
+        *reinterpret_cast<elem8*>(dst + d0) = y;
+#endif
+      }
+    if (g == 0) {
+#if CL_SPLITS > 1
+      CL_ARG_PM[prow] = m_run;
+      CL_ARG_PL[prow] = l_run;
+#elif CL_EMIT_LSE
+      CL_ARG_LSE[orow] = l_run > 0.f ? m_run + fast_log2(l_run) : CL_NEG_INF;
+#endif
+    }
+  }
+#else
+  // ---- merge the workgroup's waves through LDS ----------------------------------------------
   extern __shared__ float att_lds[];
   float* sh_m = att_lds;                               // [WAVES][16]
   float* sh_l = att_lds + CL_WAVES * 16;               // [WAVES][16]
@@ -405,6 +491,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
   }
 #endif  // CL_CHUNK_PAGES
+#endif  // one wave / merge
 }
 #endif  // CL_EMIT_PARTIAL
 

@@ -20,6 +20,13 @@ def matmul(x: cl.Tensor["M", "K"], w: cl.Tensor["K", "N"]):
 
 
 @cleave_amd.jit
+def matmul_nt(x: cl.Tensor["M", "K"], w: cl.Tensor["N", "K"]):
+    """``x @ w.T`` with the weight stored (N, K), the layout of a linear layer's weight: both operands
+    are contraction-minor (the reference's ``trans_B``, ``python/cleave/ir/ops/reduction.py:146-188``)."""
+    return x @ w.mT
+
+
+@cleave_amd.jit
 def batched_matmul(x: cl.Tensor["BX", "M", "K"], w: cl.Tensor["BW", "K", "N"]):
     """``x @ w`` per batch entry; ``BX`` may be a whole multiple of ``BW`` (entries of ``w`` shared by
     groups of ``x``).  Split over K it is the reference's ``batched_matmul_splitk_partial`` /
@@ -146,6 +153,19 @@ def inputs_c1(shapes, seed=1, device="cpu"):
     x = (torch.rand(M, K, generator=g) * 2 - 1) / math.sqrt(K)
     w = (torch.rand(K, N, generator=g) * 2 - 1) / math.sqrt(K)
     return [x.to(torch.float16).to(device), w.to(torch.float16).to(device)]
+
+
+def inputs_nt(shapes, seed=17, device="cpu", dtype=torch.float16):
+    """x (M, K) and the weight as (N, K), both U(-1, 1) / sqrt(K)."""
+    g = _gen(seed)
+    M, N, K = shapes["M"], shapes["N"], shapes["K"]
+    x = (torch.rand(M, K, generator=g) * 2 - 1) / math.sqrt(K)
+    w = (torch.rand(N, K, generator=g) * 2 - 1) / math.sqrt(K)
+    return [x.to(dtype).to(device), w.to(dtype).to(device)]
+
+
+def inputs_nt_bf16(shapes, seed=18, device="cpu"):
+    return inputs_nt(shapes, seed=seed, device=device, dtype=torch.bfloat16)
 
 
 def inputs_batched(shapes, seed=14, device="cpu"):
