@@ -481,7 +481,9 @@ class HipCodeGen:
                 grid = (items, 1, 1)
             else:
                 grid = (f"({units}) * {row_tiles}", splits, 1)
-            unit.launch(ENTRY, grid, waves * 64, attn_lds_bytes(waves, p["vdim"]), self._partial_args)
+            # (a wave that shares its rows with no other stores straight from its accumulators: no LDS)
+            lds = 0 if waves == 1 or chunk_pages else attn_lds_bytes(waves, p["vdim"])
+            unit.launch(ENTRY, grid, waves * 64, lds, self._partial_args)
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv({grid_rows} * {p['vdim'] // 4}, 256)", 1, 1), 256, 0, args)

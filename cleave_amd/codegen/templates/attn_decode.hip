@@ -388,12 +388,17 @@ _Pragma("unroll")                                                               
 
   l_run += lane_xor(l_run, lane, 16);
   l_run += lane_xor(l_run, lane, 32);
-#if CL_WAVES == 1 && !CL_CHUNK_PAGES
-  // ---- one wave: its rows leave straight from the accumulators (lane (c, g) holds, of row c, the
-  // eight neighbours from 128 vc + 32 g + 8 r on for every r) ----------------------------------
+#if CL_WAVES == 1 || CL_CHUNK_PAGES
+  // ---- a wave that shares its rows with no other (one-wave workgroups; chunked items, where every
+  // wave owns one kv head): the rows leave straight from the accumulators (lane (c, g) holds, of row
+  // c, the eight neighbours from 128 vc + 32 g + 8 r on for every r) -----------------------------
   if (c < u.rows) {
     const i64 orow = u.out_row + c;
-#if CL_SPLITS > 1
+#if CL_CHUNK_PAGES
+    const i64 prow = (i64)item * CL_Q_HEADS + (i64)head * CL_ROWS + c;      // partials are (item, query head[, d])
+    float* dst = CL_ARG_PO + prow * CL_VDIM;
+    (void)orow;
+#elif CL_SPLITS > 1
     const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
     float* dst = CL_ARG_PO + prow * CL_VDIM;
 #else
@@ -406,7 +411,7 @@ _Pragma("unroll")                                                               
       for (int r = 0; r < 4; ++r) {
         const int d0 = 128 * vc + 32 * g + 8 * r;
         if (CL_VDIM % 128 != 0 && d0 >= CL_VDIM) continue;
-#if CL_SPLITS > 1
+#if CL_SPLITS > 1 || CL_CHUNK_PAGES
         *reinterpret_cast<f32x4*>(dst + d0) = (f32x4){acc[vc][0][r], acc[vc][1][r], acc[vc][2][r], acc[vc][3][r]};
         *reinterpret_cast<f32x4*>(dst + d0 + 4) = (f32x4){acc[vc][4][r], acc[vc][5][r], acc[vc][6][r], acc[vc][7][r]};
 #else
@@ -417,7 +422,7 @@ _Pragma("unroll")                                                               
 #endif
       }
     if (g == 0) {
-#if CL_SPLITS > 1
+#if CL_SPLITS > 1 || CL_CHUNK_PAGES
       CL_ARG_PM[prow] = m_run;
       CL_ARG_PL[prow] = l_run;
 #elif CL_EMIT_LSE
@@ -446,21 +451,6 @@ _Pragma("unroll")                                                               
       }
   __syncthreads();
 
-#if CL_CHUNK_PAGES
-  // each wave owns one head: its rows leave through its own LDS slab, nothing is merged here
-  {
-    const i64 prow0 = (i64)item * CL_Q_HEADS + (i64)head * CL_ROWS;
-    for (int idx = lane; idx < CL_ROWS * (CL_VDIM / 4); idx += 64) {
-      const int row = idx / (CL_VDIM / 4), d = (idx % (CL_VDIM / 4)) * 4;
-      *reinterpret_cast<f32x4*>(CL_ARG_PO + (prow0 + row) * CL_VDIM + d) =
-          *reinterpret_cast<const f32x4*>(sh_o + (wave * 16 + row) * CL_VDIM + d);
-    }
-    if (lane < CL_ROWS) {
-      CL_ARG_PM[prow0 + lane] = sh_m[wave * 16 + lane];
-      CL_ARG_PL[prow0 + lane] = sh_l[wave * 16 + lane];
-    }
-  }
-#else
   for (int idx = threadIdx.x; idx < 16 * CL_VDIM; idx += CL_WAVES * 64) {
     const int row = idx / CL_VDIM, d = idx % CL_VDIM;
     if (row >= u.rows) continue;
@@ -490,7 +480,6 @@ _Pragma("unroll")                                                               
 #endif
 #endif
   }
-#endif  // CL_CHUNK_PAGES
 #endif  // one wave / merge
 }
 #endif  // CL_EMIT_PARTIAL

@@ -44,6 +44,10 @@ class DenseAttention:
     # `waves` is then the kv-head count) instead of `split` equal parts per request.  -1 lets the
     # launch choose the size from the page-table length so that one item lands on each compute unit.
     chunk_pages: int = 0
+    # Fixed-split form only, 0 = off: a request's splits are spread over the XCDs and of every pair of
+    # neighbouring splits the one on the even XCD takes this many thousandths of the pair's steps
+    # from the other (the template's CL_SKEW).
+    skew: int = 0
 
 
 @dataclass(frozen=True)
@@ -105,7 +109,8 @@ def read_dense_attention(plan: KernelPlan) -> DenseAttention:
     waves = int(plan.tiling.get("WAVES", 4))
     return DenseAttention(query_rows=-(-rows // 16) * 16, kv_tile=KV_STEP, head_dim=p["head_dim"],
                           n_threads=waves * 64, dtype=plan.dtype, out_dtype=plan.dtype, waves=waves,
-                          split=plan.split_factor, prefetch=int(plan.tiling.get("PREFETCH", 1)))
+                          split=plan.split_factor, prefetch=int(plan.tiling.get("PREFETCH", 1)),
+                          skew=int(plan.tiling.get("SKEW", 0)))
 
 
 def read_dense_partial(plan: KernelPlan):
@@ -190,6 +195,9 @@ def _plan(spec, dense, role, params, operands, split=None) -> KernelPlan:
     if dense.chunk_pages and split:
         tiling.update(WAVES=spec.num_kv_heads, CHUNK_PAGES=dense.chunk_pages)
         extra["derived_dims"] = [("chunk_pages", chunk_pages_expr(spec, dense.chunk_pages))]
+    elif dense.skew and split and split % 2 == 0 and role != "combine" \
+            and (spec.num_kv_heads * (-(-dense.query_rows // 16))) % 8 == 0:
+        tiling["SKEW"] = dense.skew
     return KernelPlan(template="attn_decode", role=role, family="attention", dtype=dense.dtype, extra=extra,
                       problem=_paged_problem(spec, dense), tiling=tiling, params=params,
                       operands=operands, split_factor=split, dyn_dims=dyn, n_threads=dense.n_threads, label=label)

@@ -147,13 +147,26 @@ def _load_reference(reference_cache_dir, device: str = "cuda", with_mode: bool =
 
 
 def _comparable(outputs, mode):
-    if mode != "softmax_partial":
+    if mode not in ("softmax_partial", "softmax_partial_folded"):
         return list(outputs)
     import torch
 
     pm, pl, po = (t.float() for t in outputs)
+    if mode == "softmax_partial_folded":
+        # a kernel that cuts the keys into ranges of its own (every key in exactly one of them): what
+        # does not depend on the cut is the fold of all ranges, the quantity the combine makes of them
+        m = pm.amax(0, keepdim=True)
+        f = torch.exp2(pm - m)
+        pm, pl, po = m[0], (pl * f).sum(0), (po * f.unsqueeze(-1)).sum(0)
     lse = torch.where(pl > 0, pm + torch.log2(pl.clamp_min(1e-30)), torch.full_like(pm, -1.0e30))
     return [lse, po / pl.clamp_min(1e-30).unsqueeze(-1)]
+
+
+def own_cut(kernel) -> bool:
+    """Whether a split kernel deals the keys out to its ranges by a rule of its own (the skewed
+    ranges of the streaming decode kernel) rather than in equal shares."""
+    tiling = getattr(kernel, "manifest", {}).get("tiling") or {}
+    return bool(tiling.get("SKEW"))
 
 
 def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance = DEFAULT_TOLERANCE,
@@ -169,6 +182,8 @@ def _validate_kernel_outputs(kernel, inputs, reference, *, tolerance: Tolerance 
     if len(produced) != len(reference):
         raise AssertionError(f"Kernel returned {len(produced)} outputs but the reference has {len(reference)}.")
     expected = [reconcile_output_layout(want, got.shape).to(got.device) for got, want in zip(produced, reference)]
+    if compare == "softmax_partial" and own_cut(kernel):
+        compare = "softmax_partial_folded"
     for got, want in zip(_comparable(produced, compare), _comparable(expected, compare)):
         torch.testing.assert_close(got.float(), want.float().to(got.device), rtol=tolerance.rtol,
                                    atol=tolerance.atol, equal_nan=tolerance.equal_nan)

@@ -373,15 +373,24 @@ def attn_candidates(low, role, factor, arch: Arch, waves_options=(1, 2, 4, 8)):
         steps_per_wave = _ceil(_ceil(steps, splits), waves)
         waves_live = min(blocks, per_cu * arch.compute_units) * min(waves, _ceil(steps, splits))
         inflight = waves_live * 2 * kv_regs * 64 * 4 / 2
-        bw_frac = min(1.0, inflight / (12 * 1024 * 1024))
+        # (measured on the 8192-key decode: 512 one-wave workgroups with one 16 KB step in flight each stream at
+        # the rate of the box; two and four waves per workgroup take 7 % and 20 % longer)
+        bw_frac = min(1.0, inflight / (8 * 1024 * 1024))
         bytes_total = p["units"] * row_tiles * p["skv"] * (d + vd) * 2
-        stream_us = bytes_total / (arch.hbm_gbps * 1e3 * bw_frac)
-        ramp_us = 1.5 + 0.02 * steps_per_wave * 0  # fixed launch + drain cost
+        stream_us = bytes_total / (arch.hbm_gbps * 1e3 * bw_frac) * (1.0 + 0.07 * math.log2(waves) ** 1.5)
+        ramp_us = 1.5                                    # fixed launch + drain cost
         partial_us = (2 * splits * p["units"] * rows * (vd + 2) * 4) / (arch.hbm_gbps * 1e3) if splits > 1 else 0.0
         score = (stream_us * (1.0 + 0.2 * (passes - 1)) + ramp_us + partial_us + 0.05 * waves) * 2400
         tiling = dict(WAVES=waves)
         out.append(TileDict("attn_decode", role, tiling, output_tile=[16, vd], rstep_map={"kv": 32},
                             n_threads=waves * 64, split_factor=factor, score=score, lds_bytes=lds, est_vgprs=vgprs))
+        # split ranges spread over the XCDs and skewed between even and odd ones (measured on the 8192-key
+        # decode: with all splits of a unit on one XCD the kernel ends with its slowest XCD, 4-5 % later)
+        if splits > 1 and splits % 2 == 0 and waves <= 2 and (p["units"] * row_tiles) % 8 == 0 and steps >= 4 * splits:
+            for skew in (30, 60):
+                out.append(TileDict("attn_decode", role, dict(WAVES=waves, SKEW=skew), output_tile=[16, vd],
+                                    rstep_map={"kv": 32}, n_threads=waves * 64, split_factor=factor,
+                                    score=score * (0.96 if skew == 30 else 0.965), lds_bytes=lds, est_vgprs=vgprs))
         # a second step of loads in flight (measured on the 8192-key decode: with about two waves per CU
         # streaming, the deeper ring is worth a few percent; with many waves it is not)
         if waves <= 2 and vgprs + kv_regs <= arch.vgprs_per_lane and steps_per_wave >= 8:

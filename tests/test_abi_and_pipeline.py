@@ -301,3 +301,39 @@ def test_saved_paged_kernel_holds_its_program_as_json(tmp_path):
     (folder / "program.pkl").write_bytes(b"not read")
     with pytest.raises(ValueError, match="pickle"):
         load(folder)
+
+
+def test_partials_of_a_kernel_that_cuts_the_keys_its_own_way_are_compared_through_their_fold():
+    """Softmax partials (m, l, O) of any partition of the keys fold to the same (lse, O / l); per split they
+    differ.  A kernel whose manifest says it skews its ranges is validated through the fold."""
+    from cleave_amd.runtime.validate import _comparable, own_cut
+
+    gen = torch.Generator().manual_seed(3)
+    s, v = torch.randn(6, 4, 512, generator=gen) * 3, torch.randn(6, 512, 64, generator=gen)
+
+    def parts(cuts):
+        pm, pl, po = [], [], []
+        for lo, hi in cuts:
+            if hi <= lo:
+                pm.append(torch.full((6, 4), -1.0e30)); pl.append(torch.zeros(6, 4)); po.append(torch.zeros(6, 4, 64))
+                continue
+            blk = s[..., lo:hi]
+            m = blk.amax(-1)
+            w = torch.exp2(blk - m.unsqueeze(-1))
+            pm.append(m + 3.0); pl.append(w.sum(-1) / 8.0); po.append(w @ v[:, lo:hi] / 8.0)   # (any reference point)
+        n = len(cuts)
+        return [torch.stack(pm).reshape(n, 24), torch.stack(pl).reshape(n, 24), torch.stack(po).reshape(n, 24, 64)]
+
+    equal = parts([(0, 128), (128, 256), (256, 384), (384, 512)])
+    skewed = parts([(0, 160), (160, 256), (256, 512), (512, 512)])
+    for a, b in zip(_comparable(equal, "softmax_partial_folded"), _comparable(skewed, "softmax_partial_folded")):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-5)
+    per_split = [float((a - b).abs().max()) for a, b in zip(_comparable(equal, "softmax_partial"), _comparable(skewed, "softmax_partial"))]
+    assert max(per_split) > 0.1
+    whole = torch.softmax(s * 0.6931471805599453, -1) @ v
+    torch.testing.assert_close(_comparable(skewed, "softmax_partial_folded")[1], whole.reshape(24, 64), rtol=1e-4, atol=1e-4)
+
+    class K:
+        manifest = {"tiling": {"WAVES": 1, "SKEW": 30}}
+
+    assert own_cut(K) and not own_cut(type("P", (), {"manifest": {"tiling": {"WAVES": 1}}}))

@@ -281,6 +281,53 @@ def test_gqa_decode_c3_full(split):
     _check(fn.trace(dt, **C.FULL["c3"]), mk, C.FULL["c3"], template="attn_decode", tiling=dict(WAVES=4), split=split)
 
 
+@pytest.mark.parametrize("tiling,split", [(dict(WAVES=1, SKEW=30), 8), (dict(WAVES=1, SKEW=60), 8), (dict(WAVES=1, SKEW=30), 16),
+                                          (dict(WAVES=2, SKEW=500), 8), (dict(WAVES=1, PREFETCH=2, SKEW=30), 32),
+                                          (dict(WAVES=1, PREFETCH=3), 8)],
+                         ids=lambda v: "x".join(f"{k}{x}" for k, x in v.items()) if isinstance(v, dict) else str(v))
+def test_gqa_decode_c3_full_with_ranges_skewed_between_xcds(tiling, split):
+    """The plans the search ranks first: a unit's splits rotated over the XCDs and the split ranges
+    skewed (3 %, 6 %, and all of a pair's steps to one of its two splits), deeper load rings."""
+    fn, dt, mk = C.CASES["c3"]
+    _check(fn.trace(dt, **C.FULL["c3"]), mk, C.FULL["c3"], template="attn_decode", tiling=tiling, split=split)
+
+
+@pytest.mark.parametrize("skv", [48, 432, 1008, 2064])
+def test_gqa_decode_skewed_ranges_own_every_step_once(skv):
+    """Key counts that leave pairs of splits with an odd number of steps, a single step, or none; 16 units so
+    that the grid is whole groups of eight; every prefetch depth's straight-line tail."""
+    shapes = dict(HQ=64, HKV=16, SQ=1, SKV=skv, D=128)
+    prog = C.gqa_decode_exact.trace(C.cl.f16, **shapes)
+    for tiling, split in ((dict(WAVES=1, SKEW=30), 2), (dict(WAVES=1, SKEW=250), 4), (dict(WAVES=2, SKEW=60), 8),
+                          (dict(WAVES=1, PREFETCH=2, SKEW=100), 4), (dict(WAVES=1, PREFETCH=3, SKEW=500), 6)):
+        _check(prog, C.inputs_c3, shapes, template="attn_decode", tiling=tiling, split=split)
+
+
+def test_gqa_decode_rising_maximum():
+    """Scores that grow along the KV axis raise every row's softmax reference point several times inside a
+    split (the cold path: a ballot, a cross-lane maximum, a rescale of sums and accumulators with a factor
+    strictly between 0 and 1), in every form of the streaming kernel: one to eight waves, split and
+    unsplit, skewed ranges, deeper rings."""
+    shapes = dict(HQ=64, HKV=16, SQ=1, SKV=1536, D=128)
+    prog = C.gqa_decode_exact.trace(C.cl.f16, **shapes)
+    q, k, v = C.inputs_c3(shapes, device="cpu")
+    # k gains a component along q's direction that grows with the position: the scaled scores climb by
+    # ~35 (log2 domain) over the keys, in steps far smaller than the raise threshold
+    ramp = torch.linspace(0.0, 48.0, shapes["SKV"]).reshape(1, -1, 1)
+    qdir = q.float().reshape(16, 4, 1, 128).mean(1)
+    k = (k.float() * 0.3 + ramp * qdir / qdir.norm(dim=-1, keepdim=True)).to(k.dtype)
+    ins = [q, k, v]
+    want = po.evaluate(prog, ins)[0]
+    spread = (q.float().reshape(16, 4, 128) @ k.float().mT / 128 ** 0.5)
+    assert float((spread[..., -1] - spread[..., 0]).abs().mean()) * 1.4427 > 3 * 8, "the ramp must pass the raise threshold often"
+    for tiling, split in ((dict(WAVES=1), None), (dict(WAVES=4), None), (dict(WAVES=8), 2), (dict(WAVES=1, SKEW=60), 4),
+                          (dict(WAVES=2, PREFETCH=2), 2), (dict(WAVES=1, PREFETCH=3), None)):
+        kernel = kernel_for(prog, template="attn_decode", tiling=tiling, split=split)
+        print(f"case gqa rising maximum {tiling} split={split}", flush=True)
+        got = kernel(*[t.cuda() for t in ins]).float().cpu().numpy().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("split", [None, 2])
 def test_mla_decode_small(split):
     fn, dt, mk = C.CASES["c4"]
