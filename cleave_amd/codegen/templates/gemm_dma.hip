@@ -158,11 +158,16 @@ struct GdOperand {
     }
   }
 
-  // issue this wave's i-th load of one K step; `base`: the tile's first element of this step (uniform)
-  CL_METHOD void issue_unit(int i, const elem_t* base, elem_t* lds) const {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // scalar: the LDS target goes to M0
-    const int u = wave + i * GD_WAVES;
+  // issue this wave's i-th load of one K step; `base`: the tile's first element of this step (uniform),
+  // `lds_byte`: the LDS byte address of the stage's image (a link-time constant: the images are static
+  // arrays), `wave_byte`: 1024 * the wave's index in a scalar register.  The LDS target of a load goes to
+  // M0 as one scalar add; formed from a generic pointer to the image it cost eight scalar instructions per
+  // load (the cast back into the LDS address space checks for the null pointer), 128 a step ahead of the
+  // matrix work, which a wave that has its SIMD to itself cannot hide.
+  CL_METHOD void issue_unit(int i, const elem_t* base, unsigned lds_byte, unsigned wave_byte) const {
+    const int u = (threadIdx.x >> 6) + i * GD_WAVES;
     if (UNITS % GD_WAVES == 0 || u < UNITS) {
+      const unsigned m0_value = lds_byte + i * GD_WAVES * 1024 + wave_byte;
 #if CL_ASM_LOADS
       // Written as assembly (the default): the tile's first element of the step stays in scalar
       // registers and the lane's 32-bit offset goes in as it is, where the builtin forms a 64-bit
@@ -171,27 +176,26 @@ struct GdOperand {
       // compiler spill the offsets and reload them between the loads, each reload waiting for the
       // loads before it).  The load is then not counted by the compiler; the kernel's own
       // vmcnt(0) at the end of a step covers it.  On the large matmul the two forms measure alike.
-      const unsigned lds_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)(lds + u * 512);
       if constexpr (sizeof(off_t) == 4) {
         // (scalar base + 32-bit lane offset: no 64-bit address is formed in vector registers)
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :: "v"(goff[i]), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
+                     :: "v"(goff[i]), "s"(base), "s"(m0_value)
                      : "memory", "m0");
       } else {
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     :: "v"(reinterpret_cast<const char*>(base) + goff[i]), "s"(__builtin_amdgcn_readfirstlane(lds_byte))
+                     :: "v"(reinterpret_cast<const char*>(base) + goff[i]), "s"(m0_value)
                      : "memory", "m0");
       }
 #else
       __builtin_amdgcn_global_load_lds((gd_gbl_void*)(reinterpret_cast<const char*>(base) + goff[i]),
-                                       (gd_lds_void*)(lds + u * 512), 16, 0, 0);
+                                       (gd_lds_void*)(size_t)m0_value, 16, 0, 0);
 #endif
     }
   }
   // ... all of them
-  CL_METHOD void issue(const elem_t* base, elem_t* lds) const {
+  CL_METHOD void issue(const elem_t* base, unsigned lds_byte, unsigned wave_byte) const {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) issue_unit(i, base, lds);
+    for (int i = 0; i < PER; ++i) issue_unit(i, base, lds_byte, wave_byte);
   }
 };
 
@@ -291,6 +295,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int wm = wave / CL_WN, wn = wave % CL_WN;
+  const unsigned wave_byte = (unsigned)__builtin_amdgcn_readfirstlane(wave) * 1024u;   // scalar: part of every load's LDS target
   // Workgroups are handed to the XCDs round-robin in launch order.  Renumber them so that the
   // ones an XCD runs at the same time are neighbours in C: launch id L -> the (L / 8)-th tile of
   // XCD (L % 8)'s contiguous share, tiles ordered in patches of CL_GROUP_M row-tiles.
@@ -469,17 +474,18 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define GD_A_AT(kt) (a_base + (i64)(kt) * a_step)
 #define GD_B_AT(kt) (b_base + (i64)(kt) * b_step)
 #endif
+#define GD_LDS_BYTE(image) ((unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)(image))
 #define GD_ISSUE(kt, a_lds, b_lds)                              \
-  opa.issue(GD_A_AT(kt), a_lds);                                \
-  opb.issue(GD_B_AT(kt), b_lds);                                \
+  opa.issue(GD_A_AT(kt), GD_LDS_BYTE(a_lds), wave_byte);        \
+  opb.issue(GD_B_AT(kt), GD_LDS_BYTE(b_lds), wave_byte);        \
   __builtin_amdgcn_sched_barrier(0);
 #define GD_ISSUE_SLICE(r, kt, a_lds, b_lds)                                                         \
   {                                                                                                 \
     constexpr int ua_ = decltype(opa)::PER, ub_ = decltype(opb)::PER;                               \
     constexpr int per_row_ = (ua_ + ub_ + 2 * TM - 1) / (2 * TM);                             \
     _Pragma("unroll") for (int q_ = (r) * per_row_; q_ < ((r) + 1) * per_row_; ++q_) {             \
-      if (q_ < ua_) opa.issue_unit(q_, GD_A_AT(kt), a_lds);                                         \
-      else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, GD_B_AT(kt), b_lds);                        \
+      if (q_ < ua_) opa.issue_unit(q_, GD_A_AT(kt), GD_LDS_BYTE(a_lds), wave_byte);                 \
+      else if (q_ < ua_ + ub_) opb.issue_unit(q_ - ua_, GD_B_AT(kt), GD_LDS_BYTE(b_lds), wave_byte); \
     }                                                                                               \
   }
 #define GD_NO_NEXT(r)
