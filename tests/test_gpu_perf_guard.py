@@ -6,6 +6,10 @@ catch a structural regression of a kernel or of the emitter, not drift.  The ref
 generated kernels the same way (``tests/perf/test_kernel_perf_regression.py:78-101``, threshold
 1.25 against ``tests/perf/baselines/h100-80gb-hbm3.json``, skipped on any other GPU).
 
+The nine registry operators are guarded too, as the reference guards exactly those kernels: each
+operator's shipped single kernel at its tuned tiling, timed over a sample of its captured
+workloads, the geometric mean against the record.
+
 ``CLEAVE_PERF_THRESHOLD`` overrides the allowed ratio.
 """
 
@@ -29,7 +33,7 @@ MATMUL = dict(M=4096, N=14336, K=4096)
 PLANS = {
     "c1_matmul_128x128x4096": ("c1", C.FULL["c1"], "gemm_dma", dict(BM=16, BN=32, BK=64, WM=1, WN=1), 16),
     "c2_rmsnorm_matmul_16x11008x4096": ("c2", C.FULL["c2"], "skinny", dict(WAVES_N=1, WAVES_K=2), 8),
-    "c3_gqa_decode_256h_8192": ("c3", C.FULL["c3"], "attn_decode", dict(WAVES=1), 8),
+    "c3_gqa_decode_256h_8192": ("c3", C.FULL["c3"], "attn_decode", dict(WAVES=1, SKEW=30), 8),
     "c4_mla_decode_16x128h_4096": ("c4", C.FULL["c4"], "mla_decode", dict(DUO=1, LDS_AHEAD=4), 8),
     "matmul_4096x14336x4096": ("c1", MATMUL, "gemm_dma", dict(BM=256, BN=256, BK=64, WM=4, WN=2, TAIL=128), None),
     "attention_32h_4096_d64": ("c3", ATTENTION, "attn_prefill", dict(SHARED=1), None),
@@ -65,3 +69,46 @@ def test_fixed_plan_latency(name, record):
     ratio = us / record[name]["us"]
     print(f"{name}: recorded {record[name]['us']:.1f} us, now {us:.1f} us ({ratio:.2f}x)", flush=True)
     assert ratio <= THRESHOLD, f"{name}: {us:.1f} us against the recorded {record[name]['us']:.1f} us ({ratio:.2f}x > {THRESHOLD}x)"
+
+
+REGISTRY_WORKLOADS = 4        # workloads sampled per operator (first and last included)
+
+
+def _registry_geomean(name):
+    from cleave_amd.dynamic import OPERATORS
+    from cleave_amd.runtime.autotune import geomean, time_kernel
+    from cleave_amd.runtime.compile import _compile, _load_main_kernel_from_code
+
+    op = OPERATORS[name]
+    loaded = _load_main_kernel_from_code(op.kernel_source())
+    kernel = _compile(loaded, loaded.manifest["out_idx"])
+    times = {}
+    for key, inputs, expected in op.keyed_workloads(keep=REGISTRY_WORKLOADS, dtype=torch.bfloat16)():
+        got = kernel(*inputs)
+        got = list(got) if isinstance(got, (list, tuple)) else [got]
+        torch.cuda.synchronize()
+        # (a guard of speed still refuses a kernel that has stopped being right)
+        torch.testing.assert_close(got[0].float(), expected[0].float().to(got[0].device), rtol=2e-2, atol=2e-2)
+        times[key] = time_kernel(kernel, inputs, warmup=10, iters=20, repeats=3)[0]
+        del inputs, expected, got
+        torch.cuda.empty_cache()
+    return geomean(list(times.values())), times
+
+
+def _registry_names():
+    from cleave_amd.dynamic import OPERATORS
+
+    return sorted(OPERATORS)
+
+
+@pytest.mark.parametrize("name", _registry_names())
+def test_registry_operator_latency(name, record):
+    """Geometric mean over the sampled captured workloads of the operator's shipped kernel
+    (``python/cleave/dynamic/registry.py:91-196`` names the same nine)."""
+    print(f"case perf guard registry {name}", flush=True)
+    now, times = _registry_geomean(name)
+    want = record[name]["us"]
+    ratio = now / want
+    print(f"{name}: recorded geomean {want:.2f} us, now {now:.2f} us ({ratio:.2f}x); " +
+          " ".join(f"{k}={v:.1f}" for k, v in times.items()), flush=True)
+    assert ratio <= THRESHOLD, f"{name}: geomean {now:.2f} us against the recorded {want:.2f} us ({ratio:.2f}x > {THRESHOLD}x)"
