@@ -388,10 +388,56 @@ _Pragma("unroll")                                                               
 
   l_run += lane_xor(l_run, lane, 16);
   l_run += lane_xor(l_run, lane, 32);
-#if CL_WAVES == 1 || CL_CHUNK_PAGES
-  // ---- a wave that shares its rows with no other (one-wave workgroups; chunked items, where every
-  // wave owns one kv head): the rows leave straight from the accumulators (lane (c, g) holds, of row
-  // c, the eight neighbours from 128 vc + 32 g + 8 r on for every r) -----------------------------
+#if CL_WAVES > 1 && !CL_CHUNK_PAGES
+  // ---- the workgroup's waves merged into its first one through LDS: every other wave leaves its
+  // reference points, weight sums and accumulators as they lie in its registers (one 16-byte piece
+  // per lane and accumulator: whole 1 KiB rows), and the first wave folds them into its own by the
+  // max-rescale rule: one LDS round trip for all of them --------------------------------------
+  {
+    extern __shared__ float att_lds[];
+    f32x4* sh_o = reinterpret_cast<f32x4*>(att_lds);                          // [WAVES - 1][8 ATT_VC][64]
+    float* sh_m = att_lds + (CL_WAVES - 1) * 8 * ATT_VC * 64 * 4;              // [WAVES - 1][16]
+    float* sh_l = sh_m + (CL_WAVES - 1) * 16;                                  // [WAVES - 1][16]
+    if (wave > 0) {
+#pragma unroll
+      for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sh_o[((wave - 1) * 8 * ATT_VC + 8 * vc + j) * 64 + lane] = acc[vc][j];
+      if (g == 0) {
+        sh_m[(wave - 1) * 16 + c] = m_run;
+        sh_l[(wave - 1) * 16 + c] = l_run;
+      }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float ms[CL_WAVES - 1], m = m_run;
+#pragma unroll
+    for (int w = 0; w < CL_WAVES - 1; ++w) {
+      ms[w] = sh_m[w * 16 + c];
+      m = fmaxf(m, ms[w]);
+    }
+    // (a wave without steps holds m = -huge, l = 0, zeros: factor 1 of nothing when every wave is empty)
+    const float f0 = fast_exp2(m_run - m);
+    l_run *= f0;
+#pragma unroll
+    for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[vc][j] *= f0;
+#pragma unroll
+    for (int w = 0; w < CL_WAVES - 1; ++w) {
+      const float f = fast_exp2(ms[w] - m);
+      l_run += sh_l[w * 16 + c] * f;
+#pragma unroll
+      for (int vc = 0; vc < ATT_VC; ++vc)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[vc][j] += sh_o[(w * 8 * ATT_VC + 8 * vc + j) * 64 + lane] * f;
+    }
+    m_run = m;
+  }
+#endif
+  // ---- the rows leave straight from the accumulators of the wave that owns them (the first wave of
+  // a workgroup; every wave of a chunked item, which owns one kv head): lane (c, g) holds, of row c,
+  // the eight neighbours from 128 vc + 32 g + 8 r on for every r --------------------------------
   if (c < u.rows) {
     const i64 orow = u.out_row + c;
 #if CL_CHUNK_PAGES
@@ -430,57 +476,7 @@ _Pragma("unroll")                                                               
 #endif
     }
   }
-#else
-  // ---- merge the workgroup's waves through LDS ----------------------------------------------
-  extern __shared__ float att_lds[];
-  float* sh_m = att_lds;                               // [WAVES][16]
-  float* sh_l = att_lds + CL_WAVES * 16;               // [WAVES][16]
-  float* sh_o = att_lds + CL_WAVES * 32;               // [WAVES][16][VDIM]
-  if (g == 0) {
-    sh_m[wave * 16 + c] = m_run;
-    sh_l[wave * 16 + c] = l_run;
-  }
-#pragma unroll
-  for (int vc = 0; vc < ATT_VC; ++vc)
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int d = 128 * vc + 32 * g + 8 * r + j;
-        if (CL_VDIM % 128 == 0 || d < CL_VDIM) sh_o[(wave * 16 + c) * CL_VDIM + d] = acc[vc][j][r];
-      }
-  __syncthreads();
 
-  for (int idx = threadIdx.x; idx < 16 * CL_VDIM; idx += CL_WAVES * 64) {
-    const int row = idx / CL_VDIM, d = idx % CL_VDIM;
-    if (row >= u.rows) continue;
-    float m = sh_m[row];
-#pragma unroll
-    for (int w = 1; w < CL_WAVES; ++w) m = fmaxf(m, sh_m[w * 16 + row]);
-    float l = 0.f, o = 0.f;
-#pragma unroll
-    for (int w = 0; w < CL_WAVES; ++w) {
-      const float f = fast_exp2(sh_m[w * 16 + row] - m);
-      l += sh_l[w * 16 + row] * f;
-      o += sh_o[(w * 16 + row) * CL_VDIM + d] * f;
-    }
-    const i64 orow = u.out_row + row;
-#if CL_SPLITS > 1
-    const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
-    CL_ARG_PO[prow * CL_VDIM + d] = o;
-    if (d == 0) {
-      CL_ARG_PM[prow] = m;
-      CL_ARG_PL[prow] = l;
-    }
-#else
-    // An empty request has l == 0: the floor turns 0/0 into 0 and its lse is -inf.
-    CL_ARG_OUT[orow * CL_VDIM + d] = to_elem(o / fmaxf(l, 1.0e-30f));
-#if CL_EMIT_LSE
-    if (d == 0) CL_ARG_LSE[orow] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
-#endif
-#endif
-  }
-#endif  // one wave / merge
 }
 #endif  // CL_EMIT_PARTIAL
 

@@ -341,7 +341,9 @@ def skinny_candidates(low, role, factor, arch: Arch):
 
 # ----------------------------------------------------------------------------- decode attention
 def attn_lds_bytes(waves, vdim):
-    return waves * (32 + 16 * vdim) * 4
+    """LDS of the streaming decode kernel: every wave but the first parks its accumulators (a 16-byte piece per
+    lane and accumulator, eight accumulators per 128 value features) and its 16 reference points and sums."""
+    return (waves - 1) * (-(-vdim // 128) * 8 * 64 * 16 + 128)
 
 
 def attn_ok(low) -> bool:
