@@ -296,12 +296,12 @@ def run_paged(steps, warmup, with_cpu, kernels_dir=None):
     best = None
     tried = valid = 0
     saved = saved_choice(kernels_dir, "c5")
-    configs = [dict(waves=w, split=sp, skew=sk) for w in (1, 2) for sp in (8, 16) for sk in (0, 30)]
-    configs += [dict(waves=hkv, split=8, chunk_pages=cp, prefetch=pf) for cp in (8, 16, -1) for pf in (1,)]
+    configs = [dict(waves=w, split=16, skew=sk) for w in (1, 2) for sk in (0, 30)]
+    configs += [dict(waves=hkv, split=8, chunk_pages=cp, lockstep=ls) for cp in (8, 16, -1) for ls in (False, True)]
     for cfg in configs if saved is None else ():
         dense = DenseAttention(16, 32, d, cfg["waves"] * 64, "float16", "float16", waves=cfg["waves"],
                                chunk_pages=cfg.get("chunk_pages", 0), prefetch=cfg.get("prefetch", 1),
-                               skew=cfg.get("skew", 0))
+                               skew=cfg.get("skew", 0), lockstep=cfg.get("lockstep", False))
         src = HipCodeGen().gen(build_split_decode(spec, dense, cfg["split"], CombineTiling(split=cfg["split"])))
         loaded = _load_main_kernel_from_code(src)
         k = _compile(loaded, loaded.manifest["out_idx"])

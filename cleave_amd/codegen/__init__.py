@@ -450,6 +450,10 @@ class HipCodeGen:
         unit.define("CL_PREFETCH", int(t.get("PREFETCH", 1)))
         chunk_pages = bool(t.get("CHUNK_PAGES", 0)) and paged and (plan.split_factor or 1) > 1
         unit.define("CL_CHUNK_PAGES", chunk_pages)
+        if int(t.get("LOCKSTEP", 0)):
+            if not chunk_pages:
+                raise CodegenError("LOCKSTEP (a barrier per step between the waves of a workgroup) exists for chunked items only")
+            unit.define("CL_LOCKSTEP", 1)
         skew = int(t.get("SKEW", 0))
         if skew:
             # the rotation of units over the XCDs assumes that launch index % 8 is blockIdx.x % 8

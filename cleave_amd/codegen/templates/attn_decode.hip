@@ -43,6 +43,17 @@
 #ifndef CL_SKEW
 #define CL_SKEW 0
 #endif
+#ifndef CL_LOCKSTEP
+#define CL_LOCKSTEP 0
+#endif
+#if CL_LOCKSTEP && !CL_CHUNK_PAGES
+#error "waves in step: chunked items only (every wave walks the same steps)"
+#endif
+#if CL_LOCKSTEP
+#define ATT_LOCKSTEP() __builtin_amdgcn_s_barrier();
+#else
+#define ATT_LOCKSTEP()
+#endif
 #if CL_SKEW && (CL_CHUNK_PAGES || CL_SPLITS % 2)
 #error "skewed split ranges: an even number of splits, no chunked items"
 #endif
@@ -309,11 +320,17 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 // slots hold CL_NEG_BIG; while a whole row is still masked its reference equals it too, so the weights
 // test the mask itself rather than trusting exp2 of a zero difference.  The row sum adds up the weights
 // as rounded to the element type, the ones the value product really sees.
+// CL_LOCKSTEP (chunked items): the waves of a workgroup, one per kv head, meet at a barrier before every
+// step.  Left alone they drift apart (the older wave of a SIMD is served first: in a 1024-token item the
+// first wave is done after 88 us, the last after 155) and the item is as slow as its slowest wave; in step,
+// the eight 256-byte pieces of a token row are also asked for together.  Every wave of an item walks the same
+// steps, so every wave reaches every barrier.
 // (A macro, so that the loop below holds no branch out of its body: with one, the compiler must assume
 // at the loop head that loads of the skipped part are still on their way into registers it is about to
 // reuse for addresses, and it waits for the current tile before it asks for the next.)
 #define ATT_ONE_STEP(R, STEP, LOAD)                                                                 \
     {                                                                                               \
+      ATT_LOCKSTEP()                                                                                \
       if (LOAD) att_load(u, ((STEP) + CL_PREFETCH * ATT_WSTRIDE) * ATT_STEP, c, g, ring[((R) + CL_PREFETCH) % (CL_PREFETCH + 1)]); \
       const AttTile& cur = ring[R];                                                                 \
       const int t0 = (STEP) * ATT_STEP;                                                             \

@@ -48,6 +48,8 @@ class DenseAttention:
     # neighbouring splits the one on the even XCD takes this many thousandths of the pair's steps
     # from the other (the template's CL_SKEW).
     skew: int = 0
+    # Chunked items only: the waves of a workgroup (one per kv head) meet at a barrier before every step.
+    lockstep: bool = False
 
 
 @dataclass(frozen=True)
@@ -194,6 +196,8 @@ def _plan(spec, dense, role, params, operands, split=None) -> KernelPlan:
     extra = {}
     if dense.chunk_pages and split:
         tiling.update(WAVES=spec.num_kv_heads, CHUNK_PAGES=dense.chunk_pages)
+        if dense.lockstep and role != "combine":
+            tiling["LOCKSTEP"] = 1
         extra["derived_dims"] = [("chunk_pages", chunk_pages_expr(spec, dense.chunk_pages))]
     elif dense.skew and split and split % 2 == 0 and role != "combine" \
             and (spec.num_kv_heads * (-(-dense.query_rows // 16))) % 8 == 0:

@@ -286,3 +286,27 @@ def test_widths_only_the_many_row_kernel_takes():
     # decode-shaped units of that width have no other kernel either
     _check(C.gqa_decode_exact, cl.f16, dict(HQ=8, HKV=2, SQ=1, SKV=1000, D=192), template=None)
     _check(C.gqa_decode_exact, cl.f16, dict(HQ=8, HKV=2, SQ=3, SKV=1024, D=192), template=None, split=8)
+
+
+def test_rising_maximum_in_the_many_row_kernel():
+    """Scores that grow along the key axis: every row's softmax reference point is raised several times
+    on the way (the cold path of the kernel whose waves share the key tiles: a ballot, a maximum over the
+    key groups, sums and accumulators rescaled by a factor strictly between 0 and 1), unsplit and split over
+    the keys, 64 and 128 wide."""
+    for d, split in ((64, None), (128, None), (128, 4), (64, 2)):
+        shapes = dict(HQ=8, HKV=2, SQ=160, SKV=1536, D=d)
+        prog = C.gqa_decode_exact.trace(cl.f16, **shapes)
+        q, k, v = [t.cpu() for t in prog.random_inputs(seed=23)]
+        # feature 0 of every query is 4 and feature 0 of the keys climbs with the position: every row's scaled
+        # scores climb by about 35 (log2 domain) over the keys, in steps far below the raise threshold
+        q[..., 0] = 4.0
+        k[..., 0] = torch.linspace(0.0, 35.0 * d ** 0.5 / (4 * 1.4427), shapes["SKV"]).reshape(1, -1).to(k.dtype)
+        scores = (q.float().reshape(2, 640, d) @ k.float().mT) / d ** 0.5 * 1.4427
+        climbs = scores[..., -32:].mean(-1) - scores[..., :32].mean(-1)
+        want = program_oracle.evaluate(prog, [q, k, v])[0]
+        how = dict(template="attn_prefill", tiling=dict(SHARED=1), split=split)
+        print(f"dense prefill rising maximum d={d} split={split}: mean climb {float(climbs.abs().mean()):.1f} (log2)", flush=True)
+        assert float(climbs.min()) > 24.0
+        out = kernel_for(prog, **how)(q.cuda(), k.cuda(), v.cuda())
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-2)

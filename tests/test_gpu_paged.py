@@ -16,10 +16,12 @@ from cleave_amd import examples as C
 pytestmark = pytest.mark.gpu
 
 
-def paged_kernel(page_size=64, hq=32, hkv=8, d=128, waves=4, split=None, dtype="float16", chunk_pages=0, prefetch=1):
+def paged_kernel(page_size=64, hq=32, hkv=8, d=128, waves=4, split=None, dtype="float16", chunk_pages=0, prefetch=1,
+                 skew=0, lockstep=False):
     kind = PAGED_DECODE_SLAB if page_size > 1 else "paged_decode"
     spec = PagingSpec(num_qo_heads=hq, num_kv_heads=hkv, kind=kind, page_size=page_size)
-    dense = DenseAttention(16, 32, d, waves * 64, dtype, dtype, waves=waves, chunk_pages=chunk_pages, prefetch=prefetch)
+    dense = DenseAttention(16, 32, d, waves * 64, dtype, dtype, waves=waves, chunk_pages=chunk_pages, prefetch=prefetch,
+                           skew=skew, lockstep=lockstep)
     if split:
         src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split)))
     else:
@@ -57,19 +59,21 @@ def test_paged_decode_ps64(split, waves):
 
 
 @pytest.mark.parametrize("chunk_pages", [1, 4, 7, -1])
-@pytest.mark.parametrize("prefetch", [1, 2])
-def test_paged_decode_chunked_items(chunk_pages, prefetch):
+@pytest.mark.parametrize("prefetch,lockstep", [(1, False), (2, False), (1, True)])
+def test_paged_decode_chunked_items(chunk_pages, prefetch, lockstep):
     """Work cut into items of chunk_pages pages: requests that end on, before and after a chunk
-    boundary, an empty request between two others, a request inside one chunk."""
+    boundary, an empty request between two others, a request inside one chunk; with the waves of an
+    item free-running and meeting at a barrier before every step."""
     lens = [1, 63, 64, 65, 200, 777, 0, 1500, 4 * 64, 0, 3 * 64 + 1, 7 * 64 * 3]
     args = C.paged_workload(lens, page_size=64, num_pages=300)
-    check(args, lens, 64, split=8, waves=8, chunk_pages=chunk_pages, prefetch=prefetch)
+    check(args, lens, 64, split=8, waves=8, chunk_pages=chunk_pages, prefetch=prefetch, lockstep=lockstep)
 
 
 def test_paged_decode_chunked_other_head_counts():
     lens = [130, 9, 700]
     args = C.paged_workload(lens, page_size=16, num_pages=200, hq=16, hkv=4)
     check(args, lens, 16, split=4, waves=4, hq=16, hkv=4, chunk_pages=3)
+    check(args, lens, 16, split=4, waves=4, hq=16, hkv=4, chunk_pages=2, lockstep=True)
 
 
 @pytest.mark.parametrize("page_size", [1, 16])

@@ -30,7 +30,8 @@ pytestmark = pytest.mark.gpu
 POOL, PAGE, HKV, HQ, D = 300_000, 64, 8, 32, 128
 LENS = [257, 64 * 9, 1, 64 * 17 + 5, 0, 1999, 640, 64 * 30 + 63]
 FORCED = [0, 16_383, 16_384, 16_385, 32_767, 32_768, 32_769, 65_536, 131_072, 262_144, POOL - 2, POOL - 1]
-PLANS = [dict(split=8, waves=8, chunk_pages=16), dict(split=8, waves=8, chunk_pages=-1), dict(split=8, waves=4)]
+PLANS = [dict(split=8, waves=8, chunk_pages=16), dict(split=8, waves=8, chunk_pages=-1, lockstep=True), dict(split=8, waves=4),
+         dict(split=8, waves=1, skew=30)]
 
 
 def _table(seed=21):

@@ -104,5 +104,6 @@ def test_drawn_paged_decode_requests_against_the_oracle(seed):
             args = args[:5] + args[6:]
         how = dict(waves=rng.choice([1, 2, 4, 8]), split=rng.choice([None, 2, 4, 8]), hq=kv_heads * group, hkv=kv_heads)
         if how["split"] and page == 64 and rng.random() < 0.5:
-            how.update(chunk_pages=rng.choice([1, 3, 16, -1]), prefetch=rng.choice([1, 2]), waves=8)
+            how.update(chunk_pages=rng.choice([1, 3, 16, -1]), prefetch=rng.choice([1, 2]), waves=8,
+                       lockstep=rng.choice([False, True]))
         check(args, lens, page, **how)
