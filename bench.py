@@ -138,10 +138,11 @@ def roofline(bound, nbytes, flops, us, traffic=None):
 
 
 def _plan_key(plan):
-    """A plan label without the candidate's rank in its search (``#7``): ranks move between runs."""
+    """A plan label without what moves between runs and leaves the bytes a launch moves alone: the
+    candidate's rank in its search (``#7``) and how far the split ranges are skewed."""
     import re
 
-    return re.sub(r"#\d+ ", "", plan or "")
+    return re.sub(r"SKEW=\d+", "SKEW", re.sub(r"#\d+ ", "", plan or ""))
 
 
 def measured_traffic(name, plan=None):
