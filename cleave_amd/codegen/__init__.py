@@ -583,7 +583,7 @@ class HipCodeGen:
             return
         unit.templates.append("attn_prefill.hip")
         items = f"ceildiv({p['dim_names']['total_q']}, {16 // group}) + batch"
-        unit.launch(ENTRY, (items, 1, 1), p["kv_heads"] * 64, p["kv_heads"] * 16 * d * 4, self._partial_args)
+        unit.launch(ENTRY, (items, 1, 1), p["kv_heads"] * 64, 0, self._partial_args)
 
     def _emit_mla_decode(self, unit, plan, params, partial, combine, fused):
         p, t, op = plan.problem, plan.tiling, plan.operands

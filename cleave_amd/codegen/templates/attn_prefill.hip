@@ -35,6 +35,7 @@ struct PfTile {                // one 32-token step's K and V, as loaded
 };
 
 CL_DEVICE int pf_clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+template <int V> struct PfC { static constexpr int value = V; };
 
 #if CL_EMIT_PARTIAL
 extern "C" __global__ void __launch_bounds__(CL_KV_HEADS * 64)
@@ -148,25 +149,38 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       }
     };
 
-    // two register tiles: while step n is in the matrix cores the loads of step n+1 are in flight
-    // (issued unconditionally: a step past the end repeats the last one and is never consumed)
+    // Two register tiles: while step n is in the matrix cores the loads of step n + 1 are in
+    // flight.  The loop runs whole turns of the pair whose next steps both exist, with no branch
+    // in its body (with one, the waits placed at the loop head had to assume that loads of the
+    // part branched around were still on their way, and waited for the current tile before asking
+    // for the next); the last one or two steps follow as straight-line code that asks for nothing
+    // past the item's last step.
     PfTile ring[2];
     int ids_next = 0;
 #if !CL_RAGGED
-    load_tile(0, load_ids(0), ring[0]);
-    ids_next = load_ids(1);
+    {
+      const int ids_first = load_ids(0);
+      ids_next = load_ids(1);
+      load_tile(0, ids_first, ring[0]);
+    }
 #else
     load_tile(0, 0, ring[0]);
 #endif
-    for (int base = 0; base < n_steps; base += 2) {
-#pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        const int step = base + r;
-        if (step >= n_steps) break;
-        load_tile(step + 1, ids_next, ring[r ^ 1]);
+    auto one_step = [&](auto r_c, const int step, const bool ask) __attribute__((always_inline)) {
+      constexpr int r = decltype(r_c)::value;
+      {
+        if (ask) {
+          // (the table entries of the step after next are asked for ahead of the next step's rows:
+          // loads land in the order they were asked for, so waiting for entries asked for behind
+          // the rows would wait for the rows)
 #if !CL_RAGGED
-        ids_next = load_ids(step + 2);
+          const int ids_after = load_ids(step + 2);
+          load_tile(step + 1, ids_next, ring[r ^ 1]);
+          ids_next = ids_after;
+#else
+          load_tile(step + 1, ids_next, ring[r ^ 1]);
 #endif
+        }
         const PfTile& cur = ring[r];
         const int t0 = step * PF_STEP;
 
@@ -219,38 +233,38 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           for (int j = 0; j < 8; ++j) acc[vc][j] = mfma16(as_elem8(vt[j]), pf, acc[vc][j]);
         }
       }
+    };
+    int base = 0;
+    for (; base + 2 < n_steps; base += 2) {
+      one_step(PfC<0>{}, base, true);
+      one_step(PfC<1>{}, base + 1, true);
     }
+    if (base < n_steps) one_step(PfC<0>{}, base, base + 1 < n_steps);
+    if (base + 1 < n_steps) one_step(PfC<1>{}, base + 1, false);
   }
 
-  // ---- each wave writes its head group's rows through its own LDS slab (full-row stores) -------
+  // ---- each lane writes its row's features straight from the accumulators, 16 bytes at a time ----
+  // (acc[vc][0..7][r] are the eight consecutive features 128 vc + 32 g + 8 r .. of row c)
   l_run += lane_xor(l_run, lane, 16);
   l_run += lane_xor(l_run, lane, 32);
   l_exact += lane_xor(l_exact, lane, 16);
   l_exact += lane_xor(l_exact, lane, 32);
-  extern __shared__ float pf_lds[];
-  float* sh_o = pf_lds + (size_t)head * 16 * CL_HEAD_DIM;      // [16][D]
+  if (!live) return;
   const float inv = 1.0f / fmaxf(l_run, 1.0e-30f);            // a row with no key: 0 and lse -inf
+  elem_t* dst = CL_ARG_OUT + ((i64)tok * CL_Q_HEADS + qhead) * CL_HEAD_DIM;
 #pragma unroll
   for (int vc = 0; vc < PF_VC; ++vc)
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int r = 0; r < 4; ++r) {
+      const int d = 128 * vc + 32 * g + 8 * r;
+      if (CL_HEAD_DIM % 128 != 0 && d >= CL_HEAD_DIM) continue;
+      elem8 y;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int d = 128 * vc + 32 * g + 8 * r + j;
-        if (CL_HEAD_DIM % 128 == 0 || d < CL_HEAD_DIM) sh_o[c * CL_HEAD_DIM + d] = acc[vc][j][r] * inv;
-      }
+      for (int j = 0; j < 8; ++j) y[j] = to_elem(acc[vc][j][r] * inv);
+      st16(dst + d, as_u32x4(y));
+    }
 #if CL_EMIT_LSE
-  if (g == 0 && live) CL_ARG_LSE[(i64)tok * CL_Q_HEADS + qhead] = l_exact > 0.f ? m_run + fast_log2(l_exact) : CL_NEG_INF;
+  if (g == 0) CL_ARG_LSE[(i64)tok * CL_Q_HEADS + qhead] = l_exact > 0.f ? m_run + fast_log2(l_exact) : CL_NEG_INF;
 #endif
-  __syncthreads();
-  for (int idx = lane; idx < n_rows * (CL_HEAD_DIM / 4); idx += 64) {
-    const int row = idx / (CL_HEAD_DIM / 4), d = (idx % (CL_HEAD_DIM / 4)) * 4;
-    const i64 orow = (i64)(lo + row / PF_GROUP) * CL_Q_HEADS + head * PF_GROUP + row % PF_GROUP;
-    const f32x4 o = *reinterpret_cast<const f32x4*>(sh_o + row * CL_HEAD_DIM + d);
-    elem4 y;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) y[i] = to_elem(o[i]);
-    *reinterpret_cast<elem4*>(CL_ARG_OUT + orow * CL_HEAD_DIM + d) = y;
-  }
 }
 #endif  // CL_EMIT_PARTIAL

@@ -107,6 +107,10 @@ typedef __attribute__((address_space(3))) md_s16x4 md_lds_s16x4;
 
 CL_DEVICE int md_swz(int token) { return token & 6; }
 
+// x with bits 0 and 3 trading places
+CL_DEVICE int md_trade03(int x) { return (x & ~9) | ((x & 1) << 3) | ((x >> 3) & 1); }
+static_assert(MD_QCHUNKS % 16 == 8, "the Q rows in LDS: a row's parity moves it by eight 16-byte bank groups");
+
 // 16 bytes per lane, global -> LDS; not counted by the compiler, the issuing wave waits itself
 template <int OFF>
 CL_DEVICE void md_dma16(const void* gptr, unsigned lds_byte) {
@@ -217,15 +221,20 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 
   // The Q rows of the 64 heads go through LDS: every wave asks for its share as whole 1 KiB runs
   // (64 consecutive 16-byte slots each), into the two images' worth of LDS the loop fills last;
-  // slot n holds, for head n / MD_QCHUNKS, the 16-byte chunk (n % MD_QCHUNKS) with its low three
-  // bits XOR head % 8 (the score waves' fragment reads then spread over the banks).  Read straight
-  // from global memory, a fragment is sixteen 64-byte pieces per instruction, and both token
-  // halves would fetch the same rows.
+  // row n / MD_QCHUNKS holds the head whose number is the row's with bits 0 and 3 traded, and slot
+  // n % MD_QCHUNKS of it the 16-byte chunk whose low three bits are the slot's XOR head % 8.  A
+  // fragment read has the sixteen heads of a tile side by side: the XOR spreads heads that differ
+  // in their low three bits over eight 16-byte bank groups, and since a row is an odd multiple of
+  // eight such groups long, the row's parity -- bit 3 of the head -- picks the other eight for
+  // heads c and c + 8 (with rows in head order they met in the same banks).  Read straight from
+  // global memory, a fragment is sixteen 64-byte pieces per instruction, and both token halves
+  // would fetch the same rows.
   if (n_own > 0) {
     const i64 wg_row0 = (i64)b * CL_HEADS + hg_block * MD_HEADS_PER_BLOCK;
     for (int k = wave; k < MD_QCHUNKS; k += MD_THREADS / 64) {       // 64 heads x MD_QCHUNKS slots = MD_QCHUNKS runs
       const int n = 64 * k + lane;
-      const int h = n / MD_QCHUNKS, pos = n % MD_QCHUNKS;
+      const int row = n / MD_QCHUNKS, pos = n % MD_QCHUNKS;
+      const int h = md_trade03(row);
       const int q = (pos & ~7) | ((pos ^ h) & 7);
       const elem_t* src = q < CL_CKV / 8 ? CL_ARG_Q + (wg_row0 + h) * CL_CKV + 8 * q
                                          : CL_ARG_QPE + (wg_row0 + h) * CL_KPE + 8 * (q - CL_CKV / 8);
@@ -251,8 +260,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int j = 0; j < MD_KJ; ++j) {
-          const int h = 32 * set + 16 * t + c, q = 4 * j + g;
-          qf[t][j] = *reinterpret_cast<const elem8*>(md_tiles + 2 * MD_TILE + (h * MD_QCHUNKS + ((q & ~7) | ((q ^ c) & 7))) * 8);
+          const int row = 32 * set + 16 * t + md_trade03(c), q = 4 * j + g;
+          qf[t][j] = *reinterpret_cast<const elem8*>(md_tiles + 2 * MD_TILE + (row * MD_QCHUNKS + ((q & ~7) | ((q ^ c) & 7))) * 8);
         }
     } else {
 #pragma unroll
