@@ -701,6 +701,12 @@ class HipCodeGen:
             unit.define("CL_MP_TOK", tok)
         if "LDS_AHEAD" in t:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
+        stages = int(t.get("STAGES", 2))
+        panels = (p["ckv"] + p["kpe"]) // 64
+        if stages not in (2, 3, 4) or stages * panels * 4096 > 160 * 1024 or (stages - 2) * (4 // tok) * panels > 63:
+            raise CodegenError(f"STAGES={stages}: two to four images of {panels * 4096} bytes within 160 KiB of LDS, and at most "
+                               "63 loads in flight behind the awaited step")
+        unit.define("CL_MP_STAGES", stages)
         for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE"),
                             ("INDPTR", "CL_ARG_INDPTR"), ("INDICES", "CL_ARG_INDICES")):
             unit.define(macro, op[role])

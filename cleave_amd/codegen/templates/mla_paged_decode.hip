@@ -8,7 +8,12 @@
 // latent and rope rows of a step go from global memory straight into LDS (16 bytes per lane, the
 // row of every lane looked up in the table) as the token-major image of the dense MLA kernel:
 //   tile  [D/64][32][64]   64-feature panels, 128-byte token rows, 16-byte chunk ^ (token & 6)
-// two images, the next step's rows in flight while the matrix cores work on the current one.
+// CL_MP_STAGES images (2, 3 or 4), the rows of the next CL_MP_STAGES - 1 steps in flight while the
+// matrix cores work on the current one: a step's rows take about a microsecond to arrive from the
+// cache, twice a step's matrix work, so with two images a lone item advances one round trip per
+// step (nothing else runs on its compute unit to fill the wait), with three or four its steps
+// cost what their matrix work costs; many resident items hide the same wait by their number, and
+// two images let a compute unit hold two of them.
 // Table entries are read 256 at a time into four registers per lane (entry 64 k + lane in
 // register k) one window ahead; a lane fetches the entry of the row it loads with a cross-lane
 // read.  Scores, softmax and value product are the dense kernel's (16 heads per wave, Q fragments
@@ -43,6 +48,13 @@ static_assert(MP_WAVES == 1 || MP_WAVES == 2 || MP_WAVES == 4, "1, 2 or 4 tokens
 #define MP_KJ (MP_D / 32)
 #define MP_FB (CL_CKV / 16)
 #define MP_WINDOW 256                          // table entries held in registers at a time
+#ifndef CL_MP_STAGES
+#define CL_MP_STAGES 2
+#endif
+#define MP_AHEAD (CL_MP_STAGES - 1)            // steps whose rows are asked for ahead of the one in the matrix cores
+#define MP_UNITS ((4 / MP_WAVES) * MP_PANELS)  // loads one wave issues for a step
+static_assert(CL_MP_STAGES >= 2 && CL_MP_STAGES <= 4, "two to four images");
+static_assert((MP_AHEAD - 1) * MP_UNITS <= 63, "the load counter holds the loads of the steps in flight behind the awaited one");
 #define MP_RESCALE_STEP 8.0f
 #ifndef CL_LDS_AHEAD
 #define CL_LDS_AHEAD 8
@@ -50,7 +62,7 @@ static_assert(MP_WAVES == 1 || MP_WAVES == 2 || MP_WAVES == 4, "1, 2 or 4 tokens
 static_assert(CL_CKV % 64 == 0 && CL_KPE % 64 == 0, "latent and rope widths are whole 64-feature panels");
 static_assert(CL_HEADS % 16 == 0, "16 heads per wave");
 
-__shared__ __attribute__((aligned(1024))) elem_t mp_tiles[2 * MP_TILE];
+__shared__ __attribute__((aligned(1024))) elem_t mp_tiles[CL_MP_STAGES * MP_TILE];
 
 typedef short mp_s16x4 __attribute__((ext_vector_type(4)));
 typedef short mp_s16x8 __attribute__((ext_vector_type(8)));
@@ -58,6 +70,12 @@ typedef __attribute__((address_space(3))) mp_s16x4 mp_lds_s16x4;
 
 CL_DEVICE int mp_swz(int token) { return token & 6; }
 CL_DEVICE int mp_clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+#define MP_WAITCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+// rows (16 lanes) 1 and 3 of `a` trade places with rows 0 and 2 of `b`
+CL_DEVICE void mp_swap_rows16(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+}
 
 // 16 bytes per lane, global -> LDS: the wave's 64 lanes fill 1 KiB starting at LDS byte address
 // `lds_byte` + OFF (wave-uniform), lane l from `gptr` + OFF.  Not counted by the compiler: the
@@ -122,10 +140,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #endif
 #if CL_PREFILL
   const int n_tok = n_tok_own;                        // keys this wave's token weighs
-  const int n_steps = (hi - lo + MP_STEP - 1) / MP_STEP;   // steps of the item (the same for all its waves)
+  const int n_steps = __builtin_amdgcn_readfirstlane((hi - lo + MP_STEP - 1) / MP_STEP);   // steps of the item (the same for all its waves)
 #else
   const int n_tok = hi - lo;
-  const int n_steps = (n_tok + MP_STEP - 1) / MP_STEP;
+  const int n_steps = __builtin_amdgcn_readfirstlane((n_tok + MP_STEP - 1) / MP_STEP);
 #endif
   const float scale_log2e = sm_scale * 1.4426950408889634f;
 #if CL_PREFILL
@@ -149,13 +167,15 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     for (int i = 0; i < 8; ++i) ones[i] = to_elem(1.0f);
 
     // table entries of a 256-entry window: register k holds entry 64 k + lane (positions past the
-    // item's end repeat its last entry; ids outside the pool are clamped into it)
+    // item's end repeat its last entry; ids outside the pool are clamped into it where they are
+    // used, not here: touching a loaded value waits for it, and with it for every row asked for
+    // before it)
     auto load_window = [&](int w, int (&ids)[4]) __attribute__((always_inline)) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         int pos = lo + w * MP_WINDOW + 64 * k + lane;
         pos = pos < hi - 1 ? pos : hi - 1;
-        ids[k] = mp_clamp(CL_ARG_INDICES[pos], 0, num_pages - 1);
+        ids[k] = CL_ARG_INDICES[pos];
       }
     };
     int ids_cur[4], ids_next[4];
@@ -163,26 +183,28 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) ids_next[k] = ids_cur[k];
 
-    // the rows of step s (its window's entries in `ids`) into image s % 2: lane l loads token row
+    // the rows of step s (its window's entries in `ids`) into image s % CL_MP_STAGES: lane l loads token row
     // 8 rg + l / 8 of the step, the chunk that belongs in slot l % 8 of that row
     auto issue_step = [&](int s, const int (&ids)[4]) __attribute__((always_inline)) {
       const int in_window = s % (MP_WINDOW / MP_STEP);
       const int k = in_window >> 1;
       const int held = k == 0 ? ids[0] : k == 1 ? ids[1] : k == 2 ? ids[2] : ids[3];
-      const unsigned stage_byte = tiles_byte + (unsigned)((s & 1) * MP_TILE * 2);
+      const unsigned stage_byte = tiles_byte + (unsigned)((s % CL_MP_STAGES) * MP_TILE * 2);
 #pragma unroll
       for (int i = 0; i < 4 / MP_WAVES; ++i) {
         const int rg = wave + i * MP_WAVES;             // (the waves of an item share a step's four row groups)
         const int r = 8 * rg + (lane >> 3);
         const int src_lane = 32 * (in_window & 1) + r;
-        const int id = __builtin_amdgcn_ds_bpermute(src_lane << 2, held);
+        const int id = mp_clamp(__builtin_amdgcn_ds_bpermute(src_lane << 2, held), 0, num_pages - 1);
         const int chunk = (lane & 7) ^ mp_swz(r);
         const char* lat_src = reinterpret_cast<const char*>(CL_ARG_KV) + ((i64)id * CL_CKV + 8 * chunk) * 2;
         const char* pe_src = reinterpret_cast<const char*>(CL_ARG_KPE) + ((i64)id * CL_KPE + 8 * chunk) * 2;
         mp_issue_row_group<0>(lat_src, pe_src, stage_byte + (unsigned)(rg * 1024));
       }
     };
-    issue_step(0, ids_cur);
+#pragma unroll
+    for (int i = 0; i < MP_AHEAD; ++i)
+      if (i < n_steps) issue_step(i, ids_cur);          // (all in the first window: MP_AHEAD < 8)
 
     // Q fragments (B operand of the score product): lane (c, g) holds q[head c][32 j + 8 g .. +8]
     elem8 qf[MP_KJ];
@@ -192,6 +214,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       const elem_t* src = col < CL_CKV ? CL_ARG_Q + qrow * CL_CKV + col : CL_ARG_QPE + qrow * CL_KPE + (col - CL_CKV);
       qf[j] = as_elem8(ld16(src));
     }
+    // (the wait for the Q fragments belongs here, once: left to their first use it would sit in the
+    // loop, where it waits for every row in flight at every step)
+#pragma unroll
+    for (int j = 0; j < MP_KJ; ++j) asm volatile("" :: "v"(qf[j]));
 
     // this lane's operand offsets inside an image (elements):
     //   score operand: token row c of a 16-token half, chunk g of a 32-feature block
@@ -211,23 +237,35 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       float mxl = CL_NEG_BIG;
       while (step < n_steps) {
         if (!front_done) {
-          // everything in flight is step `step` (and table entries read a window ahead): wait, then
-          // send the next step's rows into the other image (its last readers were the matrix
-          // ops of step - 1, all issued)
-          __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+          // The rows of `step` have landed when only what was asked for after them is on its way:
+          // the rows of the steps behind it that the item has, at most MP_AHEAD - 1 of them (loads
+          // land in the order they were asked for; table entries read a window ahead lie between
+          // and only make the wait stricter).  The barrier makes that everybody's share, and says
+          // that everybody is done with the image of step - 1, which the rows of step + MP_AHEAD
+          // go into (`ids_cur` are the entries of the window those rows are in).
+          {
+            const int behind = n_steps - 1 - step;
+            if (MP_AHEAD >= 3 && behind >= 2) {
+              MP_WAITCNT(2 * MP_UNITS);
+            } else if (MP_AHEAD >= 2 && behind >= 1) {
+              MP_WAITCNT(MP_UNITS);
+            } else {
+              MP_WAITCNT(0);
+            }
+          }
           __syncthreads();
           if (step % (MP_WINDOW / MP_STEP) == 0 && (step / (MP_WINDOW / MP_STEP) + 1) * MP_WINDOW < hi - lo)
             load_window(step / (MP_WINDOW / MP_STEP) + 1, ids_next);
-          if (step + 1 < n_steps) {
-            if ((step + 1) % (MP_WINDOW / MP_STEP) == 0) {
+          if (step + MP_AHEAD < n_steps) {
+            if ((step + MP_AHEAD) % (MP_WINDOW / MP_STEP) == 0) {
 #pragma unroll
               for (int k = 0; k < 4; ++k) ids_cur[k] = ids_next[k];
             }
-            issue_step(step + 1, ids_cur);
+            issue_step(step + MP_AHEAD, ids_cur);
           }
           front_done = true;
         }
-        const elem_t* tile = mp_tiles + (step & 1) * MP_TILE;
+        const elem_t* tile = mp_tiles + (step % CL_MP_STAGES) * MP_TILE;
 #if CL_PREFILL
         // a wave whose token sees none of this step's keys (or that has no token: it only helps
         // load) leaves the images to the waves that need them
@@ -331,7 +369,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
       for (int fb = 0; fb < MP_FB; ++fb) acc[fb] *= alpha;
     }
-    // no load may still be on its way into LDS when the workgroup ends
+    // (no load is on its way into LDS any more: the last step's wait left none)
     __builtin_amdgcn_s_waitcnt(0x0F70);
   }
 
@@ -359,12 +397,25 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   l_exact += lane_xor(l_exact, lane, 32);
   if (g == 0) CL_ARG_LSE[qrow] = l_exact > 0.f ? m_run + fast_log2(l_exact) : CL_NEG_INF;
 #endif
+  // A lane holds features 16 fb + 4 g .. + 3 of its head for every block fb.  Lanes g and g ^ 1
+  // trade halves of a pair of blocks (one row swap per register), so that each stores 16
+  // contiguous bytes: even g the 8 features from 4 g of the even block, odd g those from
+  // 4 (g - 1) of the odd one (as 8-byte pieces the 32 stores of a wave took over a microsecond).
+  (void)f0;
+  elem_t* dst = dst_row + 16 * (g & 1) + 4 * (g & 2);
 #pragma unroll
-  for (int fb = 0; fb < MP_FB; ++fb) {
-    elem4 y;
+  for (int fp = 0; fp < MP_FB / 2; ++fp) {
+    elem4 y0, y1;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[fb][r] * inv);
-    *reinterpret_cast<elem4*>(dst_row + f0 + 16 * fb) = y;
+    for (int r = 0; r < 4; ++r) {
+      y0[r] = to_elem(acc[2 * fp][r] * inv);
+      y1[r] = to_elem(acc[2 * fp + 1][r] * inv);
+    }
+    const u32x2 a = __builtin_bit_cast(u32x2, y0), b = __builtin_bit_cast(u32x2, y1);
+    unsigned a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1];
+    mp_swap_rows16(a0, b0);
+    mp_swap_rows16(a1, b1);
+    *reinterpret_cast<u32x4*>(dst + 32 * fp) = (u32x4){a0, a1, b0, b1};
   }
 #endif
 }

@@ -14,6 +14,8 @@ query, caches, indptr, indices, [last page len], scale, [partials], out, lse.
 
 from __future__ import annotations
 
+import dataclasses
+
 from dataclasses import dataclass
 
 from ...schedule.plan import KernelPlan, ParamSpec
@@ -68,6 +70,10 @@ class DenseMLA:
     # split form: table entries per work item; -1 lets the launch choose the size from the
     # table length so that two items land on each compute unit
     chunk_pages: int = -1
+    # images of a 32-token step a work item keeps in LDS: the rows of `stages - 1` steps are in
+    # flight while one is in the matrix cores (2: two items fit a compute unit; 3, 4: a lone item
+    # no longer advances one round trip to the cache per step)
+    stages: int = 2
 
     @property
     def query_rows(self) -> int:
@@ -343,10 +349,15 @@ def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None
     if split:
         tiling["CHUNK_PAGES"] = dense.chunk_pages
         extra["derived_dims"] = [("chunk_pages", mla_chunk_pages_expr(spec, dense.chunk_pages))]
+    if dense.stages != 2:
+        tiling["STAGES"] = int(dense.stages)
     threads = dense.n_threads * (int(tok) if prefill else 1)
+    label = f"kv={dense.kv_tile} q={dense.heads * (int(tok) if prefill else 1)} thr={threads}"
+    if dense.stages != 2:
+        label += f" stages={dense.stages}"
     return KernelPlan(template="mla_decode", role=role, family="mla", dtype=dense.dtype, extra=extra, problem=problem,
                       tiling=tiling, params=params, operands=operands, split_factor=split, dyn_dims=dyn,
-                      n_threads=threads, label=f"kv={dense.kv_tile} q={dense.heads * (int(tok) if prefill else 1)} thr={threads}")
+                      n_threads=threads, label=label)
 
 
 def _mla_split_decode(spec: MLASpec, dense: DenseMLA, split: int) -> list:
@@ -369,19 +380,25 @@ def _mla_split_decode(spec: MLASpec, dense: DenseMLA, split: int) -> list:
 
 
 def mla_prefill_variants(plan: KernelPlan, spec) -> list:
-    """The paged MLA causal prefill kernel with two, four and one query tokens per work item (the
-    search times each: an item's waves share its key images, which divides the traffic into the
-    CU and raises the number of waves a CU holds, but they also share the LDS bandwidth that
-    bounds this kernel's matrix work; two tokens per item measured best on the captured workloads)."""
-    return [apply_paging(plan, spec, tok=t) for t in (2, 4, 1)]
+    """The paged MLA causal prefill kernel with two, four and one query tokens per work item and
+    two to four images of a step in LDS (the search times each: an item's waves share its key
+    images, which divides the traffic into the CU and raises the number of waves a CU holds, but
+    they also share the LDS bandwidth that bounds this kernel's matrix work; more images keep the
+    rows of more steps in flight, which a lone item needs and many resident items do not)."""
+    return [apply_paging(plan, spec, tok=t, stages=s) for t, s in ((2, 2), (2, 3), (2, 4), (4, 2), (4, 4), (1, 2), (1, 3))]
 
 
-def apply_paging(plan: KernelPlan, spec, tok: int = 2) -> KernelPlan:
+def mla_decode_variants(plan: KernelPlan, spec) -> list:
+    """The paged MLA decode kernel with two and three images of a step in LDS."""
+    return [apply_paging(plan, spec, stages=s) for s in (2, 3)]
+
+
+def apply_paging(plan: KernelPlan, spec, tok: int = 2, stages: int = 2) -> KernelPlan:
     """A single paged kernel at ``plan``'s tiling (``tok``: query tokens per work item of the
-    paged MLA causal prefill layer)."""
+    paged MLA causal prefill layer; ``stages``: images of a step the paged MLA kernels keep in LDS)."""
     spec.validate()
     if isinstance(spec, MLASpec):
-        dense = read_dense_mla(plan)
+        dense = dataclasses.replace(read_dense_mla(plan), stages=int(stages))
         _check_tiling(spec, dense)
         params, operands = _mla_params(spec, dense)
         outs, out_ops = _mla_outputs(spec, dense)

@@ -17,9 +17,9 @@ from oracle import paged_oracle
 pytestmark = pytest.mark.gpu
 
 
-def mla_kernel(heads=16, ckv=512, kpe=64, split=None, chunk_pages=-1, dtype="bfloat16"):
+def mla_kernel(heads=16, ckv=512, kpe=64, split=None, chunk_pages=-1, dtype="bfloat16", stages=2):
     spec = MLASpec(num_qo_heads=heads)
-    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, chunk_pages=chunk_pages)
+    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, chunk_pages=chunk_pages, stages=stages)
     if split:
         src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split)))
     else:
@@ -58,6 +58,15 @@ def test_paged_mla_decode(split, chunk_pages):
     check(mla_kernel(split=split, chunk_pages=chunk_pages), args, LENS, f"split={split} chunk={chunk_pages}")
 
 
+@pytest.mark.parametrize("split,chunk_pages", [(None, -1), (4, 45), (4, 300)])
+def test_paged_mla_decode_three_images(split, chunk_pages):
+    """The rows of two steps in flight behind the one in the matrix cores: requests of one, two and
+    three steps (fewer steps than images), around the 256-entry table window, empty ones."""
+    lens = LENS + [64, 65, 96, 97, 513]
+    args = workload(lens, num_pages=6000, pad=7)
+    check(mla_kernel(split=split, chunk_pages=chunk_pages, stages=3), args, lens, f"stages=3 split={split} chunk={chunk_pages}")
+
+
 def test_paged_mla_decode_rising_maximum():
     """Scores that keep growing along a request's tokens: the reference point is raised several
     times inside an item and the accumulators rescaled."""
@@ -70,8 +79,9 @@ def test_paged_mla_decode_rising_maximum():
     ckv = ckv.clone()
     ckv[rows, 0] = (ckv[rows, 0].float() * 0.2 + ramp * direction).to(ckv.dtype)
     args = [qn, qp, ckv, kpe, indptr, idx, scale]
-    for split in (None, 2):
-        check(mla_kernel(split=split, chunk_pages=128), args, lens, f"rising maximum split={split}")
+    for split, stages in ((None, 2), (2, 2), (None, 3)):
+        check(mla_kernel(split=split, chunk_pages=128, stages=stages), args, lens,
+              f"rising maximum split={split} stages={stages}")
 
 
 def test_paged_mla_decode_two_head_groups_and_other_widths():
@@ -106,10 +116,10 @@ def test_registry_mla_operator_workloads(axes):
         check(mla_kernel(split=split), args, lens, f"registry axes {axes} split={split}")
 
 
-def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4):
+def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4, stages=2):
     spec = MLASpec(num_qo_heads=heads, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True)
     spec.validate()
-    dense = DenseMLA(heads, ckv, kpe, dtype, dtype)
+    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, stages=stages)
     params, ops = _mla_params(spec, dense)
     outs, out_ops = _mla_outputs(spec, dense)
     loaded = _load_main_kernel_from_code(HipCodeGen().gen(_mla_plan(spec, dense, "main", params + outs, {**ops, **out_ops},
@@ -117,18 +127,18 @@ def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4):
     return _compile(loaded, loaded.manifest["out_idx"])
 
 
-@pytest.mark.parametrize("tok", [1, 2, 4], ids=lambda t: f"tok{t}")
+@pytest.mark.parametrize("tok,stages", [(1, 2), (2, 2), (4, 2), (1, 3), (2, 3), (2, 4), (4, 4)], ids=lambda t: f"{t}")
 @pytest.mark.parametrize("q_lens,kv_lens", [([1, 4, 5, 33, 0, 40, 7], [1, 4, 40, 33, 9, 300, 3]), ([6, 0, 3], [0, 5, 3]),
                                             ([90], [700]), ([3, 9], [2, 5])])
-def test_paged_mla_causal_prefill(q_lens, kv_lens, tok):
+def test_paged_mla_causal_prefill(q_lens, kv_lens, tok, stages):
     """Ragged query rows, one, two or four query tokens per item (one wave each, sharing the
-    item's key images): equal lengths, a cached prefix, windows shorter than the query run (fully
+    item's two to four key images): equal lengths, a cached prefix, windows shorter than the query run (fully
     masked rows beside live ones in one item), requests without queries or without keys, a long
     prefix (table windows reloaded), items cut by request boundaries."""
     tq, tk = sum(q_lens), sum(kv_lens)
     args = dref.mla_paged_prefill_inputs((16, 512, 64, 4 * tk + 64, tk + 3, tq), q_lens, kv_lens, device="cpu")
-    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens} tok={tok}", flush=True)
-    out, lse = mla_prefill_kernel(tok=tok)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens} tok={tok} stages={stages}", flush=True)
+    out, lse = mla_prefill_kernel(tok=tok, stages=stages)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
     torch.cuda.synchronize()
     got_o, got_l = out.float().cpu().numpy(), lse.cpu().numpy()
     want_o, want_l = paged_oracle.mla_prefill(*args[:7], q_lens, kv_lens, args[7])
