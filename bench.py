@@ -412,14 +412,17 @@ def run_dynamic(names=None):
                "per_workload_us": {k: round(best.latency_us[k], 2) for k in keys},
                "search_s": round(time.perf_counter() - t0, 1)}
         if rep.dispatch:
-            # what a call of the compiled operator runs: the split pair or the single kernel by the
-            # calibrated rule; the figures above it are the best single candidate's
+            # what a call of the compiled operator runs: the split pair or the single kernel (decode), the
+            # few-token kernel or the winner (prefill), by the calibrated rule; the figures above it are the
+            # best single candidate's
             row["best_candidate_geomean_us"] = row["geomean_us"]
             row["geomean_us"] = round(rep.dispatch["geomean_us"]["hybrid"], 2)
             row["per_workload_us"] = {k: round(rep.dispatch["per_workload_us"][k], 2) for k in keys
                                       if k in rep.dispatch["per_workload_us"]}
-            row["dispatch"] = {"min_tiles": rep.dispatch["min_tiles"],
-                               "geomean_us": {k: round(v, 2) for k, v in rep.dispatch["geomean_us"].items()}}
+            row["dispatch"] = {"geomean_us": {k: round(v, 2) for k, v in rep.dispatch["geomean_us"].items()}}
+            for key in ("min_tiles", "max_tokens", "few_label"):
+                if key in rep.dispatch:
+                    row["dispatch"][key] = rep.dispatch[key]
         if ref:
             row["reference_h100_us"] = {k: ref[k] for k in keys if k in ref}
             row["reference_h100_geomean_us"] = round(geomean([ref[k] for k in keys if k in ref]), 2)

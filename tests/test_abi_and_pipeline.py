@@ -337,3 +337,22 @@ def test_partials_of_a_kernel_that_cuts_the_keys_its_own_way_are_compared_throug
         manifest = {"tiling": {"WAVES": 1, "SKEW": 30}}
 
     assert own_cut(K) and not own_cut(type("P", (), {"manifest": {"tiling": {"WAVES": 1}}}))
+
+
+def test_token_threshold_of_the_prefill_dispatch():
+    """The rule "the other kernel up to T query tokens" is chosen by the geometric mean over the
+    workloads: a threshold only where the other kernel wins on every workload below it by enough
+    to pay for those it loses, and none when the winner is better everywhere."""
+    from cleave_amd.pipeline.dynamic import pick_token_threshold
+
+    tokens = {"a": 1, "b": 34, "c": 969, "d": 16294}
+    winner = {"a": 4.0, "b": 5.5, "c": 10.0, "d": 170.0}
+    small = {"a": 3.4, "b": 5.0, "c": 14.0, "d": 600.0}
+    t, us = pick_token_threshold(winner, small, tokens)
+    assert t == 34 and us < (4.0 * 5.5 * 10.0 * 170.0) ** 0.25
+    mixed = {"a": 6.0, "b": 5.0, "c": 14.0, "d": 600.0}          # loses on the smallest, wins on the next
+    t, us = pick_token_threshold(winner, mixed, tokens)
+    assert t is None and abs(us - (4.0 * 5.5 * 10.0 * 170.0) ** 0.25) < 1e-9
+    t, _ = pick_token_threshold(winner, {"a": 3.0, "b": 9.0, "c": 14.0, "d": 600.0}, tokens)
+    assert t == 1
+    assert pick_token_threshold(winner, {"x": 1.0}, tokens) == (None, float("inf"))

@@ -216,6 +216,21 @@ def test_registry_prefill_operators(cache_root, name):
     live = np.isfinite(want_l)
     np.testing.assert_allclose(lse.cpu().numpy()[live], want_l[live], rtol=1e-3, atol=1e-3)
     assert np.all(np.isneginf(lse.cpu().numpy()[~live]))
+    # a call of one query token: with a calibrated few-token rule this runs the other kernel
+    if kernel.dispatch:
+        assert kernel.dispatch["by"] == "query_tokens" and kernel.token_role(1) == "few"
+        assert kernel.token_role(kernel.dispatch["max_tokens"] + 1) == "many"
+    q_lens, kv_lens = [1], [37]
+    if ragged:
+        args = dref.gqa_ragged_prefill_inputs((hq, hkv, d, 1, 37), q_lens, kv_lens, device="cuda")
+        table = None
+    else:
+        args = dref.gqa_paged_prefill_inputs((hq, hkv, d, 500, 37, 1), q_lens, kv_lens, device="cuda")
+        table = args[5].cpu()
+    out, lse = kernel(*args)
+    want_o, want_l = paged_oracle.prefill(*[a.cpu() for a in args[:5]], table, q_lens, kv_lens, args[-1])
+    _close(out, want_o)
+    np.testing.assert_allclose(lse.cpu().numpy(), want_l, rtol=1e-3, atol=1e-3)
 
 
 def test_registry_mla_prefill_operator(cache_root):
