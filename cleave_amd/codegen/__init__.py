@@ -701,12 +701,17 @@ class HipCodeGen:
             unit.define("CL_MP_TOK", tok)
         if "LDS_AHEAD" in t:
             unit.define("CL_LDS_AHEAD", int(t["LDS_AHEAD"]))
-        stages = int(t.get("STAGES", 2))
+        stages, ksplit = int(t.get("STAGES", 2)), int(t.get("KSPLIT", 1))
         panels = (p["ckv"] + p["kpe"]) // 64
-        if stages not in (2, 3, 4) or stages * panels * 4096 > 160 * 1024 or (stages - 2) * (4 // tok) * panels > 63:
-            raise CodegenError(f"STAGES={stages}: two to four images of {panels * 4096} bytes within 160 KiB of LDS, and at most "
-                               "63 loads in flight behind the awaited step")
+        if ksplit not in (1, 2) or (ksplit > 1 and (chunked or tok != 1)):
+            raise CodegenError("KSPLIT (two waves dealing an item's steps out between them) is 1 or 2, for the single kernel "
+                               "with one query token per item")
+        share = 1 if ksplit > 1 else tok
+        if stages not in (2, 3, 4) or ksplit * stages * panels * 4096 > 160 * 1024 or (stages - 2) * (4 // share) * panels > 63:
+            raise CodegenError(f"STAGES={stages} KSPLIT={ksplit}: two to four images of {panels * 4096} bytes per key-sharing "
+                               "wave within 160 KiB of LDS, and at most 63 loads in flight behind the awaited step")
         unit.define("CL_MP_STAGES", stages)
+        unit.define("CL_MP_KSPLIT", ksplit)
         for role, macro in (("Q", "CL_ARG_Q"), ("QPE", "CL_ARG_QPE"), ("KV", "CL_ARG_KV"), ("KPE", "CL_ARG_KPE"),
                             ("INDPTR", "CL_ARG_INDPTR"), ("INDICES", "CL_ARG_INDICES")):
             unit.define(macro, op[role])
@@ -715,7 +720,7 @@ class HipCodeGen:
             items = f"ceildiv({p['dim_names']['n_idx']}, chunk_pages) + {batch_name}" if chunked else batch_name
             if prefill:
                 items = f"ceildiv({p['dim_names']['total_q']}, {tok}) + batch"
-            unit.launch(ENTRY, (items, p["heads"] // 16, 1), 64 * tok, 0, self._partial_args)
+            unit.launch(ENTRY, (items, p["heads"] // 16, 1), 64 * max(tok, ksplit), 0, self._partial_args)
         if combine:
             entry, args = self._combine_args
             unit.launch(entry, (f"ceildiv(({batch_name} * {p['heads']}) * {p['ckv'] // 4}, 256)", 1, 1), 256, 0, args)

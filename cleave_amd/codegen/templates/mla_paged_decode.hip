@@ -27,6 +27,14 @@
 // query token.  Four tokens per item quarter the traffic into the CU and put eight waves on a CU
 // where single-token items have two (an item's images take 72 KB of LDS whatever its wave count).
 //
+// CL_MP_KSPLIT = 2 (single kernel; prefill: one token per item): two waves share an item's keys
+// instead -- wave w walks steps w, w + 2, .. through images of its own, with no barrier between
+// them, and at the end the second leaves its reference point, sums and accumulators in LDS for
+// the first to fold into its own by the max-rescale rule.  A lone wave issues an instruction
+// every four or five clocks and a step is about 600 of them, so an item alone on its compute unit
+// takes 1.4 us per 32 keys whatever is in flight: two waves halve that where there are too few
+// items to fill the chip.
+//
 //   CL_HEADS (multiple of 16)  CL_CKV  CL_KPE (multiples of 64)  CL_CHUNKED  CL_PREFILL
 //   run-time: batch, num_pages, n_idx [, chunk_pages]; scalar sm_scale (> 0 or not: the
 //   maximum is taken over scaled scores)
@@ -37,8 +45,16 @@
 #ifndef CL_MP_TOK
 #define CL_MP_TOK 1
 #endif
-#define MP_WAVES (CL_PREFILL ? CL_MP_TOK : 1)   // waves per workgroup
-static_assert(MP_WAVES == 1 || MP_WAVES == 2 || MP_WAVES == 4, "1, 2 or 4 tokens per prefill item");
+#ifndef CL_MP_KSPLIT
+#define CL_MP_KSPLIT 1
+#endif
+#define MP_KS CL_MP_KSPLIT                                            // waves that deal an item's steps out between them
+#define MP_TOKENS (CL_PREFILL && MP_KS == 1 ? CL_MP_TOK : 1)          // query tokens per work item
+#define MP_WAVES (MP_KS > 1 ? MP_KS : MP_TOKENS)                      // waves per workgroup
+#define MP_SHARE (MP_KS > 1 ? 1 : MP_WAVES)                           // waves that load and read one image together
+static_assert(MP_TOKENS == 1 || MP_TOKENS == 2 || MP_TOKENS == 4, "1, 2 or 4 tokens per prefill item");
+static_assert(MP_KS == 1 || (MP_KS == 2 && !CL_CHUNKED && (!CL_PREFILL || CL_MP_TOK == 1)),
+              "keys shared between two waves: single kernel, one token per item");
 #define MP_STEP 32
 #define MP_D (CL_CKV + CL_KPE)
 #define MP_PANEL (MP_STEP * 64)
@@ -52,7 +68,7 @@ static_assert(MP_WAVES == 1 || MP_WAVES == 2 || MP_WAVES == 4, "1, 2 or 4 tokens
 #define CL_MP_STAGES 2
 #endif
 #define MP_AHEAD (CL_MP_STAGES - 1)            // steps whose rows are asked for ahead of the one in the matrix cores
-#define MP_UNITS ((4 / MP_WAVES) * MP_PANELS)  // loads one wave issues for a step
+#define MP_UNITS ((4 / MP_SHARE) * MP_PANELS)  // loads one wave issues for a step
 static_assert(CL_MP_STAGES >= 2 && CL_MP_STAGES <= 4, "two to four images");
 static_assert((MP_AHEAD - 1) * MP_UNITS <= 63, "the load counter holds the loads of the steps in flight behind the awaited one");
 #define MP_RESCALE_STEP 8.0f
@@ -62,7 +78,8 @@ static_assert((MP_AHEAD - 1) * MP_UNITS <= 63, "the load counter holds the loads
 static_assert(CL_CKV % 64 == 0 && CL_KPE % 64 == 0, "latent and rope widths are whole 64-feature panels");
 static_assert(CL_HEADS % 16 == 0, "16 heads per wave");
 
-__shared__ __attribute__((aligned(1024))) elem_t mp_tiles[CL_MP_STAGES * MP_TILE];
+__shared__ __attribute__((aligned(1024))) elem_t mp_tiles[MP_KS * CL_MP_STAGES * MP_TILE];   // (a key-sharing wave has images of its own)
+static_assert(MP_KS == 1 || (MP_FB * 64 * 4 + 3 * 64) * 4 <= MP_TILE * 2, "a wave's sums fit one of its images");
 
 typedef short mp_s16x4 __attribute__((ext_vector_type(4)));
 typedef short mp_s16x8 __attribute__((ext_vector_type(8)));
@@ -102,6 +119,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int head0 = 16 * blockIdx.y;
+  const int tw = MP_KS > 1 ? 0 : wave;                // which of the item's tokens (or load shares) is this wave's
+  const int kw = MP_KS > 1 ? wave : 0;                // which of the item's steps: kw, kw + MP_KS, ..
 #if CL_CHUNKED
   const int item = blockIdx.x;
   // the request whose items include `item`: the last b with b + indptr[b] / C <= item
@@ -113,16 +132,16 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   if (hi <= lo) return;                               // an index no (chunk, request) pair maps to
 #elif CL_PREFILL
   // causal prefill: the request whose items include `item` is the last b with
-  // b + qo_indptr[b] / MP_WAVES <= item; token t of it sees the keys kv_pos <= kv_len - q_len + (t - q0)
+  // b + qo_indptr[b] / MP_TOKENS <= item; token t of it sees the keys kv_pos <= kv_len - q_len + (t - q0)
   const int item = blockIdx.x;
-  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, MP_WAVES, 1, item, lane, CL_ARG_INDPTR, n_idx);
+  const ClRequest found = cl_find_request(CL_ARG_QINDPTR, batch, total_q, MP_TOKENS, 1, item, lane, CL_ARG_INDPTR, n_idx);
   const int req = found.req, q0 = found.p0, q1 = found.p1;
   const int chunk = item - req;
-  const int t_lo = q0 > chunk * MP_WAVES ? q0 : chunk * MP_WAVES;
-  const int t_hi = q1 < (chunk + 1) * MP_WAVES ? q1 : (chunk + 1) * MP_WAVES;
+  const int t_lo = q0 > chunk * MP_TOKENS ? q0 : chunk * MP_TOKENS;
+  const int t_hi = q1 < (chunk + 1) * MP_TOKENS ? q1 : (chunk + 1) * MP_TOKENS;
   if (t_hi <= t_lo) return;                           // an index no (chunk, request) pair maps to
-  const bool tok_live = t_lo + wave < t_hi;           // this wave's token (a wave past the item's tokens only helps load)
-  const int qtok = tok_live ? t_lo + wave : t_lo;
+  const bool tok_live = t_lo + tw < t_hi;             // this wave's token (a wave past the item's tokens only helps load)
+  const int qtok = tok_live ? t_lo + tw : t_lo;
   const int lo = found.s0;
   int hi, n_tok_own;
   {
@@ -151,7 +170,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #else
   const i64 qrow = (i64)req * CL_HEADS + head0 + c;
 #endif
-  const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)mp_tiles;
+  elem_t* my_tiles = mp_tiles + kw * (CL_MP_STAGES * MP_TILE);     // (key-sharing waves: images of one's own)
+  const unsigned tiles_byte = (unsigned)(size_t)(__attribute__((address_space(3))) elem_t*)my_tiles;
 
   float m_run = CL_NEG_BIG;            // softmax reference point of head c (log2 domain), uniform over g
   f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};  // every component: sum of the (element-typed) weights of head c: normalises out
@@ -178,21 +198,36 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         ids[k] = CL_ARG_INDICES[pos];
       }
     };
+    // `ids_cur`: the entries of window `cur_window`, the one the rows asked for next are in;
+    // `ids_next`: those of the window after it, asked for when `ids_cur` was taken up
     int ids_cur[4], ids_next[4];
+    int cur_window = 0;
     load_window(0, ids_cur);
+    if (MP_WINDOW < hi - lo) {
+      load_window(1, ids_next);
+    } else {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) ids_next[k] = ids_cur[k];
+      for (int k = 0; k < 4; ++k) ids_next[k] = ids_cur[k];
+    }
 
-    // the rows of step s (its window's entries in `ids`) into image s % CL_MP_STAGES: lane l loads token row
-    // 8 rg + l / 8 of the step, the chunk that belongs in slot l % 8 of that row
-    auto issue_step = [&](int s, const int (&ids)[4]) __attribute__((always_inline)) {
+    // the rows of step s into this wave's image `image`: lane l loads token row 8 rg + l / 8 of the
+    // step (its table entry fetched from the lane of `ids_cur` that holds it), the chunk that belongs
+    // in slot l % 8 of that row.  Steps are asked for in rising order; stepping into the next
+    // window takes its entries up and asks for those of the one after.
+    auto issue_step = [&](int s, int image) __attribute__((always_inline)) {
+      if (s / (MP_WINDOW / MP_STEP) != cur_window) {
+        cur_window = s / (MP_WINDOW / MP_STEP);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) ids_cur[k] = ids_next[k];
+        if ((cur_window + 1) * MP_WINDOW < hi - lo) load_window(cur_window + 1, ids_next);
+      }
       const int in_window = s % (MP_WINDOW / MP_STEP);
       const int k = in_window >> 1;
-      const int held = k == 0 ? ids[0] : k == 1 ? ids[1] : k == 2 ? ids[2] : ids[3];
-      const unsigned stage_byte = tiles_byte + (unsigned)((s % CL_MP_STAGES) * MP_TILE * 2);
+      const int held = k == 0 ? ids_cur[0] : k == 1 ? ids_cur[1] : k == 2 ? ids_cur[2] : ids_cur[3];
+      const unsigned stage_byte = tiles_byte + (unsigned)(image * MP_TILE * 2);
 #pragma unroll
-      for (int i = 0; i < 4 / MP_WAVES; ++i) {
-        const int rg = wave + i * MP_WAVES;             // (the waves of an item share a step's four row groups)
+      for (int i = 0; i < 4 / MP_SHARE; ++i) {
+        const int rg = tw * (MP_SHARE > 1) + i * MP_SHARE;   // (the waves of a shared image divide a step's four row groups)
         const int r = 8 * rg + (lane >> 3);
         const int src_lane = 32 * (in_window & 1) + r;
         const int id = mp_clamp(__builtin_amdgcn_ds_bpermute(src_lane << 2, held), 0, num_pages - 1);
@@ -204,7 +239,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     };
 #pragma unroll
     for (int i = 0; i < MP_AHEAD; ++i)
-      if (i < n_steps) issue_step(i, ids_cur);          // (all in the first window: MP_AHEAD < 8)
+      if (kw + i * MP_KS < n_steps) issue_step(kw + i * MP_KS, i);
 
     // Q fragments (B operand of the score product): lane (c, g) holds q[head c][32 j + 8 g .. +8]
     elem8 qf[MP_KJ];
@@ -230,7 +265,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // row sums by one more matrix op against ones, nothing crosses lanes in the hot loop; a
     // score more than MP_RESCALE_STEP above the reference leaves the loop before the step is
     // consumed, the cold block raises the reference, rescales (l, O) and re-enters at the step.
-    int step = 0;
+    int step = kw;                     // this wave's steps: kw, kw + MP_KS, ..
+    int image = 0;                     // the image `step` is in: its number among this wave's steps, modulo the images
     bool front_done = false;           // the loads of `step` have been waited for and the next ones issued
     for (;;) {
       bool raise_any = false;
@@ -242,9 +278,9 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
           // land in the order they were asked for; table entries read a window ahead lie between
           // and only make the wait stricter).  The barrier makes that everybody's share, and says
           // that everybody is done with the image of step - 1, which the rows of step + MP_AHEAD
-          // go into (`ids_cur` are the entries of the window those rows are in).
+          // go into (key-sharing waves have images of their own and no barrier).
           {
-            const int behind = n_steps - 1 - step;
+            const int behind = (n_steps - 1 - step) / MP_KS;       // steps of this wave's behind `step`
             if (MP_AHEAD >= 3 && behind >= 2) {
               MP_WAITCNT(2 * MP_UNITS);
             } else if (MP_AHEAD >= 2 && behind >= 1) {
@@ -253,24 +289,17 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
               MP_WAITCNT(0);
             }
           }
-          __syncthreads();
-          if (step % (MP_WINDOW / MP_STEP) == 0 && (step / (MP_WINDOW / MP_STEP) + 1) * MP_WINDOW < hi - lo)
-            load_window(step / (MP_WINDOW / MP_STEP) + 1, ids_next);
-          if (step + MP_AHEAD < n_steps) {
-            if ((step + MP_AHEAD) % (MP_WINDOW / MP_STEP) == 0) {
-#pragma unroll
-              for (int k = 0; k < 4; ++k) ids_cur[k] = ids_next[k];
-            }
-            issue_step(step + MP_AHEAD, ids_cur);
-          }
+          if (MP_SHARE > 1) __syncthreads();
+          if (step + MP_AHEAD * MP_KS < n_steps) issue_step(step + MP_AHEAD * MP_KS, (image + MP_AHEAD) % CL_MP_STAGES);
           front_done = true;
         }
-        const elem_t* tile = mp_tiles + (step % CL_MP_STAGES) * MP_TILE;
+        const elem_t* tile = my_tiles + image * MP_TILE;
 #if CL_PREFILL
         // a wave whose token sees none of this step's keys (or that has no token: it only helps
         // load) leaves the images to the waves that need them
         if (step * MP_STEP >= n_tok) {
-          ++step;
+          step += MP_KS;
+          image = (image + 1) % CL_MP_STAGES;
           front_done = false;
           continue;
         }
@@ -307,7 +336,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
             v = fmaxf(v, st[h][r]);
           }
         mxl = v;
-        if (step == 0 && m_run < 0.5f * CL_NEG_BIG) {
+        if (step == kw && m_run < 0.5f * CL_NEG_BIG) {
           // first step (nothing accumulated yet): its own maximum is the reference
           float mx = mxl;
           mx = fmaxf(mx, lane_xor(mx, lane, 16));
@@ -352,7 +381,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         }
         __builtin_amdgcn_sched_group_barrier(0x008, CL_LDS_AHEAD / 2, 0);
 
-        ++step;
+        step += MP_KS;
+        image = (image + 1) % CL_MP_STAGES;
         front_done = false;
       }
       if (!raise_any) break;
@@ -372,6 +402,40 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // (no load is on its way into LDS any more: the last step's wait left none)
     __builtin_amdgcn_s_waitcnt(0x0F70);
   }
+
+#if MP_KS > 1
+  // ---- the key-sharing waves fold into the first --------------------------------------------------
+  // Every other wave leaves (accumulators, reference point, sums) in its first image as they lie in
+  // its registers -- nothing reads that image any more and no load is on its way into it -- and
+  // the first wave folds them into its own by the max-rescale rule (a wave that had no step stands
+  // at the lowest reference point with sums of zero).
+  {
+    constexpr int sums_at = MP_FB * 64 * 4;
+    if (kw > 0) {
+      float* park = reinterpret_cast<float*>(my_tiles);
+#pragma unroll
+      for (int fb = 0; fb < MP_FB; ++fb) *reinterpret_cast<f32x4*>(park + (fb * 64 + lane) * 4) = acc[fb];
+      park[sums_at + lane] = m_run;
+      park[sums_at + 64 + lane] = l_acc[0];
+      park[sums_at + 128 + lane] = l_exact;
+    }
+    __syncthreads();
+    if (kw > 0) return;
+#pragma unroll
+    for (int w = 1; w < MP_KS; ++w) {
+      const float* theirs = reinterpret_cast<const float*>(mp_tiles + w * (CL_MP_STAGES * MP_TILE));
+      const float m_o = theirs[sums_at + lane];
+      const float m_new = fmaxf(m_run, m_o);
+      const float a = fast_exp2(m_run - m_new), b = fast_exp2(m_o - m_new);
+      m_run = m_new;
+      l_acc = l_acc * a + theirs[sums_at + 64 + lane] * b;
+      l_exact = l_exact * a + theirs[sums_at + 128 + lane] * b;
+#pragma unroll
+      for (int fb = 0; fb < MP_FB; ++fb)
+        acc[fb] = acc[fb] * a + *reinterpret_cast<const f32x4*>(theirs + (fb * 64 + lane) * 4) * b;
+    }
+  }
+#endif
 
   // ---- write this wave's heads ------------------------------------------------------------------
 #if CL_PREFILL

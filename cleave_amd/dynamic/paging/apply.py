@@ -74,6 +74,9 @@ class DenseMLA:
     # flight while one is in the matrix cores (2: two items fit a compute unit; 3, 4: a lone item
     # no longer advances one round trip to the cache per step)
     stages: int = 2
+    # waves that deal a work item's steps out between them (single kernel, one token per item):
+    # 2 halves the time of an item that is alone on its compute unit
+    ksplit: int = 1
 
     @property
     def query_rows(self) -> int:
@@ -351,10 +354,14 @@ def _mla_plan(spec: MLASpec, dense: DenseMLA, role, params, operands, split=None
         extra["derived_dims"] = [("chunk_pages", mla_chunk_pages_expr(spec, dense.chunk_pages))]
     if dense.stages != 2:
         tiling["STAGES"] = int(dense.stages)
-    threads = dense.n_threads * (int(tok) if prefill else 1)
+    if dense.ksplit != 1 and not split:
+        tiling["KSPLIT"] = int(dense.ksplit)
+    threads = dense.n_threads * max(int(tok) if prefill else 1, int(tiling.get("KSPLIT", 1)))
     label = f"kv={dense.kv_tile} q={dense.heads * (int(tok) if prefill else 1)} thr={threads}"
     if dense.stages != 2:
         label += f" stages={dense.stages}"
+    if tiling.get("KSPLIT"):
+        label += f" ksplit={dense.ksplit}"
     return KernelPlan(template="mla_decode", role=role, family="mla", dtype=dense.dtype, extra=extra, problem=problem,
                       tiling=tiling, params=params, operands=operands, split_factor=split, dyn_dims=dyn,
                       n_threads=threads, label=label)
@@ -385,20 +392,25 @@ def mla_prefill_variants(plan: KernelPlan, spec) -> list:
     images, which divides the traffic into the CU and raises the number of waves a CU holds, but
     they also share the LDS bandwidth that bounds this kernel's matrix work; more images keep the
     rows of more steps in flight, which a lone item needs and many resident items do not)."""
-    return [apply_paging(plan, spec, tok=t, stages=s) for t, s in ((2, 2), (2, 3), (2, 4), (4, 2), (4, 4), (1, 2), (1, 3))]
+    return [apply_paging(plan, spec, tok=t, stages=s, ksplit=k)
+            for t, s, k in ((2, 2, 1), (2, 3, 1), (2, 4, 1), (4, 2, 1), (4, 4, 1), (1, 2, 1), (1, 3, 1), (1, 2, 2))]
 
 
 def mla_decode_variants(plan: KernelPlan, spec) -> list:
-    """The paged MLA decode kernel with two and three images of a step in LDS."""
-    return [apply_paging(plan, spec, stages=s) for s in (2, 3)]
+    """The paged MLA decode kernel with two and three images of a step in LDS, and with two waves
+    dealing a request's steps out between them."""
+    return [apply_paging(plan, spec, stages=s, ksplit=k) for s, k in ((2, 1), (3, 1), (2, 2))]
 
 
-def apply_paging(plan: KernelPlan, spec, tok: int = 2, stages: int = 2) -> KernelPlan:
+def apply_paging(plan: KernelPlan, spec, tok: int = 2, stages: int = 2, ksplit: int = 1) -> KernelPlan:
     """A single paged kernel at ``plan``'s tiling (``tok``: query tokens per work item of the
-    paged MLA causal prefill layer; ``stages``: images of a step the paged MLA kernels keep in LDS)."""
+    paged MLA causal prefill layer; ``stages``: images of a step the paged MLA kernels keep in LDS;
+    ``ksplit``: waves that deal an item's steps out between them)."""
     spec.validate()
     if isinstance(spec, MLASpec):
-        dense = dataclasses.replace(read_dense_mla(plan), stages=int(stages))
+        dense = dataclasses.replace(read_dense_mla(plan), stages=int(stages), ksplit=int(ksplit))
+        if ksplit > 1:
+            tok = 1
         _check_tiling(spec, dense)
         params, operands = _mla_params(spec, dense)
         outs, out_ops = _mla_outputs(spec, dense)

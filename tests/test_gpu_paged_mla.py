@@ -17,9 +17,9 @@ from oracle import paged_oracle
 pytestmark = pytest.mark.gpu
 
 
-def mla_kernel(heads=16, ckv=512, kpe=64, split=None, chunk_pages=-1, dtype="bfloat16", stages=2):
+def mla_kernel(heads=16, ckv=512, kpe=64, split=None, chunk_pages=-1, dtype="bfloat16", stages=2, ksplit=1):
     spec = MLASpec(num_qo_heads=heads)
-    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, chunk_pages=chunk_pages, stages=stages)
+    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, chunk_pages=chunk_pages, stages=stages, ksplit=ksplit)
     if split:
         src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split)))
     else:
@@ -67,6 +67,18 @@ def test_paged_mla_decode_three_images(split, chunk_pages):
     check(mla_kernel(split=split, chunk_pages=chunk_pages, stages=3), args, lens, f"stages=3 split={split} chunk={chunk_pages}")
 
 
+def test_paged_mla_decode_two_waves_share_a_request():
+    """Two waves deal a request's steps out between them and the second folds into the first:
+    requests of no, one, two and three steps (a wave without a step), odd and even step counts,
+    around the 256-entry table window, and a second head group."""
+    lens = LENS + [64, 65, 96, 97, 513]
+    args = workload(lens, num_pages=6000, pad=7)
+    check(mla_kernel(ksplit=2), args, lens, "ksplit=2")
+    lens = [40, 300, 7]
+    args = workload(lens, num_pages=900, heads=32, ckv=256, kpe=64)
+    check(mla_kernel(heads=32, ckv=256, kpe=64, ksplit=2), args, lens, "h32 ckv256 ksplit=2")
+
+
 def test_paged_mla_decode_rising_maximum():
     """Scores that keep growing along a request's tokens: the reference point is raised several
     times inside an item and the accumulators rescaled."""
@@ -79,9 +91,9 @@ def test_paged_mla_decode_rising_maximum():
     ckv = ckv.clone()
     ckv[rows, 0] = (ckv[rows, 0].float() * 0.2 + ramp * direction).to(ckv.dtype)
     args = [qn, qp, ckv, kpe, indptr, idx, scale]
-    for split, stages in ((None, 2), (2, 2), (None, 3)):
-        check(mla_kernel(split=split, chunk_pages=128, stages=stages), args, lens,
-              f"rising maximum split={split} stages={stages}")
+    for split, stages, ksplit in ((None, 2, 1), (2, 2, 1), (None, 3, 1), (None, 2, 2)):
+        check(mla_kernel(split=split, chunk_pages=128, stages=stages, ksplit=ksplit), args, lens,
+              f"rising maximum split={split} stages={stages} ksplit={ksplit}")
 
 
 def test_paged_mla_decode_two_head_groups_and_other_widths():
@@ -116,10 +128,10 @@ def test_registry_mla_operator_workloads(axes):
         check(mla_kernel(split=split), args, lens, f"registry axes {axes} split={split}")
 
 
-def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4, stages=2):
+def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4, stages=2, ksplit=1):
     spec = MLASpec(num_qo_heads=heads, kind=MLA_PAGED_PREFILL_CAUSAL, causal=True)
     spec.validate()
-    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, stages=stages)
+    dense = DenseMLA(heads, ckv, kpe, dtype, dtype, stages=stages, ksplit=ksplit)
     params, ops = _mla_params(spec, dense)
     outs, out_ops = _mla_outputs(spec, dense)
     loaded = _load_main_kernel_from_code(HipCodeGen().gen(_mla_plan(spec, dense, "main", params + outs, {**ops, **out_ops},
@@ -127,18 +139,19 @@ def mla_prefill_kernel(heads=16, ckv=512, kpe=64, dtype="bfloat16", tok=4, stage
     return _compile(loaded, loaded.manifest["out_idx"])
 
 
-@pytest.mark.parametrize("tok,stages", [(1, 2), (2, 2), (4, 2), (1, 3), (2, 3), (2, 4), (4, 4)], ids=lambda t: f"{t}")
+@pytest.mark.parametrize("tok,stages,ksplit", [(1, 2, 1), (2, 2, 1), (4, 2, 1), (1, 3, 1), (2, 3, 1), (2, 4, 1), (4, 4, 1), (1, 2, 2)],
+                         ids=lambda t: f"{t}")
 @pytest.mark.parametrize("q_lens,kv_lens", [([1, 4, 5, 33, 0, 40, 7], [1, 4, 40, 33, 9, 300, 3]), ([6, 0, 3], [0, 5, 3]),
                                             ([90], [700]), ([3, 9], [2, 5])])
-def test_paged_mla_causal_prefill(q_lens, kv_lens, tok, stages):
+def test_paged_mla_causal_prefill(q_lens, kv_lens, tok, stages, ksplit):
     """Ragged query rows, one, two or four query tokens per item (one wave each, sharing the
-    item's two to four key images): equal lengths, a cached prefix, windows shorter than the query run (fully
+    item's two to four key images), or two waves on one token dealing its steps out between them: equal lengths, a cached prefix, windows shorter than the query run (fully
     masked rows beside live ones in one item), requests without queries or without keys, a long
     prefix (table windows reloaded), items cut by request boundaries."""
     tq, tk = sum(q_lens), sum(kv_lens)
     args = dref.mla_paged_prefill_inputs((16, 512, 64, 4 * tk + 64, tk + 3, tq), q_lens, kv_lens, device="cpu")
-    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens} tok={tok} stages={stages}", flush=True)
-    out, lse = mla_prefill_kernel(tok=tok, stages=stages)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+    print(f"paged mla prefill q_lens={q_lens} kv_lens={kv_lens} tok={tok} stages={stages} ksplit={ksplit}", flush=True)
+    out, lse = mla_prefill_kernel(tok=tok, stages=stages, ksplit=ksplit)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
     torch.cuda.synchronize()
     got_o, got_l = out.float().cpu().numpy(), lse.cpu().numpy()
     want_o, want_l = paged_oracle.mla_prefill(*args[:7], q_lens, kv_lens, args[7])
