@@ -40,8 +40,9 @@
 // Ends of the kernel.  The 64 heads' Q rows reach the score waves through LDS (whole 1 KiB runs
 // into the LDS of the two images loaded last; read straight from global memory a fragment is
 // sixteen 64-byte pieces per instruction and both token halves would fetch the same rows: 3 us
-// more before the first step at 16 x 128 heads), and the value waves' results leave through LDS
-// as whole half rows (2 us less than 8-byte pieces).
+// more before the first step at 16 x 128 heads), and the value waves' results leave as 16-byte
+// pieces after a row swap between lane groups (as the 8-byte pieces the accumulators hold they
+// took 2 us longer).
 //
 // Softmax reference points without a handshake.  A score wave raises a head's reference point
 // only when a score of its own tokens passes it by 2^8, so its weights never exceed 2^8; with
@@ -75,7 +76,6 @@
 #define MD_UNITS_PER MD_PANELS                  // 1 KiB loads per value wave and step: its 8-token group of every panel
 #define MD_RESCALE_STEP 8.0f
 #define MD_QCHUNKS (MD_D / 8)                    // 16-byte chunks of one head's Q row (latent + rope)
-#define MD_OROW (16 * MD_FBW * 2 + 16)           // bytes of a staged half row of results: its 16-bit values and a 16-byte gap
 #define MD_REF_FLOOR (-1.0e20f)                   // lowest reference point: a token half with every token masked stands here
 #ifndef CL_LDS_AHEAD
 #define CL_LDS_AHEAD 8
@@ -92,12 +92,15 @@ static_assert(CL_CKV % 128 == 0 && CL_KPE % 64 == 0, "whole 64-feature panels, t
 static_assert(CL_HEADS % MD_HEADS_PER_BLOCK == 0, "64 heads per workgroup");
 static_assert(CL_SCALE_LOG2E > 0.f, "the largest raw score must be the largest scaled one");
 static_assert(MD_UNITS_PER < 32, "load counter range");
-static_assert(4 * 16 * MD_OROW <= MD_TILE * 2, "the four value waves' staged rows fit one image slot");
+static_assert(MD_FBW % 2 == 0, "a value wave's feature blocks leave in pairs");
 constexpr bool MD_RAGGED = CL_SKV % MD_STEP != 0;
 
 __shared__ __attribute__((aligned(1024))) elem_t md_tiles[MD_STAGES * MD_TILE];
-// [step parity][head set][head tile][lane][token half]: the lane's four weights of each token half
-__shared__ __attribute__((aligned(16))) u32x2 md_weights[2][2][2][64][2];
+// [step parity][head set][head tile][token half][lane]: the lane's four weights of each token half.  A
+// score wave writes 8 bytes per lane side by side (lanes 16 bytes apart, the two halves interleaved,
+// put lanes l and l + 16 into the same banks); a value wave reads its lane's two halves as two
+// 8-byte pieces.
+__shared__ __attribute__((aligned(16))) u32x2 md_weights[2][2][2][2][64];
 // [step parity][head set][head tile][head][token half]: the reference point those weights stand against
 __shared__ __attribute__((aligned(8))) float md_ref[2][2][2][16][2];
 
@@ -106,6 +109,11 @@ typedef short md_s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) md_s16x4 md_lds_s16x4;
 
 CL_DEVICE int md_swz(int token) { return token & 6; }
+
+// rows (16 lanes) 1 and 3 of `a` trade places with rows 0 and 2 of `b`
+CL_DEVICE void md_swap_rows16(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0" : "+v"(a), "+v"(b));
+}
 
 // x with bits 0 and 3 trading places
 CL_DEVICE int md_trade03(int x) { return (x & ~9) | ((x & 1) << 3) | ((x >> 3) & 1); }
@@ -360,7 +368,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
         elem4 pf;
 #pragma unroll
         for (int r = 0; r < 4; ++r) pf[r] = to_elem(fast_exp2(__builtin_fmaf(st[t][r], CL_SCALE_LOG2E, -m_run[t])));
-        md_weights[it & 1][set][t][lane][half] = __builtin_bit_cast(u32x2, pf);
+        md_weights[it & 1][set][t][half][lane] = __builtin_bit_cast(u32x2, pf);
         if (g == 0) md_ref[it & 1][set][t][c][half] = m_run[t];
       }
     }
@@ -432,7 +440,10 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     f32x2 ref[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      pf[t] = as_elem8(*reinterpret_cast<const u32x4*>(&md_weights[(it - 1) & 1][set][t][lane][0]));
+      {
+        const u32x2 lo2 = md_weights[(it - 1) & 1][set][t][0][lane], hi2 = md_weights[(it - 1) & 1][set][t][1][lane];
+        pf[t] = as_elem8((u32x4){lo2[0], lo2[1], hi2[0], hi2[1]});
+      }
       ref[t] = *reinterpret_cast<const f32x2*>(&md_ref[(it - 1) & 1][set][t][c][0]);
     }
     if (__builtin_amdgcn_ballot_w64(ref[0][0] != m_acc[0] || ref[0][1] != m_acc[0] || ref[1][0] != m_acc[1] ||
@@ -488,15 +499,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   __builtin_amdgcn_s_waitcnt(0x0F70);               // no load may still be on its way into LDS when the workgroup ends
 
   // ---- this wave writes its half of the features of its head set --------------------------------
-  // Through LDS, so that a store instruction covers whole half rows (two of 512 bytes at a latent
-  // width of 512) instead of sixteen 32-byte pieces: 16 head rows of MD_OROW bytes in a piece of
-  // LDS only this wave touches -- in the image slot (n_own + 2) % 4, which nothing reads any more
-  // (its image was used up one iteration ago) and no load still in flight writes (those go to the
-  // slots of images n_own and n_own + 1).
-  char* rows = reinterpret_cast<char*>(md_tiles) + ((n_own + 2) % MD_STAGES) * (MD_TILE * 2) + loader * (16 * MD_OROW);
-  constexpr int lanes_per_row = 16 * MD_FBW * 2 / 16;            // 16-byte pieces of a half row
-  constexpr int rows_per_store = 64 / lanes_per_row;
-  static_assert(lanes_per_row <= 64 && 64 % lanes_per_row == 0 && 16 % rows_per_store == 0, "a store covers whole half rows");
+  // A lane holds features 16 fb + 4 g .. + 3 of its head for every block fb of the wave's half.
+  // Lanes g and g ^ 1 trade halves of a pair of blocks (one row swap per register), so that each
+  // stores 16 contiguous bytes and a store instruction covers 64 contiguous bytes of sixteen rows:
+  // even g the 8 features from 4 g of the even block, odd g those from 4 (g - 1) of the odd one.
+  // (Before: the rows went through LDS so that a store covered whole half rows; the paired 8-byte
+  // LDS writes of that staging were the kernel's remaining bank conflicts.)
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const float m = m_acc[t], l = l_acc[t][0];
@@ -504,28 +512,30 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     const float inv = 1.0f / fmaxf(l, 1.0e-30f);
 #if CL_SPLITS > 1
     const i64 prow = (i64)split * CL_TOTAL_ROWS + orow;
-    char* dst = reinterpret_cast<char*>(CL_ARG_PO + prow * CL_CKV + 16 * MD_FBW * fhalf);
+    elem_t* dst = CL_ARG_PO + (prow + c) * CL_CKV + 16 * MD_FBW * fhalf + 16 * (g & 1) + 4 * (g & 2);
     if (g == 0 && fhalf == 0) {
       CL_ARG_PM[prow + c] = l > 0.f ? m + fast_log2(l) : CL_NEG_BIG;
       CL_ARG_PL[prow + c] = l > 0.f ? 1.0f : 0.f;
     }
 #else
-    char* dst = reinterpret_cast<char*>(CL_ARG_OUT + orow * CL_CKV + 16 * MD_FBW * fhalf);
+    elem_t* dst = CL_ARG_OUT + (orow + c) * CL_CKV + 16 * MD_FBW * fhalf + 16 * (g & 1) + 4 * (g & 2);
 #if CL_EMIT_LSE
     if (g == 0 && fhalf == 0) CL_ARG_LSE[orow + c] = l > 0.f ? m + fast_log2(l) : CL_NEG_INF;
 #endif
 #endif
 #pragma unroll
-    for (int fb = 0; fb < MD_FBW; ++fb) {
-      elem4 y;
+    for (int fp = 0; fp < MD_FBW / 2; ++fp) {
+      elem4 y0, y1;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) y[r] = to_elem(acc[t][fb][r] * inv);
-      *reinterpret_cast<elem4*>(rows + c * MD_OROW + (16 * fb + 4 * g) * 2) = y;
-    }
-#pragma unroll
-    for (int i = 0; i < 16 / rows_per_store; ++i) {
-      const int r = rows_per_store * i + lane / lanes_per_row, piece = lane % lanes_per_row;
-      *reinterpret_cast<u32x4*>(dst + (i64)r * (CL_CKV * 2) + 16 * piece) = *reinterpret_cast<const u32x4*>(rows + r * MD_OROW + 16 * piece);
+      for (int r = 0; r < 4; ++r) {
+        y0[r] = to_elem(acc[t][2 * fp][r] * inv);
+        y1[r] = to_elem(acc[t][2 * fp + 1][r] * inv);
+      }
+      const u32x2 a = __builtin_bit_cast(u32x2, y0), b = __builtin_bit_cast(u32x2, y1);
+      unsigned a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1];
+      md_swap_rows16(a0, b0);
+      md_swap_rows16(a1, b1);
+      *reinterpret_cast<u32x4*>(dst + 32 * fp) = (u32x4){a0, a1, b0, b1};
     }
   }
 }
