@@ -130,3 +130,33 @@ def test_page_permutation_leaves_output_bit_identical():
     moved = [q, k_cache[perm], v_cache[perm], indptr, inv[indices.long()].to(torch.int32), last, scale]
     new_o, new_l = run(kernel, moved)
     assert np.array_equal(base_o, new_o) and np.array_equal(base_l, new_l)
+
+
+@pytest.mark.parametrize("page_size", [1, 64])
+def test_paged_decode_rising_maximum(page_size):
+    """Scores that grow along a request's tokens: the softmax reference point of every row is raised
+    several times inside a split or an item (the cold path: a rescale by a factor strictly between
+    0 and 1), in the fixed-split, skewed, chunked and lockstep forms."""
+    lens = [1500, 700, 65]
+    args = C.paged_workload(lens, page_size=page_size, num_pages=4000 if page_size == 1 else 80, seed=3)
+    q, k_cache, v_cache, indptr, indices = args[:5]
+    q[..., 0] = 4.0
+    d = q.shape[-1]
+    for b, n in enumerate(lens):
+        ramp = torch.linspace(0.0, 35.0 * d ** 0.5 / (4 * 1.4427), n).to(k_cache.dtype)
+        pages = indices[int(indptr[b]):int(indptr[b + 1])].long()
+        for i, pg in enumerate(pages.tolist()):
+            chunk = ramp[i * page_size:(i + 1) * page_size]
+            k_cache[pg, :len(chunk), :, 0] = chunk.reshape(-1, 1)
+    if page_size == 1:
+        args = args[:5] + args[6:]
+    plans = [dict(split=None, waves=4), dict(split=4, waves=1), dict(split=8, waves=2, skew=30)]
+    if page_size > 1:
+        plans += [dict(split=8, waves=8, chunk_pages=4), dict(split=8, waves=8, chunk_pages=-1, lockstep=True)]
+    for plan in plans:
+        kernel = paged_kernel(page_size=page_size, **plan)
+        print(f"paged rising maximum page={page_size} {plan}", flush=True)
+        got_o, got_l = run(kernel, args)
+        want_o, want_l = paged_oracle.decode(*args[:5], lens, page_size, args[-1], out_dtype="float16")
+        np.testing.assert_allclose(got_o, want_o, rtol=1e-2, atol=1e-2)
+        np.testing.assert_allclose(got_l, want_l, rtol=1e-3, atol=2e-3)

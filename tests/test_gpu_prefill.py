@@ -100,3 +100,32 @@ def test_causal_prefill_random_shapes(seed):
     check(ragged, q_lens, kv_lens, hkv=hkv, pad=int(rng.integers(0, 9)), what=f"random seed {seed}", shared=True)
     if seed % 2:
         check(ragged, q_lens, kv_lens, hkv=hkv, what=f"random seed {seed}", shared=False)
+
+
+@SHARED
+@pytest.mark.parametrize("ragged", [False, True])
+def test_causal_prefill_rising_maximum(ragged, shared):
+    """Scores that grow along a request's keys: every row's softmax reference point is raised several
+    times on the way (the cold path: sums and accumulators rescaled by a factor strictly between 0
+    and 1), in both prefill kernels and both key layouts, a cached prefix included."""
+    hq, hkv, d = 32, 8, 128
+    q_lens, kv_lens = [40, 3, 150], [600, 500, 150]
+    total_q, total_kv = sum(q_lens), sum(kv_lens)
+    if ragged:
+        args = dref.gqa_ragged_prefill_inputs((hq, hkv, d, total_q, total_kv), q_lens, kv_lens, device="cpu")
+        table, rows = None, torch.arange(total_kv)
+    else:
+        args = dref.gqa_paged_prefill_inputs((hq, hkv, d, 4 * total_kv + 50, total_kv, total_q), q_lens, kv_lens, device="cpu")
+        table = args[5]
+        rows = table[:total_kv].long()
+    q, k = args[0], args[1]
+    q[..., 0] = 4.0
+    ramp = torch.cat([torch.linspace(0.0, 35.0 * d ** 0.5 / (4 * 1.4427), n) for n in kv_lens])
+    kk = k.reshape(-1, hkv, d)
+    kk[rows, :, 0] = ramp.reshape(-1, 1).to(k.dtype)
+    print(f"prefill rising maximum ragged={ragged} shared={shared}", flush=True)
+    out, lse = prefill_kernel(ragged, hq, hkv, d, shared=shared)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+    torch.cuda.synchronize()
+    want_o, want_l = paged_oracle.prefill(args[0], args[1], args[2], args[3], args[4], table, q_lens, kv_lens, args[-1])
+    np.testing.assert_allclose(out.float().cpu().numpy(), want_o, rtol=1e-2, atol=1e-2)
+    np.testing.assert_allclose(lse.cpu().numpy(), want_l, rtol=1e-3, atol=2e-3)
