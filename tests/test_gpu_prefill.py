@@ -129,3 +129,12 @@ def test_causal_prefill_rising_maximum(ragged, shared):
     want_o, want_l = paged_oracle.prefill(args[0], args[1], args[2], args[3], args[4], table, q_lens, kv_lens, args[-1])
     np.testing.assert_allclose(out.float().cpu().numpy(), want_o, rtol=1e-2, atol=1e-2)
     np.testing.assert_allclose(lse.cpu().numpy(), want_l, rtol=1e-3, atol=2e-3)
+
+
+@SHARED
+@pytest.mark.parametrize("d", [64, 256])
+def test_causal_prefill_other_head_widths(d, shared):
+    """64-wide heads (half a 128-feature block of accumulators: the lanes past the width store nothing)
+    and 256-wide ones (two blocks), both key forms, both kernels."""
+    check(True, [5, 70, 1, 33], [5, 70, 50, 40], d=d, what=f"d={d}", shared=shared)
+    check(False, [40, 3], [200, 35], d=d, pad=3, what=f"d={d}", shared=shared)
