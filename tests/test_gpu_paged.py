@@ -23,7 +23,7 @@ def paged_kernel(page_size=64, hq=32, hkv=8, d=128, waves=4, split=None, dtype="
     dense = DenseAttention(16, 32, d, waves * 64, dtype, dtype, waves=waves, chunk_pages=chunk_pages, prefetch=prefetch,
                            skew=skew, lockstep=lockstep)
     if split:
-        src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split)))
+        src = HipCodeGen().gen(build_split_decode(spec, dense, split, CombineTiling(split=split, cols=min(128, d))))
     else:
         params, ops = _paged_params(spec, dense)
         outs, out_ops = _paged_outputs(spec, dense)
@@ -160,3 +160,14 @@ def test_paged_decode_rising_maximum(page_size):
         want_o, want_l = paged_oracle.decode(*args[:5], lens, page_size, args[-1], out_dtype="float16")
         np.testing.assert_allclose(got_o, want_o, rtol=1e-2, atol=1e-2)
         np.testing.assert_allclose(got_l, want_l, rtol=1e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("d", [64, 256])
+def test_paged_decode_other_head_widths(d):
+    """64-wide heads (half a 128-feature block) and 256-wide ones (two blocks) through the single
+    kernel, a fixed split and chunked items."""
+    lens = [130, 9, 700, 0, 64]
+    args = C.paged_workload(lens, page_size=16, num_pages=200, d=d)
+    check(args, lens, 16, d=d, waves=2)
+    check(args, lens, 16, d=d, waves=1, split=4)
+    check(args, lens, 16, d=d, waves=8, split=8, chunk_pages=5, lockstep=True)
