@@ -444,13 +444,19 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const float l = l_acc[0];
   const int f0 = 4 * g;
 #if CL_CHUNKED
+  // The partial sum that leaves is the one of the unrounded weights (the combined lse is read from
+  // it), and the accumulators leave rescaled by exact / rounded sum, so that this chunk's
+  // accumulators over its sum stay what the rounded weights give.
   const i64 prow = (i64)item * CL_HEADS + head0 + c;
+  l_exact += lane_xor(l_exact, lane, 16);
+  l_exact += lane_xor(l_exact, lane, 32);
+  const float to_exact = l > 0.f ? l_exact / l : 1.0f;
 #pragma unroll
   for (int fb = 0; fb < MP_FB; ++fb)
-    *reinterpret_cast<f32x4*>(CL_ARG_PO + prow * CL_CKV + f0 + 16 * fb) = acc[fb];
+    *reinterpret_cast<f32x4*>(CL_ARG_PO + prow * CL_CKV + f0 + 16 * fb) = acc[fb] * to_exact;
   if (g == 0) {
     CL_ARG_PM[prow] = m_run;
-    CL_ARG_PL[prow] = l;
+    CL_ARG_PL[prow] = l_exact;
   }
 #else
   // an empty request has l == 0: the floor turns 0/0 into 0 and its lse is -inf

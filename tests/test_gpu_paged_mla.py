@@ -96,6 +96,19 @@ def test_paged_mla_decode_rising_maximum():
               f"rising maximum split={split} stages={stages} ksplit={ksplit}")
 
 
+def test_paged_mla_decode_lse_of_short_requests_is_not_rounded():
+    """Requests of a handful of tokens show the element-type rounding of the weights in their lse
+    unless the sum behind the lse is the one of the unrounded weights: single-item, chunked and
+    key-sharing kernels alike (tolerance 2e-4 in log2 units; bf16 rounding would show up to 3e-3)."""
+    lens = [2, 3, 1, 5, 2, 7, 3, 2]
+    args = workload(lens, num_pages=200, heads=32, seed=11)
+    want = paged_oracle.mla_decode(*args[:6], lens, args[6], out_dtype="bfloat16")[1]
+    for kw in (dict(), dict(split=2), dict(split=4, chunk_pages=1), dict(ksplit=2), dict(stages=3)):
+        print(f"paged mla short lse {kw}", flush=True)
+        _, lse = mla_kernel(heads=32, **kw)(*[a.cuda() if isinstance(a, torch.Tensor) else a for a in args])
+        np.testing.assert_allclose(lse.cpu().numpy(), want, rtol=0, atol=2e-4, err_msg=str(kw))
+
+
 def test_paged_mla_decode_two_head_groups_and_other_widths():
     lens = [40, 300, 7]
     args = workload(lens, num_pages=900, heads=32, ckv=256, kpe=64)
