@@ -38,6 +38,16 @@ def test_dense_prefill_against_the_oracle(shapes):
     _check(C.gqa_decode_exact, cl.f16, shapes)
 
 
+@pytest.mark.parametrize("keys", [32, 64, 96, 128, 160, 256])
+def test_widest_head_with_whole_steps_of_keys(keys):
+    """256-wide heads over one to eight whole 32-key steps (no masked tail).  Four steps once came
+    back wrong in the first row tile of every wave: the step count is a constant in this mode, the
+    compiler laid the four steps out in a straight line and, short of registers, restored a spilled
+    query fragment with one register missing.  The loop's trip count is kept from the optimiser now."""
+    _check(C.gqa_decode_exact, cl.f16, dict(HQ=1, HKV=1, SQ=152, SKV=keys, D=256), seed=37705)
+    _check(C.gqa_decode_exact, cl.bf16, dict(HQ=4, HKV=2, SQ=40, SKV=keys, D=256), seed=3)
+
+
 def test_dense_prefill_bf16_and_the_shifted_softmax_form():
     _check(C.gqa_decode_exact, cl.bf16, dict(HQ=8, HKV=2, SQ=96, SKV=257, D=128))
     _check(C.gqa_decode_shift, cl.f16, dict(HQ=8, HKV=4, SQ=100, SKV=200, D=64))
