@@ -165,7 +165,11 @@ struct GdOperand {
   // load (the cast back into the LDS address space checks for the null pointer), 128 a step ahead of the
   // matrix work, which a wave that has its SIMD to itself cannot hide.
   CL_METHOD void issue_unit(int i, const elem_t* base, unsigned lds_byte, unsigned wave_byte) const {
-    const int u = (threadIdx.x >> 6) + i * GD_WAVES;
+    // (the wave's index out of the scalar `wave_byte`: taken from threadIdx the test below is a
+    // divergent branch to the compiler, which then keeps `base` in vector registers inside it and
+    // hands the assembly a vector pair where it names a scalar one -- tiles with fewer units than
+    // waves did not compile)
+    const int u = (int)(wave_byte >> 10) + i * GD_WAVES;
     if (UNITS % GD_WAVES == 0 || u < UNITS) {
       const unsigned m0_value = lds_byte + i * GD_WAVES * 1024 + wave_byte;
 #if CL_ASM_LOADS

@@ -58,7 +58,8 @@ def test_matmul_gemm_large_tiles(tiling):
 DMA_TILES = [dict(BM=16, BN=16, BK=64, WM=1, WN=1), dict(BM=32, BN=64, BK=64, WM=1, WN=2),
              dict(BM=64, BN=64, BK=64, WM=2, WN=2), dict(BM=128, BN=128, BK=64, WM=2, WN=2),
              dict(BM=256, BN=128, BK=64, WM=4, WN=2), dict(BM=128, BN=256, BK=64, WM=2, WN=4, GROUP_M=2),
-             dict(BM=256, BN=256, BK=64, WM=2, WN=2)]
+             dict(BM=256, BN=256, BK=64, WM=2, WN=2),
+             dict(BM=16, BN=64, BK=64, WM=1, WN=4)]             # fewer load units for A than waves
 
 
 @pytest.mark.parametrize("tiling", DMA_TILES, ids=lambda t: "x".join(str(v) for v in t.values()))

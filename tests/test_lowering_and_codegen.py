@@ -375,3 +375,21 @@ def test_searches_that_find_nothing_say_why():
     for rows in (512, 1):
         wide = search_tiling(stage_graph(C.gqa_decode_exact.trace(cl.f16, HQ=8, HKV=2, SQ=rows, SKV=1000, D=192)))
         assert wide and {c.template for c in wide} == {"attn_prefill"}
+
+
+def test_matmul_tiles_with_fewer_load_units_than_waves_compile():
+    """A 16-row tile under four waves has two 1 KiB load units for A: only two waves load it.  The
+    test for that must be scalar to the compiler (the wave index out of a scalar register), or the
+    tile's base address reaches the load's assembly in vector registers and the source does not
+    compile: found at these shapes by a sweep of the default plan (needs the compiler, no GPU)."""
+    from cleave_amd.runtime import shim
+    shim.load()
+    for shapes in (dict(M=336, N=1536, K=1024), dict(M=768, N=792, K=1024)):
+        for fn, dtype in ((C.matmul_nt, cl.f16), (C.matmul_nt, cl.bf16)):
+            source = source_for(fn.trace(dtype, **shapes))
+            text = source if isinstance(source, str) else source.code
+            code, _ = shim.compile_source(text, "cleave_kernel.hip", "gfx950")
+            assert len(code) > 1000
+    tiling = dict(BM=16, BN=64, BK=64, WM=1, WN=4)
+    source = source_for(C.matmul.trace(cl.f16, M=600, N=776, K=576), template="gemm_dma", tiling=tiling)
+    shim.compile_source(source if isinstance(source, str) else source.code, "cleave_kernel.hip", "gfx950")
