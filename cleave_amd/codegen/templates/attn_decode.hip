@@ -319,7 +319,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 // rescaled: both happen only when some lane asks (the two ballots are wave-uniform and cold).  Masked
 // slots hold CL_NEG_BIG; while a whole row is still masked its reference equals it too, so the weights
 // test the mask itself rather than trusting exp2 of a zero difference.  The row sum adds up the weights
-// as rounded to the element type, the ones the value product really sees.
+// before they are rounded to the element type (as the reference's kernels do): it normalises the output
+// and is the lse, which at bf16 showed the rounding (1 - 2e-3) for requests of a few tokens otherwise.
 // CL_LOCKSTEP (chunked items): the waves of a workgroup, one per kv head, meet at a barrier before every
 // step.  Left alone they drift apart (the older wave of a SIMD is served first: in a 1024-token item the
 // first wave is done after 88 us, the last after 155) and the item is as slow as its slowest wave; in step,
@@ -365,9 +366,8 @@ _Pragma("unroll")                                                               
 _Pragma("unroll")                                                                                   \
       for (int i = 0; i < 8; ++i) {                                                                 \
         float p = s[i] > 0.5f * CL_NEG_BIG ? fast_exp2(s[i] - m_new) : 0.f;                         \
-        elem_t pe = to_elem(p);                                                                     \
-        psum += to_f32(pe);                                                                         \
-        pf[i] = pe;                                                                                 \
+        psum += p;                                                                                  \
+        pf[i] = to_elem(p);                                                                         \
       }                                                                                             \
       l_run = l_run * alpha + psum;                                                                 \
                                                                                                     \

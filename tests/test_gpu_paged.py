@@ -76,6 +76,23 @@ def test_paged_decode_chunked_other_head_counts():
     check(args, lens, 16, split=4, waves=4, hq=16, hkv=4, chunk_pages=2, lockstep=True)
 
 
+def test_paged_decode_bf16_lse_of_short_requests_is_not_rounded():
+    """At bf16 a request of a few tokens shows the rounding of its weights (2^-9 each) in the lse
+    unless the row sum adds them up unrounded: single kernel, fixed split and chunked items, page
+    sizes 1 and 64 (tolerance 2e-4; the rounded sum was off by up to 2e-3)."""
+    lens = [2, 3, 1, 5, 2, 7, 3, 2, 4, 6]
+    for page_size in (1, 64):
+        args = C.paged_workload(lens, page_size=page_size, num_pages=40, hq=32, hkv=4, dtype=torch.bfloat16, seed=3)
+        call = args if page_size > 1 else args[:5] + args[6:]
+        want = paged_oracle.decode(*args[:5], lens, page_size, args[-1], out_dtype="bfloat16")[1]
+        for kw in (dict(), dict(split=4), dict(split=4, chunk_pages=1, waves=4)):
+            if kw.get("chunk_pages") and page_size == 1:
+                continue
+            print(f"paged bf16 short lse page={page_size} {kw}", flush=True)
+            _, lse = run(paged_kernel(page_size=page_size, hq=32, hkv=4, dtype="bfloat16", **kw), call)
+            np.testing.assert_allclose(lse, want, rtol=0, atol=2e-4, err_msg=f"page={page_size} {kw}")
+
+
 @pytest.mark.parametrize("page_size", [1, 16])
 def test_paged_decode_other_page_sizes(page_size):
     lens = [5, 33, 130, 64]
