@@ -427,7 +427,8 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 
   // scores^T of one step out of the K image in stage SLOT: a 16-byte read per 16-key half and
   // 32-feature block, each feeding the wave's two row tiles
-  auto k_frag = [&](auto slot_c, int j, int h) __attribute__((always_inline)) {
+  // (`lo`: the lane's operand offset a_lo / v_lo, or a body's own copy of it, see do_step)
+  auto k_frag = [&](auto slot_c, int j, int h, int lo) __attribute__((always_inline)) {
     constexpr int SLOT = decltype(slot_c)::value;
 #if CL_KT
     // sixteen lanes address a 4 (feature) x 16 (key) patch, lane c: feature row c / 4, keys 4 (c % 4) .. + 3,
@@ -439,14 +440,14 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     return __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
 #else
     return *reinterpret_cast<const elem8*>(pl_tiles + SLOT * PL_STAGE + (j >> 1) * PL_PANEL + 16 * h * 64 +
-                                           (a_lo ^ ((4 * (j & 1)) << 3)));
+                                           (lo ^ ((4 * (j & 1)) << 3)));
 #endif
   };
   // value operand for feature block fb out of the V image in stage SLOT: rows = features
   // 16 fb + (0..15), slots = keys 4 g + (0..3), 16 + 4 g + (0..3)
-  auto v_frag = [&](auto slot_c, int fb) __attribute__((always_inline)) {
+  auto v_frag = [&](auto slot_c, int fb, int lo) __attribute__((always_inline)) {
     constexpr int SLOT = decltype(slot_c)::value;
-    const elem_t* p = pl_tiles + SLOT * PL_STAGE + PL_KIMG + (fb >> 2) * PL_PANEL + (v_lo ^ (((2 * fb) & 7) << 3));
+    const elem_t* p = pl_tiles + SLOT * PL_STAGE + PL_KIMG + (fb >> 2) * PL_PANEL + (lo ^ (((2 * fb) & 7) << 3));
     const pl_s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p));
     const pl_s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pl_lds_s16x4*)(p + 16 * 64));
     return __builtin_bit_cast(elem8, (pl_s16x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -494,7 +495,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     for (int j = 0; j < PL_KJ; ++j)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const elem8 a = k_frag(PlC<0>{}, j, h);
+        const elem8 a = k_frag(PlC<0>{}, j, h, a_lo);
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) st[rt][h] = mfma16(a, qf[rt][j], st[rt][h]);
 #if CL_KNORM
@@ -525,15 +526,24 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #define PL_ISSUE(place) issue_quarter(row_ahead, (SLOT + 3) % PL_STAGES, PlC<place>{})
     PL_ISSUE(0);
 
-    // operands of this body's matrix work: K of step + 1, V of step (8 + 16 LDS reads)
+    // operands of this body's matrix work: K of step + 1, V of step (8 + 16 LDS reads).
+    // With more than 64 KiB of images (keys wider than 128) the offset field of an LDS instruction no
+    // longer reaches every stage from one register per lane pattern, and the dozen address registers
+    // the optimiser then kept across the loop were spilled, every reload waiting for the tile loads
+    // in flight: each body forms its addresses from a copy of the two lane offsets that the
+    // optimiser cannot see through, so none of them lives longer than the body's reads (192-wide
+    // keys: 14 spilled registers -> none, 8 % faster; at exactly 64 KiB, 128-wide heads, the same
+    // step takes the one spilled register away and costs 4 %: not done there).
+    int a_lo_b = a_lo, v_lo_b = v_lo;
+    if constexpr (PL_STAGES * PL_STAGE * 2 > 65536) asm volatile("" : "+v"(a_lo_b), "+v"(v_lo_b));
     elem8 kf[PL_KJ][2];
 #pragma unroll
     for (int j = 0; j < PL_KJ; ++j)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) kf[j][h] = k_frag(PlC<(SLOT + 1) % PL_STAGES>{}, j, h);
+      for (int h = 0; h < 2; ++h) kf[j][h] = k_frag(PlC<(SLOT + 1) % PL_STAGES>{}, j, h, a_lo_b);
     elem8 vf[PL_FB];
 #pragma unroll
-    for (int fb = 0; fb < PL_FB; ++fb) vf[fb] = v_frag(slot_c, fb);
+    for (int fb = 0; fb < PL_FB; ++fb) vf[fb] = v_frag(slot_c, fb, v_lo_b);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- maxima of the step's scores; raise a row's reference when they pass it by 2^8 -------
@@ -672,12 +682,11 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // (where the trip count is a small constant it is kept from the optimiser: a handful of steps
   // would otherwise be laid out in a straight line, and at a 256-wide head that form, short of
   // registers, came back from the compiler with one register of a spilled query fragment not
-  // restored; with keys wider than 128 the loop the optimiser cannot count also spills less:
-  // 1530 -> 1420 us at 192-wide keys, 4096 x 4096, 128 heads, while 64- and 128-wide heads with
-  // many steps run 1 - 3 % faster on the counted loop)
+  // restored; with many steps the counted loop stays a loop and runs 1 - 4 % faster than the
+  // one the optimiser cannot count, except at 256-wide heads, where it spills four times as much)
   int trips = n_steps;
 #if CL_DENSE
-  if constexpr (steps_per_split <= 16 || CL_HEAD_DIM > 128) asm volatile("" : "+s"(trips));
+  if constexpr (steps_per_split <= 16 || CL_HEAD_DIM > 192) asm volatile("" : "+s"(trips));
 #endif
   for (int step = 0;;) {
     do_step(PlC<0>{}, step);
