@@ -96,6 +96,37 @@ def compile_code_object(source: str, arch: str = "gfx950") -> bytes:
     return code
 
 
+def code_object_stats(code: bytes) -> list[dict]:
+    """Per kernel of a gfx950 code object, what the compiler's metadata note says of it: ``name``,
+    ``vgprs``, ``agprs``, ``sgprs``, ``spilled_vgprs``, ``spilled_sgprs``, ``scratch_bytes`` (per lane)
+    and ``lds_bytes``.  A kernel with scratch traffic in its loop pays for it twice here (the reload
+    waits for every tile load in flight), so searches and tests read this rather than guess."""
+    import struct
+
+    import msgpack
+
+    if code[:4] != b"\x7fELF":
+        raise CompileError("not an ELF code object")
+    shoff, = struct.unpack_from("<Q", code, 0x28)
+    shentsize, shnum = struct.unpack_from("<HH", code, 0x3A)
+    out = []
+    for i in range(shnum):
+        _, kind, _, _, off, size = struct.unpack_from("<IIQQQQ", code, shoff + i * shentsize)
+        pos = off
+        while kind == 7 and pos + 12 <= off + size:                     # SHT_NOTE
+            namesz, descsz, ntype = struct.unpack_from("<III", code, pos)
+            at = pos + 12 + ((namesz + 3) & ~3)
+            if ntype == 32:                                              # NT_AMDGPU_METADATA
+                for k in msgpack.unpackb(code[at:at + descsz], raw=False).get("amdhsa.kernels", ()):
+                    out.append({"name": k.get(".name"), "vgprs": k.get(".vgpr_count", 0), "agprs": k.get(".agpr_count", 0),
+                                "sgprs": k.get(".sgpr_count", 0), "spilled_vgprs": k.get(".vgpr_spill_count", 0),
+                                "spilled_sgprs": k.get(".sgpr_spill_count", 0),
+                                "scratch_bytes": k.get(".private_segment_fixed_size", 0),
+                                "lds_bytes": k.get(".group_segment_fixed_size", 0)})
+            pos = at + ((descsz + 3) & ~3)
+    return out
+
+
 class CompiledKernel:
     def __init__(self, loaded: LoadedKernel, out_idx, code: bytes):
         self.loaded = loaded
@@ -113,6 +144,11 @@ class CompiledKernel:
             norm = sorted(i if i < 0 else i - len(self._caller_params) for i in self.out_idx)
             if norm != want:
                 raise CompileError(f"out_idx {self.out_idx} does not name the kernel's {self._n_out} trailing outputs")
+
+    @property
+    def stats(self) -> list[dict]:
+        """Registers, spills, scratch and LDS of every entry point (``code_object_stats``)."""
+        return code_object_stats(self._code)
 
     # the reference's callers read these two
     def get_kernel_source(self) -> str:

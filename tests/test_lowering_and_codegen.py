@@ -393,3 +393,31 @@ def test_matmul_tiles_with_fewer_load_units_than_waves_compile():
     tiling = dict(BM=16, BN=64, BK=64, WM=1, WN=4)
     source = source_for(C.matmul.trace(cl.f16, M=600, N=776, K=576), template="gemm_dma", tiling=tiling)
     shim.compile_source(source if isinstance(source, str) else source.code, "cleave_kernel.hip", "gfx950")
+
+
+def test_hot_kernels_keep_their_values_in_registers():
+    """The graded operators' kernels as the run-time compiler builds them: no spilled register and
+    no scratch memory (needs the compiler, no GPU).  A spill inside a kernel's loop costs more than
+    its own traffic here, because the reload waits for every tile load in flight: the wide-key
+    attention kernel ran a quarter slower for fourteen spilled address registers, and the listing
+    of the offline compiler, which allocates differently, did not show them."""
+    from cleave_amd.pipeline.direct import kernel_for
+    from cleave_amd.runtime import shim
+    shim.load()
+    plans = [
+        ("rmsnorm -> matmul M=16", C.CASES["c2"], C.FULL["c2"], dict(template="skinny", tiling=dict(WAVES_N=1, WAVES_K=2), split=8)),
+        ("GQA decode", C.CASES["c3"], C.FULL["c3"], dict(template="attn_decode", tiling=dict(WAVES=1, SKEW=30), split=8)),
+        ("MLA decode", C.CASES["c4"], C.FULL["c4"], dict(template="mla_decode", tiling=dict(DUO=1, LDS_AHEAD=4), split=8)),
+        ("matmul 4096x14336x4096", C.CASES["c1"], dict(M=4096, N=14336, K=4096),
+         dict(template="gemm_dma", tiling=dict(BM=256, BN=256, BK=64, WM=4, WN=2, TAIL=128))),
+        ("dense attention d=64", C.CASES["c3"], dict(HQ=32, HKV=8, SQ=4096, SKV=4096, D=64),
+         dict(template="attn_prefill", tiling=dict(SHARED=1))),
+    ]
+    kernels = [(label, kernel_for(case[0].trace(case[1], **sizes), **how)) for label, case, sizes, how in plans]
+    kernels.append(("attention 192/128 wide", kernel_for(C.mla_prefill.trace(cl.f16, H=128, SQ=4096, SKV=4096, DK=192, DV=128))))
+    for label, kernel in kernels:
+        stages = getattr(kernel, "stages", None) or [kernel]
+        for stage in stages:
+            for entry in stage.stats:
+                assert entry["spilled_vgprs"] == 0 and entry["scratch_bytes"] == 0, (label, entry)
+                assert entry["vgprs"] <= 512 and entry["lds_bytes"] <= 160 * 1024, (label, entry)
