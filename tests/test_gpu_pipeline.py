@@ -30,6 +30,10 @@ def test_compile_matmul_end_to_end(cache_root, tmp_path):
     assert len(report.correct) >= 1 and set(report.timings) >= {"superoptimize", "schedule", "build"}
     assert "main_kernel" in kernel.source
     assert "superoptimize" in report.summary() and "benchmark" in report.summary()
+    # the leaders a caller may want to time again under its own conditions: the winner first, all within the margin
+    close = report.contenders(top=3, within=0.5)
+    assert 1 <= len(close) <= 3 and close[0].label == kernel.label and close[0].variant == kernel.variant
+    assert all(c.latency_us <= 1.5 * close[0].latency_us + 1e-9 for c in close)
 
     prog = cleave_amd.trace(C.matmul, SHAPES, cl.f16)
     x, w = prog.random_inputs(seed=1)
