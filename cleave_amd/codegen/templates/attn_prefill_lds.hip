@@ -536,9 +536,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
     // step takes the one spilled register away and costs 4 %: not done there).
     int a_lo_b = a_lo, v_lo_b = v_lo;
     if constexpr (PL_STAGES * PL_STAGE * 2 > 65536) asm volatile("" : "+v"(a_lo_b), "+v"(v_lo_b));
-    elem8 kf[PL_KJ][2];
+    // (256-wide keys: the fragments of the key image are held half at a time -- the second half is
+    // read once the score products of the first have gone out -- or query fragments are spilled)
+    constexpr int KH = (PL_KJ > 6 && !CL_KNORM) ? PL_KJ / 2 : PL_KJ;
+    elem8 kf[KH][2];
 #pragma unroll
-    for (int j = 0; j < PL_KJ; ++j)
+    for (int j = 0; j < KH; ++j)
 #pragma unroll
       for (int h = 0; h < 2; ++h) kf[j][h] = k_frag(PlC<(SLOT + 1) % PL_STAGES>{}, j, h, a_lo_b);
     elem8 vf[PL_FB];
@@ -572,6 +575,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[j][h], qf[rt][j], sn[rt][h]);
+    if constexpr (KH < PL_KJ) {
+#pragma unroll
+      for (int j = KH; j < PL_KJ; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) kf[j - KH][h] = k_frag(PlC<(SLOT + 1) % PL_STAGES>{}, j, h, a_lo_b);
+    }
 #if !CL_LINEAR
     // (the lane's own eight scores of each row; a row's four lane groups are compared only when
     // some lane passes its row's reference: no row does unless one of its lanes does)
@@ -588,6 +597,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
     }
+    if constexpr (KH < PL_KJ) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (PL_KJ - KH), 0);
     if (__builtin_amdgcn_ballot_w64(mx[0] > m_run[0] + 8.0f || mx[1] > m_run[1] + 8.0f)) {
       // cold after the first steps of an item: weights stay below 2^8 against a reference that
       // lags the running maximum by less than 8 (log2 domain)
@@ -632,7 +642,7 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[j][h], qf[rt][j], sn[rt][h]);
+        for (int rt = 0; rt < 2; ++rt) sn[rt][h] = mfma16(kf[KH < PL_KJ ? j - KH : j][h], qf[rt][j], sn[rt][h]);
     weigh(0);
 #pragma unroll
     for (int i = 0; i < 2 * PL_KJ; ++i) {
