@@ -140,7 +140,16 @@ CL_DEVICE int att_clamp_ptr(int p, int n_idx) { return p < 0 ? 0 : (p > n_idx ? 
 #endif
 
 #if CL_EMIT_PARTIAL
-extern "C" __global__ void __launch_bounds__(CL_WAVES * 64)
+// (one tile in flight and heads of up to 128: the kernel fits the 256 registers that let two waves
+// share a SIMD, but the compiler only aims for that when told -- left alone it used 260 and halved the
+// occupancy of the four-wave form; deeper rings and wider heads need more and are left alone)
+// (the second figure of the launch bounds is waves per SIMD)
+#if CL_PREFETCH == 1 && CL_HEAD_DIM <= 128 && CL_VDIM <= 128
+#define ATT_WAVES_PER_SIMD 2
+#else
+#define ATT_WAVES_PER_SIMD 1
+#endif
+extern "C" __global__ void __launch_bounds__(CL_WAVES * 64, ATT_WAVES_PER_SIMD)
 CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
