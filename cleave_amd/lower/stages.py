@@ -63,7 +63,10 @@ def partial_buffers(low: Lowered, factor: int) -> list:
 
 
 def _split_extent(low: Lowered) -> int:
-    return low.problem["skv"] if low.family in ("attention", "mla") else low.problem["K"]
+    key = "skv" if low.family in ("attention", "mla") else "K"
+    if key not in low.problem:
+        raise LoweringRejected(f"family {low.family!r} has no split form")
+    return low.problem[key]
 
 
 def split_stages(graph: StageGraph, factor: int) -> list:

@@ -421,3 +421,13 @@ def test_hot_kernels_keep_their_values_in_registers():
             for entry in stage.stats:
                 assert entry["spilled_vgprs"] == 0 and entry["scratch_bytes"] == 0, (label, entry)
                 assert entry["vgprs"] <= 512 and entry["lds_bytes"] <= 160 * 1024, (label, entry)
+
+
+def test_a_split_of_a_family_without_a_contraction_is_refused_with_its_reason():
+    """Row reductions have nothing to split: asking for a split is a refusal that says so (it
+    was a KeyError from inside the lowering)."""
+    graph = stage_graph(C.rowsum_div.trace(cl.f16, M=64, N=256))
+    with pytest.raises(LoweringRejected, match="no split form"):
+        split_stages(graph, 4)
+    with pytest.raises(LoweringRejected, match="no split form"):
+        source_for(C.rowsum_div.trace(cl.f16, M=64, N=256), split=4)
