@@ -693,10 +693,12 @@ CL_PARTIAL_NAME(CL_PARTIAL_PARAMS) {
   // would otherwise be laid out in a straight line, and at a 256-wide head that form, short of
   // registers, came back from the compiler with one register of a spilled query fragment not
   // restored; with many steps the counted loop stays a loop and runs 1 - 4 % faster than the
-  // one the optimiser cannot count, except at 256-wide heads, where it spills four times as much)
+  // one the optimiser cannot count, except at 256-wide heads, where it spills four times as much,
+  // and at counts that are not whole turns of the four bodies, where the optimiser peels the rest
+  // off and spills sixty registers doing so)
   int trips = n_steps;
 #if CL_DENSE
-  if constexpr (steps_per_split <= 16 || CL_HEAD_DIM > 192) asm volatile("" : "+s"(trips));
+  if constexpr (steps_per_split <= 16 || steps_per_split % 4 != 0 || CL_HEAD_DIM > 192) asm volatile("" : "+s"(trips));
 #endif
   for (int step = 0;;) {
     do_step(PlC<0>{}, step);
