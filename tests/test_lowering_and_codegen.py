@@ -431,3 +431,20 @@ def test_a_split_of_a_family_without_a_contraction_is_refused_with_its_reason():
         split_stages(graph, 4)
     with pytest.raises(LoweringRejected, match="no split form"):
         source_for(C.rowsum_div.trace(cl.f16, M=64, N=256), split=4)
+
+
+def test_shipped_registry_kernels_keep_their_values_in_registers():
+    """The nine registry operators' shipped kernels as the run-time compiler builds them: nothing
+    spilled, no scratch memory, and the streaming decode forms within the 256 registers that let two
+    waves share a SIMD (needs the compiler, no GPU)."""
+    from cleave_amd.dynamic import OPERATORS
+    from cleave_amd.runtime import shim
+    from cleave_amd.runtime.compile import _compile, _load_main_kernel_from_code
+    shim.load()
+    assert len(OPERATORS) == 9
+    for name, op in OPERATORS.items():
+        loaded = _load_main_kernel_from_code(op.kernel_source())
+        for entry in _compile(loaded, loaded.manifest["out_idx"]).stats:
+            assert entry["spilled_vgprs"] == 0 and entry["scratch_bytes"] == 0, (name, entry)
+            if name.startswith("gqa_paged_decode"):
+                assert entry["vgprs"] <= 256, (name, entry)
